@@ -1,0 +1,177 @@
+/* ti8.h -- C ABI of libti8.so: gfx950 (MI355X) kernels for the INT8 quantized linear
+ * layer of jiaoch/Triton-INT8 (quantize -> int8 GEMM on i8 MFMA -> dequant, fwd + bwd).
+ *
+ * Conventions
+ *   - Every pointer is a BORROWED DEVICE pointer (hipMalloc'd / torch CUDA storage);
+ *     the library allocates nothing and keeps nothing after a call returns.
+ *   - Work is enqueued on `stream` (a hipStream_t passed as void*; NULL = null
+ *     stream) of the CURRENT device; calls return after enqueueing.
+ *   - Strides and leading dimensions are in ELEMENTS of the tensor they describe.
+ *   - Every function returns TI8_OK (0) or an error code and never throws; the
+ *     message of the last failure on the calling thread is ti8_last_error().
+ *     Arguments are validated on the host before anything is launched.
+ *   - bf16 tensors are passed as void* / uint16_t bit patterns.
+ *
+ * The reference has no FFI: its boundary is a set of Python functions, each a host
+ * wrapper around one Triton kernel.  Each entry point below names the reference
+ * wrapper + kernel it replaces (paths relative to the reference checkout).
+ */
+#ifndef TI8_H
+#define TI8_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* ti8_stream_t;
+
+enum ti8_status {
+    TI8_OK = 0,
+    TI8_ERR_NULL = 1,        /* a required pointer is NULL */
+    TI8_ERR_SHAPE = 2,       /* a size is not positive or not a multiple of what the kernel needs */
+    TI8_ERR_ALIGN = 3,       /* a pointer / leading dimension breaks the 16-byte access contract */
+    TI8_ERR_MODE = 4,        /* unknown or unsupported flag / mode combination */
+    TI8_ERR_HIP = 5          /* the HIP runtime reported an error at launch */
+};
+
+/* quantiser flags (bit set) */
+enum ti8_qflags {
+    TI8_Q_CLAMP = 1,        /* clamp floor(x*scale+0.5) to [-128,127] before the int8 cast */
+    TI8_Q_EPS_ADD = 2,      /* amax + 1e-5 (fused kernels) instead of max(amax, 1e-4) */
+    TI8_Q_SCALE_BF16 = 4    /* round the stored scale through bf16 (TileLang copy) */
+};
+
+/* which number is written to the scale tensor */
+enum ti8_inv_mode {
+    TI8_INV_RCP_OF_SCALE = 0,     /* 1.0f / (127.0f / amax)   block + per-token kernels */
+    TI8_INV_AMAX_DIV_127 = 1,     /* amax / 127.0f            two-pass per-row quantiser */
+    TI8_INV_AMAX_MUL_RCP127 = 2,  /* amax * (1.0f / 127.0f)   torch-GPU evaluation of the same */
+    TI8_INV_MULTIPLIER = 3        /* 127.0f / amax            fused kernels keep the multiplier */
+};
+
+/* scale descriptor of a GEMM operand (rows = M for A, N for B; kb = K block of 128) */
+enum ti8_scale_mode {
+    TI8_SCALE_ROW = 0,       /* s[batch*bs + row*rs]                          */
+    TI8_SCALE_BLOCK128 = 1,  /* s[batch*bs + (row/128)*rs + kb*ks]            */
+    TI8_SCALE_ROW_K128 = 2,  /* s[batch*bs + row*rs + kb*ks]                  */
+    TI8_SCALE_BLOCK_K256 = 3 /* s[batch*bs + (row/128)*rs + (kb/2)*ks]        */
+};
+
+/* how one K block's exact integer dot d enters the fp32 accumulator */
+enum ti8_combine {
+    TI8_COMBINE_MUL_MUL = 0,   /* acc += (f32(d) * sa) * sb      Triton block-channel kernels */
+    TI8_COMBINE_MUL_PROD = 1,  /* acc += f32(d) * (sa * sb)      TileLang kernels            */
+    TI8_COMBINE_DIV_PROD = 2   /* acc += f32(d) / (sa * sb)      fused kernels (s = multipliers) */
+};
+
+enum ti8_gemm_flags {
+    TI8_GEMM_STRICT = 1   /* evaluate the combine formula literally (separate roundings, true
+                             division); without it the kernel may use fma / reciprocal, which
+                             moves results by a few fp32 ulps before the bf16 rounding */
+};
+
+/* Library version (major*10000 + minor*100 + patch). */
+int ti8_version(void);
+/* Message of the last error on this thread ("" if none). */
+const char* ti8_last_error(void);
+/* Name of the GPU architecture the kernels were compiled for ("gfx950"). */
+const char* ti8_arch(void);
+
+/* ---------------------------------------------------------------------------------
+ * Per-block absmax quantiser: replaces triton_per_block_quant + per_block_quant_kernel
+ * (triton/block_channel_fwd32.py:160-212 clamped; triton/block_channel_bwd33.py:87-138
+ * unclamped; tilelang/block_channel_fwd.py:152-203 with group_c = 256 and bf16 scales).
+ *
+ *   x   bf16 [B][R][C], rows contiguous, leading dim ldx, batch stride bsx
+ *   q   int8 [B][R][C] (ldq, bsq)   same orientation as x            -- may be NULL
+ *   qT  int8 [B][C][R] (ldqt, bsqt) the transposed copy of q          -- may be NULL
+ *   s   fp32, scale of tile (b, rb, cb) at s[b*ssb + rb*ssr + cb*ssc]
+ * Tiles are 128 x group_c (group_c = 128 or 256; qT needs 128).  A 128x128 block
+ * quantisation commutes with transposition, so a transposed VIEW is quantised by
+ * passing its underlying row-major memory and swapping (q, qT) and (ssr, ssc).
+ * At least one of q / qT must be given.  R % 128 == 0, C % group_c == 0. */
+int ti8_quant_block(const void* x, int64_t bsx, int64_t ldx,
+                    int8_t* q, int64_t bsq, int64_t ldq,
+                    int8_t* qT, int64_t bsqt, int64_t ldqt,
+                    float* s, int64_t ssb, int64_t ssr, int64_t ssc,
+                    int64_t B, int64_t R, int64_t C, int group_c,
+                    int qflags, int inv_mode, ti8_stream_t stream);
+
+/* ---------------------------------------------------------------------------------
+ * Per-row absmax quantiser in ONE pass over x: replaces triton_per_token_quant +
+ * per_token_quant_kernel (triton/block_channel_fwd32.py:101-157) and the two-pass
+ * triton_per_row_quant_2d/3d + _pass1/_pass2 kernels with their torch glue
+ * (triton/double-channle_fwd32.py:93-266, triton/double_channel_bwd33.py:90-176).
+ *
+ *   x bf16 [rows][cols] (ldx) -> q int8 [rows][cols] (ldq)
+ *   group = 0:   one scale per row,                 s[rows]
+ *   group = 128: one scale per (row, 128 columns),  s[rows][cols/128]   (B operand of
+ *                the fused kernel, triton/fused_triton_fwd32.py:57-59)
+ * cols % 128 == 0, cols <= 32768. */
+int ti8_quant_row(const void* x, int64_t ldx, int8_t* q, int64_t ldq, float* s,
+                  int64_t rows, int64_t cols, int group,
+                  int qflags, int inv_mode, ti8_stream_t stream);
+
+/* ---------------------------------------------------------------------------------
+ * Per-COLUMN absmax quantiser with transposed output = the per-row quantiser applied
+ * to x^T without materialising x^T in bf16.  Serves the reference's calls on
+ * transposed operands (fwd_32(dY, W^T): triton/block_channel_fwd32.py:221-222 with
+ * b = W^T; bwd_33(dY^T, X^T) of the double-channel scheme).
+ *
+ *   x bf16 [R][C] (ldx) -> qT int8 [C][R] (ldqt), s[C]
+ *   ws: workspace of C floats (column absmax), contents undefined afterwards.
+ * R % 128 == 0, C % 128 == 0. */
+int ti8_quant_col_t(const void* x, int64_t ldx, int8_t* qT, int64_t ldqt, float* s, float* ws,
+                    int64_t R, int64_t C, int qflags, int inv_mode, ti8_stream_t stream);
+
+/* ---------------------------------------------------------------------------------
+ * Un-normalised Walsh-Hadamard transform along the last dim (Sylvester order):
+ * replaces fast_hadamard_transform.hadamard_transform at its call sites
+ * (triton/double-channle_fwd32.py:273-274,299-300; triton/double_channel_bwd33.py:
+ * 189-190,208-209).  bf16 in, fp32 butterflies (strides 1,2,4,...), times `scale`,
+ * one rounding to bf16 out.  Transforms contiguous groups of n along each row:
+ * n = cols is the reference's full-length rotation, n = 128 the block-diagonal one.
+ * n a power of two, 128 <= n <= 32768, cols % n == 0.  x == y is allowed. */
+int ti8_fwht(const void* x, int64_t ldx, void* y, int64_t ldy,
+             int64_t rows, int64_t cols, int64_t n, float scale, ti8_stream_t stream);
+
+/* ---------------------------------------------------------------------------------
+ * INT8 NT GEMM with fused dequantising epilogue, C[b] = dequant(A[b] * B[b]^T):
+ * replaces triton_gemm + int8_gemm_kernel of every scheme
+ *   block-channel 3Dx2D  triton/block_channel_fwd32.py:12-96   (A BLOCK128, B ROW)
+ *   block-channel 3Dx3D  triton/block_channel_bwd33.py:8-84    (A BLOCK128, B BLOCK128)
+ *   double-channel       triton/double-channle_fwd32.py:11-90, double_channel_bwd33.py:11-87
+ *   TileLang mains       tilelang/block_channel_fwd.py:46-86, block_channel_bwd.py:47-86
+ * and the GEMM half of the fused kernels (triton/fused_triton_fwd32.py:42-65).
+ *
+ *   A int8 [batch][M][K] (lda, bsa), B int8 [batch][N][K] (ldb, bsb; bsb = 0 shares
+ *   one B), C bf16 [batch][M][N] (ldc, bsc).  Both operands contiguous along K.
+ *   acc_i32_full = 1: int32 accumulation over the whole K, both scales TI8_SCALE_ROW,
+ *       C = bf16((f32(acc) * sA[m]) * sB[n]); if post_scale != 0 a second rounding
+ *       C = bf16(f32(C) * post_scale) follows (the reference's `C * inv_K`).
+ *   acc_i32_full = 0: per 128-deep K block, exact int32 dot d, then `combine`;
+ *       C = bf16(acc * out_scale) (out_scale = 1 for none).
+ * M, N, K multiples of 128. */
+int ti8_gemm_i8_nt(const int8_t* A, int64_t bsa, int64_t lda,
+                   const int8_t* B, int64_t bsb, int64_t ldb,
+                   void* C, int64_t bsc, int64_t ldc,
+                   const float* sA, int modeA, int64_t sa_bs, int64_t sa_rs, int64_t sa_ks,
+                   const float* sB, int modeB, int64_t sb_bs, int64_t sb_rs, int64_t sb_ks,
+                   int64_t batch, int64_t M, int64_t N, int64_t K,
+                   int acc_i32_full, int combine, float out_scale, float post_scale,
+                   int gemm_flags, ti8_stream_t stream);
+
+/* Raw int32 accumulators of the same GEMM over the whole K, C int32 [batch][M][N]:
+ * the accumulator of int8_gemm_kernel in triton/double-channle_fwd32.py:44,56.
+ * Exists so that tests can compare accumulators bit for bit. */
+int ti8_gemm_i8_nt_i32(const int8_t* A, int64_t bsa, int64_t lda,
+                       const int8_t* B, int64_t bsb, int64_t ldb,
+                       int32_t* C, int64_t bsc, int64_t ldc,
+                       int64_t batch, int64_t M, int64_t N, int64_t K, ti8_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TI8_H */

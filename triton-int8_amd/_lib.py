@@ -1,0 +1,71 @@
+"""ctypes binding of ``libti8.so`` (the C ABI declared in ``include/ti8.h``).
+
+The library is the product: there is no fallback.  If it has not been built
+(``python triton-int8_amd/build.py``) importing any operator raises.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libti8.so")
+
+_i64, _int, _f32, _vp = ctypes.c_int64, ctypes.c_int, ctypes.c_float, ctypes.c_void_p
+
+# name -> argument types, in the order of include/ti8.h
+PROTOTYPES = {
+    "ti8_quant_block": [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _i64,
+                        _i64, _i64, _i64, _int, _int, _int, _vp],
+    "ti8_quant_row": [_vp, _i64, _vp, _i64, _vp, _i64, _i64, _int, _int, _int, _vp],
+    "ti8_quant_col_t": [_vp, _i64, _vp, _i64, _vp, _vp, _i64, _i64, _int, _int, _vp],
+    "ti8_fwht": [_vp, _i64, _vp, _i64, _i64, _i64, _i64, _f32, _vp],
+    "ti8_gemm_i8_nt": [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64,
+                       _vp, _int, _i64, _i64, _i64, _vp, _int, _i64, _i64, _i64,
+                       _i64, _i64, _i64, _i64, _int, _int, _f32, _f32, _int, _vp],
+    "ti8_gemm_i8_nt_i32": [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp],
+}
+EXPORTS = ["ti8_version", "ti8_last_error", "ti8_arch"] + list(PROTOTYPES)
+
+# enums of include/ti8.h
+Q_CLAMP, Q_EPS_ADD, Q_SCALE_BF16 = 1, 2, 4
+INV_RCP_OF_SCALE, INV_AMAX_DIV_127, INV_AMAX_MUL_RCP127, INV_MULTIPLIER = 0, 1, 2, 3
+SCALE_ROW, SCALE_BLOCK128, SCALE_ROW_K128, SCALE_BLOCK_K256 = 0, 1, 2, 3
+COMBINE_MUL_MUL, COMBINE_MUL_PROD, COMBINE_DIV_PROD = 0, 1, 2
+GEMM_STRICT = 1
+
+_lib = None
+
+
+class Ti8Error(RuntimeError):
+    """A libti8 entry point returned a non-zero status."""
+
+    def __init__(self, fn, code, msg):
+        super().__init__(f"{fn} failed with status {code}: {msg}")
+        self.code = code
+
+
+def lib():
+    """The loaded library (loaded once).  Raises if it was never built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is missing: build it with `python triton-int8_amd/build.py` "
+                "(hipcc, gfx950).  There is no fallback implementation.")
+        l = ctypes.CDLL(LIB_PATH)
+        l.ti8_version.restype = _int
+        l.ti8_last_error.restype = ctypes.c_char_p
+        l.ti8_arch.restype = ctypes.c_char_p
+        for name, args in PROTOTYPES.items():
+            fn = getattr(l, name)
+            fn.argtypes = args
+            fn.restype = _int
+        _lib = l
+    return _lib
+
+
+def call(name, *args):
+    """Call an entry point; raise :class:`Ti8Error` with the library's message on failure."""
+    l = lib()
+    rc = getattr(l, name)(*args)
+    if rc != 0:
+        raise Ti8Error(name, rc, l.ti8_last_error().decode())

@@ -1,0 +1,394 @@
+// INT8 NT GEMM on CDNA4 i8 MFMA (v_mfma_i32_32x32x32_i8) with fused dequantisation.
+//
+// C[b][m][n] = dequant( sum_k A[b][m][k] * B[b][n][k] ), both operands K-contiguous.
+//
+// Data flow per workgroup (BM x BN output tile, K walked in tiles of 128 bytes):
+//   HBM --global_load_lds_dwordx4--> LDS (double buffered, 16-byte chunks XOR-swizzled
+//   by row so that the 32 rows a wave reads at one k offset fall in distinct banks)
+//   --ds_read_b128--> MFMA operand registers --> int32 accumulators.
+// A K tile is exactly one 128-deep quantisation block, so the block-channel variants
+// convert and scale the int32 partial into an fp32 accumulator once per K tile.
+//
+// MFMA operand/result layout used (32x32x32 i8): lane l supplies row (l % 32) of its
+// operand and the 16 bytes k = 16*(l / 32) .. +15 of the 32-deep slice (the same map
+// for both operands, which is all an NT dot product needs); result register r of lane
+// l is C[8*(r/4) + 4*(l/32) + r%4][l % 32] with rows from A and columns from B.
+#include "ti8_common.h"
+
+namespace ti8 {
+
+struct ScaleDesc {
+    const float* p;
+    int mode;         // ti8_scale_mode
+    int64_t bs, rs, ks;
+};
+
+struct GemmArgs {
+    const int8_t* A;
+    const int8_t* B;
+    void* C;
+    int64_t bsa, lda, bsb, ldb, bsc, ldc;
+    ScaleDesc sa, sb;
+    int M, N, K;
+    int tiles_m, tiles_n;
+    int combine;
+    int strict;
+    float out_scale, post_scale;
+};
+
+enum { EPI_I32 = 0, EPI_ROWS = 1, EPI_PROMOTE = 2, EPI_STRICT = 3 };
+
+
+// scale of operand row `row` at K block kb
+__device__ __forceinline__ float scale_at(const ScaleDesc& d, int64_t batch, int row, int kb) {
+    switch (d.mode) {
+        case TI8_SCALE_ROW: return d.p[batch * d.bs + (int64_t)row * d.rs];
+        case TI8_SCALE_BLOCK128: return d.p[batch * d.bs + (int64_t)(row >> 7) * d.rs + (int64_t)kb * d.ks];
+        case TI8_SCALE_ROW_K128: return d.p[batch * d.bs + (int64_t)row * d.rs + (int64_t)kb * d.ks];
+        default: return d.p[batch * d.bs + (int64_t)(row >> 7) * d.rs + (int64_t)(kb >> 1) * d.ks];
+    }
+}
+
+// One wave's share of a K tile: NI global->LDS instructions of 64 x 16 bytes; instruction i
+// fills the 1 KiB slab at lds + i*1024 (lane l lands at byte 16*l of the slab).
+template <int NI>
+__device__ __forceinline__ void issue_tile_loads(const int8_t* const (&gp)[NI], int koff, int8_t* lds) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the builtin only exists in the device pass
+#pragma unroll
+    for (int i = 0; i < NI; ++i) __builtin_amdgcn_global_load_lds(gp[i] + koff, lds + i * 1024, 16, 0, 0);
+#else
+    (void)gp; (void)koff; (void)lds;
+#endif
+}
+
+template <int BM, int BN, int WM, int WN, int EPI>
+__global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g) {
+    constexpr int NW = WM * WN;
+    constexpr int TM = BM / WM / 32;  // 32x32 blocks per wave along M
+    constexpr int TN = BN / WN / 32;
+    constexpr int A_INSTR = BM / 8 / NW;  // global->LDS wave instructions per K tile per wave
+    constexpr int B_INSTR = BN / 8 / NW;
+    constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128;
+    constexpr bool PROMOTE = (EPI == EPI_PROMOTE || EPI == EPI_STRICT);
+    static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "tile/wave mismatch");
+
+    extern __shared__ __attribute__((aligned(1024))) int8_t smem[];
+    // layout: [A buf0][A buf1][B buf0][B buf1]
+    int8_t* const ldsA = smem;
+    int8_t* const ldsB = smem + 2 * A_BYTES;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+
+    // ---- tile assignment: XCD-aware remap, then groups of 8 tile rows -----------------
+    const int ntiles = g.tiles_m * g.tiles_n;
+    int pid = blockIdx.x;
+    if ((ntiles & 7) == 0) pid = (pid & 7) * (ntiles >> 3) + (pid >> 3);  // one contiguous range per XCD
+    constexpr int GROUP = 8;
+    const int per_group = GROUP * g.tiles_n;
+    const int group_id = pid / per_group;
+    const int first_m = group_id * GROUP;
+    const int gsz = min(g.tiles_m - first_m, GROUP);
+    const int tile_m = first_m + (pid % per_group) % gsz;
+    const int tile_n = (pid % per_group) / gsz;
+    const int batch = blockIdx.y;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    const int8_t* Ab = g.A + (int64_t)batch * g.bsa;
+    const int8_t* Bb = g.B + (int64_t)batch * g.bsb;
+
+    // ---- global -> LDS mapping --------------------------------------------------------
+    // wave instruction t covers tile rows 8t..8t+7; lane l writes LDS chunk l of that 1 KiB
+    // slab = (row 8t + l/8, physical chunk l%8), which holds logical chunk (l%8) ^ (l/8).
+    const int ld_row = lane >> 3;
+    const int ld_chunk = (lane & 7) ^ ld_row;
+    const int8_t* gA[A_INSTR];
+    const int8_t* gB[B_INSTR];
+#pragma unroll
+    for (int i = 0; i < A_INSTR; ++i) {
+        const int r = min(m0 + (wave * A_INSTR + i) * 8 + ld_row, g.M - 1);
+        gA[i] = Ab + (int64_t)r * g.lda + ld_chunk * 16;
+    }
+#pragma unroll
+    for (int i = 0; i < B_INSTR; ++i) {
+        const int r = min(n0 + (wave * B_INSTR + i) * 8 + ld_row, g.N - 1);
+        gB[i] = Bb + (int64_t)r * g.ldb + ld_chunk * 16;
+    }
+
+    // ---- LDS -> register mapping ------------------------------------------------------
+    const int fr_row = lane & 31;
+    const int fr_half = lane >> 5;
+    const int sw = lane & 7;  // row & 7 (every block starts on a multiple of 8 rows)
+    const int a_row_off = (wm * TM * 32 + fr_row) * 128;
+    const int b_row_off = (wn * TN * 32 + fr_row) * 128;
+
+    v16i acc[TM][TN];
+    float accf[PROMOTE ? TM : 1][PROMOTE ? TN : 1][16];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+            if (PROMOTE) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) accf[i][j][r] = 0.0f;
+            }
+        }
+
+    const int nk = g.K >> 7;
+    issue_tile_loads<A_INSTR>(gA, 0, ldsA + wave * A_INSTR * 1024);
+    issue_tile_loads<B_INSTR>(gB, 0, ldsB + wave * B_INSTR * 1024);
+    __builtin_amdgcn_s_waitcnt(0x0f70 & 0);  // vmcnt(0) (all counters to zero)
+    __syncthreads();
+
+    for (int kt = 0; kt < nk; ++kt) {
+        const int buf = kt & 1;
+        if (kt + 1 < nk) {
+            issue_tile_loads<A_INSTR>(gA, (kt + 1) * 128, ldsA + (buf ^ 1) * A_BYTES + wave * A_INSTR * 1024);
+            issue_tile_loads<B_INSTR>(gB, (kt + 1) * 128, ldsB + (buf ^ 1) * B_BYTES + wave * B_INSTR * 1024);
+        }
+
+        const int8_t* sA = ldsA + buf * A_BYTES + a_row_off;
+        const int8_t* sB = ldsB + buf * B_BYTES + b_row_off;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const int choff = ((ks * 2 + fr_half) ^ sw) * 16;
+            v4i a[TM], b[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) a[i] = *reinterpret_cast<const v4i*>(sA + i * 32 * 128 + choff);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) b[j] = *reinterpret_cast<const v4i*>(sB + j * 32 * 128 + choff);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+
+        if (EPI == EPI_PROMOTE) {
+            // in-loop factor: scalar per 128-row block of A (unless A is per-row) times the
+            // per-column value of B (unless B is per-row); per-row parts wait for the epilogue
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const int mrow = min(m0 + (wm * TM + i) * 32, g.M - 1);
+                const float fa = (g.sa.mode == TI8_SCALE_ROW) ? 1.0f : scale_at(g.sa, batch, mrow, kt);
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    const int ncol = min(n0 + (wn * TN + j) * 32 + fr_row, g.N - 1);
+                    const float fb = (g.sb.mode == TI8_SCALE_ROW) ? 1.0f : scale_at(g.sb, batch, ncol, kt);
+                    float f = fa * fb;
+                    if (g.combine == TI8_COMBINE_DIV_PROD) f = 1.0f / f;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        accf[i][j][r] = __builtin_fmaf(static_cast<float>(acc[i][j][r]), f, accf[i][j][r]);
+                        acc[i][j][r] = 0;
+                    }
+                }
+            }
+        } else if (EPI == EPI_STRICT) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    const int ncol = min(n0 + (wn * TN + j) * 32 + fr_row, g.N - 1);
+                    const float sb = scale_at(g.sb, batch, ncol, kt);
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int mrow = min(m0 + (wm * TM + i) * 32 + 8 * (r >> 2) + 4 * fr_half + (r & 3), g.M - 1);
+                        const float sa = scale_at(g.sa, batch, mrow, kt);
+                        const float d = static_cast<float>(acc[i][j][r]);
+                        float t;
+                        if (g.combine == TI8_COMBINE_MUL_MUL) {
+                            t = d * sa;
+                            t = t * sb;
+                        } else if (g.combine == TI8_COMBINE_MUL_PROD) {
+                            t = d * (sa * sb);
+                        } else {
+                            t = d / (sa * sb);
+                        }
+                        accf[i][j][r] = accf[i][j][r] + t;  // separate rounding: contraction is off
+                        acc[i][j][r] = 0;
+                    }
+                }
+        }
+
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+    }
+
+    // ---- epilogue ---------------------------------------------------------------------
+    // Each wave moves its accumulators through a private 16 KiB LDS slab, 32 tile rows at
+    // a time, so that the global stores are whole row segments (4 columns per lane, two
+    // rows of WN-th of the tile per wave instruction) instead of one column per lane.
+    // The main loop ended with a workgroup barrier, so the operand buffers are free.
+    constexpr int WCOLS = TN * 32;                       // columns of the wave tile
+    constexpr int LPR = WCOLS / 4;                       // lanes per row in the read-back
+    constexpr int RPI = 64 / LPR;                        // rows per wave instruction
+    static_assert(WCOLS * 32 * 4 * NW <= 2 * (A_BYTES + B_BYTES), "epilogue slab does not fit");
+    uint32_t* slab = reinterpret_cast<uint32_t*>(smem) + wave * (32 * WCOLS);
+    const int rb_col = (lane % LPR) * 4;
+    const int rb_row = lane / LPR;
+    const int ncol0 = n0 + wn * WCOLS + rb_col;          // first of this lane's 4 columns
+    float coln[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+    if (EPI == EPI_ROWS || (EPI == EPI_PROMOTE && g.sb.mode == TI8_SCALE_ROW)) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            coln[c] = scale_at(g.sb, batch, min(ncol0 + c, g.N - 1), 0);
+            if (EPI == EPI_PROMOTE && g.combine == TI8_COMBINE_DIV_PROD) coln[c] = 1.0f / coln[c];
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int rr = 8 * (r >> 2) + 4 * fr_half + (r & 3);
+                const uint32_t bits = PROMOTE ? __float_as_uint(accf[PROMOTE ? i : 0][PROMOTE ? j : 0][r])
+                                              : static_cast<uint32_t>(acc[i][j][r]);
+                slab[rr * WCOLS + j * 32 + fr_row] = bits;
+            }
+        // same wave reads what it wrote: an LDS counter wait is enough, no barrier
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+        __builtin_amdgcn_wave_barrier();
+        const int mbase = m0 + (wm * TM + i) * 32;
+        for (int rr = rb_row; rr < 32; rr += RPI) {
+            const int m = mbase + rr;
+            const uint4 w = *reinterpret_cast<const uint4*>(slab + rr * WCOLS + rb_col);
+            if (m >= g.M || ncol0 >= g.N) continue;  // N is a multiple of 4: a lane's 4 columns are all in or all out
+            const int64_t off = (int64_t)batch * g.bsc + (int64_t)m * g.ldc + ncol0;
+            if (EPI == EPI_I32) {
+                *reinterpret_cast<uint4*>(reinterpret_cast<int32_t*>(g.C) + off) = w;
+                continue;
+            }
+            float t[4];
+            const uint32_t wb[4] = {w.x, w.y, w.z, w.w};
+            if (EPI == EPI_ROWS) {
+                const float rowm = scale_at(g.sa, batch, m, 0);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    float v = static_cast<float>(static_cast<int32_t>(wb[c])) * rowm;
+                    v = v * coln[c];
+                    if (g.post_scale != 0.0f) v = __uint_as_float(f32_to_bf16_bits(v) << 16) * g.post_scale;
+                    t[c] = v;
+                }
+            } else {
+                float rowm = 1.0f;
+                const bool row_part = (EPI == EPI_PROMOTE && g.sa.mode == TI8_SCALE_ROW);
+                if (row_part) {
+                    rowm = scale_at(g.sa, batch, m, 0);
+                    if (g.combine == TI8_COMBINE_DIV_PROD) rowm = 1.0f / rowm;
+                }
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    float v = __uint_as_float(wb[c]);
+                    if (row_part) v = v * rowm;
+                    if (EPI == EPI_PROMOTE && g.sb.mode == TI8_SCALE_ROW) v = v * coln[c];
+                    if (g.out_scale != 1.0f) v = v * g.out_scale;
+                    t[c] = v;
+                }
+            }
+            uint2 o;
+            o.x = f32_to_bf16_bits(t[0]) | (f32_to_bf16_bits(t[1]) << 16);
+            o.y = f32_to_bf16_bits(t[2]) | (f32_to_bf16_bits(t[3]) << 16);
+            *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(g.C) + off) = o;
+        }
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
+template <int BM, int BN, int WM, int WN, int EPI>
+static int launch(const GemmArgs& a0, int64_t batch, hipStream_t st) {
+    GemmArgs a = a0;
+    a.tiles_m = (a.M + BM - 1) / BM;
+    a.tiles_n = (a.N + BN - 1) / BN;
+    const size_t shmem = 2 * (size_t)(BM + BN) * 128;
+    static thread_local int attr_dev = -1;
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    auto kern = gemm_i8_kernel<BM, BN, WM, WN, EPI>;
+    if (shmem > 64 * 1024 && attr_dev != dev) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+        if (e != hipSuccess) return fail(TI8_ERR_HIP, "gemm: cannot raise the LDS limit to %zu: %s", shmem, hipGetErrorString(e));
+        attr_dev = dev;
+    }
+    dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)batch), block(64 * WM * WN);
+    hipLaunchKernelGGL(kern, grid, block, shmem, st, a);
+    return check_launch("ti8_gemm_i8_nt");
+}
+
+static int check_operands(const char* fn, const void* A, int64_t bsa, int64_t lda, const void* B, int64_t bsb, int64_t ldb,
+                          const void* C, int64_t ldc, int64_t batch, int64_t M, int64_t N, int64_t K) {
+    if (!A || !B || !C) return fail(TI8_ERR_NULL, "%s: A, B and C are required", fn);
+    if (batch <= 0 || M <= 0 || N <= 0 || K <= 0 || K % 128 || M % 128 || N % 128)
+        return fail(TI8_ERR_SHAPE, "%s: need batch>0 and M, N, K positive multiples of 128; got batch=%lld M=%lld N=%lld K=%lld",
+                    fn, (long long)batch, (long long)M, (long long)N, (long long)K);
+    if (M > 0x3fffffff || N > 0x3fffffff || K > 0x3fffffff || batch > 65535)
+        return fail(TI8_ERR_SHAPE, "%s: dimension too large", fn);
+    if (lda < K || ldb < K || ldc < N) return fail(TI8_ERR_SHAPE, "%s: leading dimension smaller than the row length", fn);
+    if (!aligned16(A) || !aligned16(B) || (lda % 16) || (ldb % 16) || (bsa % 16) || (bsb % 16))
+        return fail(TI8_ERR_ALIGN, "%s: A and B must be 16-byte aligned with strides multiples of 16", fn);
+    return TI8_OK;
+}
+
+static int check_scale(const char* fn, const char* which, const float* p, int mode) {
+    if (!p) return fail(TI8_ERR_NULL, "%s: scale pointer of %s is NULL", fn, which);
+    if (mode < 0 || mode > 3) return fail(TI8_ERR_MODE, "%s: unknown scale mode %d for %s", fn, mode, which);
+    return TI8_OK;
+}
+
+}  // namespace ti8
+
+using namespace ti8;
+
+extern "C" int ti8_gemm_i8_nt(const int8_t* A, int64_t bsa, int64_t lda, const int8_t* B, int64_t bsb, int64_t ldb,
+                              void* C, int64_t bsc, int64_t ldc, const float* sA, int modeA, int64_t sa_bs,
+                              int64_t sa_rs, int64_t sa_ks, const float* sB, int modeB, int64_t sb_bs, int64_t sb_rs,
+                              int64_t sb_ks, int64_t batch, int64_t M, int64_t N, int64_t K, int acc_i32_full,
+                              int combine, float out_scale, float post_scale, int gemm_flags, ti8_stream_t stream) {
+    const char* fn = "ti8_gemm_i8_nt";
+    if (int e = check_operands(fn, A, bsa, lda, B, bsb, ldb, C, ldc, batch, M, N, K)) return e;
+    if (int e = check_scale(fn, "A", sA, modeA)) return e;
+    if (int e = check_scale(fn, "B", sB, modeB)) return e;
+    if (combine < 0 || combine > 2) return fail(TI8_ERR_MODE, "%s: unknown combine %d", fn, combine);
+    if (gemm_flags & ~TI8_GEMM_STRICT) return fail(TI8_ERR_MODE, "%s: unknown flag 0x%x", fn, gemm_flags);
+    if (acc_i32_full && (modeA != TI8_SCALE_ROW || modeB != TI8_SCALE_ROW))
+        return fail(TI8_ERR_MODE, "%s: int32 accumulation over the whole K needs per-row scales on both operands", fn);
+    if ((modeA == TI8_SCALE_BLOCK_K256 || modeB == TI8_SCALE_BLOCK_K256) && (K % 256))
+        return fail(TI8_ERR_SHAPE, "%s: 256-wide scale groups need K %% 256 == 0", fn);
+    if ((reinterpret_cast<uintptr_t>(C) & 7) || (ldc % 4) || (bsc % 4)) return fail(TI8_ERR_ALIGN, "%s: C must be 8-byte aligned with strides multiples of 4", fn);
+    GemmArgs a;
+    a.A = A; a.B = B; a.C = C;
+    a.bsa = bsa; a.lda = lda; a.bsb = bsb; a.ldb = ldb; a.bsc = bsc; a.ldc = ldc;
+    a.sa = ScaleDesc{sA, modeA, sa_bs, sa_rs, sa_ks};
+    a.sb = ScaleDesc{sB, modeB, sb_bs, sb_rs, sb_ks};
+    a.M = (int)M; a.N = (int)N; a.K = (int)K;
+    a.tiles_m = a.tiles_n = 0;
+    a.combine = combine;
+    a.strict = (gemm_flags & TI8_GEMM_STRICT) ? 1 : 0;
+    a.out_scale = out_scale; a.post_scale = post_scale;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (acc_i32_full) return launch<256, 256, 2, 2, EPI_ROWS>(a, batch, st);
+    const bool a_loop_per_row = (modeA == TI8_SCALE_ROW_K128);  // would need a per-register factor
+    if (a.strict || a_loop_per_row) return launch<128, 128, 2, 2, EPI_STRICT>(a, batch, st);
+    return launch<256, 128, 2, 2, EPI_PROMOTE>(a, batch, st);
+}
+
+extern "C" int ti8_gemm_i8_nt_i32(const int8_t* A, int64_t bsa, int64_t lda, const int8_t* B, int64_t bsb, int64_t ldb,
+                                  int32_t* C, int64_t bsc, int64_t ldc, int64_t batch, int64_t M, int64_t N, int64_t K,
+                                  ti8_stream_t stream) {
+    const char* fn = "ti8_gemm_i8_nt_i32";
+    if (int e = check_operands(fn, A, bsa, lda, B, bsb, ldb, C, ldc, batch, M, N, K)) return e;
+    GemmArgs a;
+    a.A = A; a.B = B; a.C = C;
+    a.bsa = bsa; a.lda = lda; a.bsb = bsb; a.ldb = ldb; a.bsc = bsc; a.ldc = ldc;
+    a.sa = ScaleDesc{nullptr, 0, 0, 0, 0};
+    a.sb = a.sa;
+    a.M = (int)M; a.N = (int)N; a.K = (int)K;
+    a.tiles_m = a.tiles_n = 0;
+    a.combine = 0; a.strict = 0; a.out_scale = 1.0f; a.post_scale = 0.0f;
+    return launch<256, 256, 2, 2, EPI_I32>(a, batch, static_cast<hipStream_t>(stream));
+}

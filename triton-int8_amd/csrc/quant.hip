@@ -1,0 +1,437 @@
+// Absmax -> int8 quantisers for gfx950.  All are HBM-bound: each reads every bf16
+// element once with 16-byte loads, keeps it in registers while the group's absmax is
+// reduced (wave shuffles + a few LDS words), and writes packed int8.
+//
+// This file MUST be compiled with -ffp-contract=off: `x*scale + 0.5f` has to round
+// twice (multiply, then add) to reproduce the reference arithmetic bit for bit.
+#include "ti8_common.h"
+
+namespace ti8 {
+
+struct QMode {
+    int clamp;       // TI8_Q_CLAMP
+    int eps_add;     // TI8_Q_EPS_ADD
+    int scale_bf16;  // TI8_Q_SCALE_BF16
+    int inv_mode;    // ti8_inv_mode
+};
+
+__device__ __forceinline__ float amax_floor(float amax, int eps_add) {
+    // triton/block_channel_fwd32.py:182 `where(amax > 1e-4, amax, 1e-4)`;
+    // triton/fused_triton_fwd32.py:49 `max|x| + 1e-5`
+    return eps_add ? (amax + 1e-5f) : (amax > 1e-4f ? amax : 1e-4f);
+}
+
+__device__ __forceinline__ float stored_scale(float amax, float scale, const QMode& m) {
+    float s;
+    switch (m.inv_mode) {
+        case TI8_INV_RCP_OF_SCALE: s = 1.0f / scale; break;
+        case TI8_INV_AMAX_DIV_127: s = amax / 127.0f; break;
+        case TI8_INV_AMAX_MUL_RCP127: s = amax * (1.0f / 127.0f); break;
+        default: s = scale; break;
+    }
+    if (m.scale_bf16) s = __uint_as_float(f32_to_bf16_bits(s) << 16);
+    return s;
+}
+
+__device__ __forceinline__ uint32_t q1(float x, float scale, int clamp) {
+    float r = floorf(x * scale + 0.5f);  // two roundings (contraction is off)
+    if (clamp) r = fminf(fmaxf(r, -128.0f), 127.0f);
+    return static_cast<uint32_t>(static_cast<int>(r)) & 0xffu;
+}
+
+// 8 bf16 (one 16-byte load) -> 8 int8 in two dwords, element 0 in the low byte
+__device__ __forceinline__ uint2 quant8(const uint4& v, float scale, int clamp) {
+    uint2 o;
+    o.x = q1(bf16_lo(v.x), scale, clamp) | (q1(bf16_hi(v.x), scale, clamp) << 8) |
+          (q1(bf16_lo(v.y), scale, clamp) << 16) | (q1(bf16_hi(v.y), scale, clamp) << 24);
+    o.y = q1(bf16_lo(v.z), scale, clamp) | (q1(bf16_hi(v.z), scale, clamp) << 8) |
+          (q1(bf16_lo(v.w), scale, clamp) << 16) | (q1(bf16_hi(v.w), scale, clamp) << 24);
+    return o;
+}
+
+__device__ __forceinline__ float absmax8(const uint4& v, float m) {
+    m = fmaxf(m, fabsf(bf16_lo(v.x)));
+    m = fmaxf(m, fabsf(bf16_hi(v.x)));
+    m = fmaxf(m, fabsf(bf16_lo(v.y)));
+    m = fmaxf(m, fabsf(bf16_hi(v.y)));
+    m = fmaxf(m, fabsf(bf16_lo(v.z)));
+    m = fmaxf(m, fabsf(bf16_hi(v.z)));
+    m = fmaxf(m, fabsf(bf16_lo(v.w)));
+    m = fmaxf(m, fabsf(bf16_hi(v.w)));
+    return m;
+}
+
+// max over the 256 threads of a workgroup (4 waves), result in every thread
+__device__ __forceinline__ float block_max_256(float v, float* red4) {
+    v = wave_max(v);
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) red4[wave] = v;
+    __syncthreads();
+    v = fmaxf(fmaxf(red4[0], red4[1]), fmaxf(red4[2], red4[3]));
+    return v;
+}
+
+// byte e (0..3) of four dwords -> one dword (row 0 in the low byte): a 4x4 byte transpose column
+__device__ __forceinline__ uint32_t gather_byte(uint32_t r0, uint32_t r1, uint32_t r2, uint32_t r3, int e) {
+    const int sh = e * 8;
+    return ((r0 >> sh) & 0xffu) | (((r1 >> sh) & 0xffu) << 8) | (((r2 >> sh) & 0xffu) << 16) |
+           (((r3 >> sh) & 0xffu) << 24);
+}
+
+// ---------------------------------------------------------------------------------
+// 128 x (128*NSUB) tile per workgroup of 256 threads.  Thread t owns, in every
+// 128x128 sub-tile, rows {64h + 4*(t/16) + j : h<2, j<4} x columns [8*(t%16), +8):
+// a wave load instruction covers whole 256-byte row segments, and the 4-row patches
+// transpose in registers for the optional transposed output (staged through LDS so
+// that the global writes of qT are 128-byte rows too).
+template <int NSUB, bool WRITE_Q, bool WRITE_QT>
+__global__ __launch_bounds__(256) void quant_block_kernel(
+    const uint16_t* __restrict__ x, int64_t bsx, int64_t ldx, int8_t* __restrict__ q, int64_t bsq, int64_t ldq,
+    int8_t* __restrict__ qT, int64_t bsqt, int64_t ldqt, float* __restrict__ s, int64_t ssb, int64_t ssr,
+    int64_t ssc, int nrb, int ncb, QMode mode) {
+    __shared__ float red4[4];
+    __shared__ uint32_t tileT[WRITE_QT ? 128 * 33 : 1];
+
+    int tile = blockIdx.x;
+    const int cb = tile % ncb;
+    tile /= ncb;
+    const int rb = tile % nrb;
+    const int b = tile / nrb;
+
+    const int tid = threadIdx.x;
+    const int cc = tid & 15;   // 8-column chunk
+    const int rg = tid >> 4;   // 4-row group
+
+    const uint16_t* xt = x + b * bsx + (int64_t)rb * 128 * ldx + (int64_t)cb * (128 * NSUB);
+    uint4 v[NSUB][2][4];
+#pragma unroll
+    for (int u = 0; u < NSUB; ++u)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int row = h * 64 + rg * 4 + j;
+                v[u][h][j] = *reinterpret_cast<const uint4*>(xt + (int64_t)row * ldx + u * 128 + cc * 8);
+            }
+
+    float amax = 0.0f;
+#pragma unroll
+    for (int u = 0; u < NSUB; ++u)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) amax = absmax8(v[u][h][j], amax);
+    amax = block_max_256(amax, red4);
+    amax = amax_floor(amax, mode.eps_add);
+    const float scale = 127.0f / amax;
+    if (tid == 0) s[b * ssb + rb * ssr + cb * ssc] = stored_scale(amax, scale, mode);
+
+#pragma unroll
+    for (int u = 0; u < NSUB; ++u) {
+        uint2 o[2][4];
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o[h][j] = quant8(v[u][h][j], scale, mode.clamp);
+
+        if (WRITE_Q) {
+            int8_t* qt = q + b * bsq + (int64_t)rb * 128 * ldq + (int64_t)cb * (128 * NSUB) + u * 128 + cc * 8;
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    *reinterpret_cast<uint2*>(qt + (int64_t)(h * 64 + rg * 4 + j) * ldq) = o[h][j];
+        }
+        if (WRITE_QT) {  // NSUB == 1 only (checked on the host)
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const uint32_t w = (e < 4) ? gather_byte(o[h][0].x, o[h][1].x, o[h][2].x, o[h][3].x, e)
+                                               : gather_byte(o[h][0].y, o[h][1].y, o[h][2].y, o[h][3].y, e - 4);
+                    tileT[(cc * 8 + e) * 33 + h * 16 + rg] = w;  // [column of x][4-row group]
+                }
+            __syncthreads();
+            int8_t* qtt = qT + b * bsqt + (int64_t)cb * 128 * ldqt + (int64_t)rb * 128;
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                const int tr = p * 32 + (tid >> 3);  // row of the transposed tile = column of x
+                const int tc = tid & 7;              // 16-byte chunk along the original rows
+                uint4 w;
+                w.x = tileT[tr * 33 + tc * 4 + 0];
+                w.y = tileT[tr * 33 + tc * 4 + 1];
+                w.z = tileT[tr * 33 + tc * 4 + 2];
+                w.w = tileT[tr * 33 + tc * 4 + 3];
+                *reinterpret_cast<uint4*>(qtt + (int64_t)tr * ldqt + tc * 16) = w;
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// Per-row quantiser, one pass.  WG_ROW = false: one wavefront per row (4 rows per
+// workgroup); WG_ROW = true: one 256-thread workgroup per row.  Each thread keeps
+// NLOAD 16-byte chunks of its row in registers.  GROUP16: one scale per 16 chunks
+// (128 columns) instead of per row.
+template <int NLOAD, bool WG_ROW, bool GROUP16>
+__global__ __launch_bounds__(256) void quant_row_kernel(const uint16_t* __restrict__ x, int64_t ldx,
+                                                        int8_t* __restrict__ q, int64_t ldq,
+                                                        float* __restrict__ s, int64_t rows, int cols,
+                                                        QMode mode) {
+    __shared__ float red4[4];
+    constexpr int T = WG_ROW ? 256 : 64;
+    const int t = WG_ROW ? threadIdx.x : (threadIdx.x & 63);
+    const int64_t row = WG_ROW ? (int64_t)blockIdx.x : (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;  // whole wave (or workgroup) leaves together
+    const int nchunk = cols >> 3;
+    const uint16_t* xr = x + row * ldx;
+
+    uint4 v[NLOAD];
+#pragma unroll
+    for (int i = 0; i < NLOAD; ++i) {
+        const int c = t + i * T;
+        v[i] = (c < nchunk) ? *reinterpret_cast<const uint4*>(xr + c * 8) : make_uint4(0, 0, 0, 0);
+    }
+    int8_t* qr = q + row * ldq;
+    if (GROUP16) {
+        const int ngrp = cols >> 7;
+#pragma unroll
+        for (int i = 0; i < NLOAD; ++i) {
+            const int c = t + i * T;
+            float amax = absmax8(v[i], 0.0f);
+#pragma unroll
+            for (int off = 8; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+            amax = amax_floor(amax, mode.eps_add);
+            const float scale = 127.0f / amax;
+            if (c < nchunk) {
+                *reinterpret_cast<uint2*>(qr + c * 8) = quant8(v[i], scale, mode.clamp);
+                if ((c & 15) == 0) s[row * ngrp + (c >> 4)] = stored_scale(amax, scale, mode);
+            }
+        }
+        return;
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NLOAD; ++i) amax = absmax8(v[i], amax);
+    if (WG_ROW)
+        amax = block_max_256(amax, red4);
+    else
+        amax = wave_max(amax);
+    amax = amax_floor(amax, mode.eps_add);
+    const float scale = 127.0f / amax;
+    if (t == 0) s[row] = stored_scale(amax, scale, mode);
+#pragma unroll
+    for (int i = 0; i < NLOAD; ++i) {
+        const int c = t + i * T;
+        if (c < nchunk) *reinterpret_cast<uint2*>(qr + c * 8) = quant8(v[i], scale, mode.clamp);
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// Column absmax: workgroup = 128 rows x 256 columns; thread t reads 16-byte chunks of
+// column chunk t%32 from rows t/32 + 8i.  Partial maxima meet in LDS and are merged
+// into ws[] with an unsigned atomic max (non-negative floats order like their bits).
+__global__ __launch_bounds__(256) void col_absmax_kernel(const uint16_t* __restrict__ x, int64_t ldx,
+                                                         unsigned int* __restrict__ ws, int64_t R, int C) {
+    __shared__ float part[8][256];
+    const int tid = threadIdx.x;
+    const int cc = tid & 31, rg = tid >> 5;
+    const int c0 = blockIdx.x * 256 + cc * 8;
+    const int64_t r0 = (int64_t)blockIdx.y * 128;
+    float m[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (c0 < C) {
+        uint4 v[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+            v[i] = *reinterpret_cast<const uint4*>(x + (r0 + rg + 8 * i) * ldx + c0);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            m[0] = fmaxf(m[0], fabsf(bf16_lo(v[i].x)));
+            m[1] = fmaxf(m[1], fabsf(bf16_hi(v[i].x)));
+            m[2] = fmaxf(m[2], fabsf(bf16_lo(v[i].y)));
+            m[3] = fmaxf(m[3], fabsf(bf16_hi(v[i].y)));
+            m[4] = fmaxf(m[4], fabsf(bf16_lo(v[i].z)));
+            m[5] = fmaxf(m[5], fabsf(bf16_hi(v[i].z)));
+            m[6] = fmaxf(m[6], fabsf(bf16_lo(v[i].w)));
+            m[7] = fmaxf(m[7], fabsf(bf16_hi(v[i].w)));
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) part[rg][cc * 8 + e] = m[e];
+    __syncthreads();
+    float a = part[0][tid];
+#pragma unroll
+    for (int g = 1; g < 8; ++g) a = fmaxf(a, part[g][tid]);
+    const int c = blockIdx.x * 256 + tid;
+    if (c < C) atomicMax(ws + c, __float_as_uint(a));
+}
+
+__global__ void fill_u32_kernel(unsigned int* p, int n, unsigned int v) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+// Quantise a 128x128 tile of x with one scale PER COLUMN (from ws[]) and write it
+// transposed: qT[c][r].  Same thread <-> element map as quant_block_kernel.
+__global__ __launch_bounds__(256) void quant_col_t_kernel(const uint16_t* __restrict__ x, int64_t ldx,
+                                                          int8_t* __restrict__ qT, int64_t ldqt,
+                                                          float* __restrict__ s, const float* __restrict__ ws,
+                                                          int ncb, QMode mode) {
+    __shared__ uint32_t tileT[128 * 33];
+    const int cb = blockIdx.x % ncb;
+    const int rb = blockIdx.x / ncb;
+    const int tid = threadIdx.x;
+    const int cc = tid & 15, rg = tid >> 4;
+    const uint16_t* xt = x + (int64_t)rb * 128 * ldx + (int64_t)cb * 128;
+
+    uint4 v[2][4];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            v[h][j] = *reinterpret_cast<const uint4*>(xt + (int64_t)(h * 64 + rg * 4 + j) * ldx + cc * 8);
+
+    float scale[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const float amax = amax_floor(ws[cb * 128 + cc * 8 + e], mode.eps_add);
+        scale[e] = 127.0f / amax;
+        if (rb == 0 && rg == 0) s[cb * 128 + cc * 8 + e] = stored_scale(amax, scale[e], mode);
+    }
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        uint32_t qq[4][8];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint4& w = v[h][j];
+            qq[j][0] = q1(bf16_lo(w.x), scale[0], mode.clamp);
+            qq[j][1] = q1(bf16_hi(w.x), scale[1], mode.clamp);
+            qq[j][2] = q1(bf16_lo(w.y), scale[2], mode.clamp);
+            qq[j][3] = q1(bf16_hi(w.y), scale[3], mode.clamp);
+            qq[j][4] = q1(bf16_lo(w.z), scale[4], mode.clamp);
+            qq[j][5] = q1(bf16_hi(w.z), scale[5], mode.clamp);
+            qq[j][6] = q1(bf16_lo(w.w), scale[6], mode.clamp);
+            qq[j][7] = q1(bf16_hi(w.w), scale[7], mode.clamp);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            tileT[(cc * 8 + e) * 33 + h * 16 + rg] =
+                qq[0][e] | (qq[1][e] << 8) | (qq[2][e] << 16) | (qq[3][e] << 24);
+    }
+    __syncthreads();
+    int8_t* qtt = qT + (int64_t)cb * 128 * ldqt + (int64_t)rb * 128;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const int tr = p * 32 + (tid >> 3);
+        const int tc = tid & 7;
+        uint4 w;
+        w.x = tileT[tr * 33 + tc * 4 + 0];
+        w.y = tileT[tr * 33 + tc * 4 + 1];
+        w.z = tileT[tr * 33 + tc * 4 + 2];
+        w.w = tileT[tr * 33 + tc * 4 + 3];
+        *reinterpret_cast<uint4*>(qtt + (int64_t)tr * ldqt + tc * 16) = w;
+    }
+}
+
+static int parse_mode(int qflags, int inv_mode, QMode* m) {
+    if (qflags & ~(TI8_Q_CLAMP | TI8_Q_EPS_ADD | TI8_Q_SCALE_BF16)) return fail(TI8_ERR_MODE, "unknown quantiser flag 0x%x", qflags);
+    if (inv_mode < 0 || inv_mode > 3) return fail(TI8_ERR_MODE, "unknown inv_mode %d", inv_mode);
+    m->clamp = (qflags & TI8_Q_CLAMP) ? 1 : 0;
+    m->eps_add = (qflags & TI8_Q_EPS_ADD) ? 1 : 0;
+    m->scale_bf16 = (qflags & TI8_Q_SCALE_BF16) ? 1 : 0;
+    m->inv_mode = inv_mode;
+    return TI8_OK;
+}
+
+}  // namespace ti8
+
+using namespace ti8;
+
+extern "C" int ti8_quant_block(const void* x, int64_t bsx, int64_t ldx, int8_t* q, int64_t bsq, int64_t ldq,
+                               int8_t* qT, int64_t bsqt, int64_t ldqt, float* s, int64_t ssb, int64_t ssr,
+                               int64_t ssc, int64_t B, int64_t R, int64_t C, int group_c, int qflags,
+                               int inv_mode, ti8_stream_t stream) {
+    QMode mode;
+    if (int e = parse_mode(qflags, inv_mode, &mode)) return e;
+    if (!x || !s || (!q && !qT)) return fail(TI8_ERR_NULL, "ti8_quant_block: x, s and one of q/qT are required");
+    if (group_c != 128 && group_c != 256) return fail(TI8_ERR_MODE, "ti8_quant_block: group_c must be 128 or 256, got %d", group_c);
+    if (qT && group_c != 128) return fail(TI8_ERR_MODE, "ti8_quant_block: the transposed output needs group_c = 128");
+    if (B <= 0 || R <= 0 || C <= 0 || R % 128 || C % group_c)
+        return fail(TI8_ERR_SHAPE, "ti8_quant_block: need B>0, R%%128==0, C%%%d==0; got B=%lld R=%lld C=%lld", group_c,
+                    (long long)B, (long long)R, (long long)C);
+    if (ldx < C || (q && ldq < C) || (qT && ldqt < R)) return fail(TI8_ERR_SHAPE, "ti8_quant_block: leading dimension smaller than the row length");
+    if (!aligned16(x) || (ldx % 8) || (bsx % 8) || (q && (!aligned16(q) || (ldq % 16) || (bsq % 16))) ||
+        (qT && (!aligned16(qT) || (ldqt % 16) || (bsqt % 16))))
+        return fail(TI8_ERR_ALIGN, "ti8_quant_block: pointers must be 16-byte aligned and strides multiples of 16 bytes");
+    const int64_t ntiles = B * (R / 128) * (C / group_c);
+    if (ntiles > 0x7fffffffLL) return fail(TI8_ERR_SHAPE, "ti8_quant_block: too many tiles");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uint16_t* xp = static_cast<const uint16_t*>(x);
+    const int nrb = (int)(R / 128), ncb = (int)(C / group_c);
+    dim3 grid((unsigned)ntiles), block(256);
+#define TI8_LAUNCH_QB(NSUB, WQ, WQT)                                                                          \
+    hipLaunchKernelGGL((quant_block_kernel<NSUB, WQ, WQT>), grid, block, 0, st, xp, bsx, ldx, q, bsq, ldq, qT, \
+                       bsqt, ldqt, s, ssb, ssr, ssc, nrb, ncb, mode)
+    if (group_c == 256) TI8_LAUNCH_QB(2, true, false);
+    else if (q && qT) TI8_LAUNCH_QB(1, true, true);
+    else if (q) TI8_LAUNCH_QB(1, true, false);
+    else TI8_LAUNCH_QB(1, false, true);
+#undef TI8_LAUNCH_QB
+    return check_launch("ti8_quant_block");
+}
+
+extern "C" int ti8_quant_row(const void* x, int64_t ldx, int8_t* q, int64_t ldq, float* s, int64_t rows,
+                             int64_t cols, int group, int qflags, int inv_mode, ti8_stream_t stream) {
+    QMode mode;
+    if (int e = parse_mode(qflags, inv_mode, &mode)) return e;
+    if (!x || !q || !s) return fail(TI8_ERR_NULL, "ti8_quant_row: x, q and s are required");
+    if (group != 0 && group != 128) return fail(TI8_ERR_MODE, "ti8_quant_row: group must be 0 or 128, got %d", group);
+    if (rows <= 0 || cols <= 0 || cols % 128 || cols > 32768 || rows > 0x7fffffffLL)
+        return fail(TI8_ERR_SHAPE, "ti8_quant_row: need rows>0, cols%%128==0, cols<=32768; got rows=%lld cols=%lld",
+                    (long long)rows, (long long)cols);
+    if (ldx < cols || ldq < cols) return fail(TI8_ERR_SHAPE, "ti8_quant_row: leading dimension smaller than cols");
+    if (!aligned16(x) || !aligned16(q) || (ldx % 8) || (ldq % 16))
+        return fail(TI8_ERR_ALIGN, "ti8_quant_row: pointers must be 16-byte aligned and strides multiples of 16 bytes");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uint16_t* xp = static_cast<const uint16_t*>(x);
+    const int nchunk = (int)(cols / 8);
+    const int c = (int)cols;
+#define TI8_LAUNCH_QR(NL, WG, G16, GRID) \
+    hipLaunchKernelGGL((quant_row_kernel<NL, WG, G16>), dim3((unsigned)(GRID)), dim3(256), 0, st, xp, ldx, q, ldq, s, rows, c, mode)
+    const int64_t g4 = (rows + 3) / 4;
+    if (group == 128) {
+        if (nchunk <= 64 * 8) TI8_LAUNCH_QR(8, false, true, g4);
+        else if (nchunk <= 256 * 8) TI8_LAUNCH_QR(8, true, true, rows);
+        else TI8_LAUNCH_QR(16, true, true, rows);
+    } else if (nchunk <= 64 * 2) TI8_LAUNCH_QR(2, false, false, g4);
+    else if (nchunk <= 64 * 4) TI8_LAUNCH_QR(4, false, false, g4);
+    else if (nchunk <= 64 * 8) TI8_LAUNCH_QR(8, false, false, g4);
+    else if (nchunk <= 256 * 4) TI8_LAUNCH_QR(4, true, false, rows);
+    else if (nchunk <= 256 * 8) TI8_LAUNCH_QR(8, true, false, rows);
+    else TI8_LAUNCH_QR(16, true, false, rows);
+#undef TI8_LAUNCH_QR
+    return check_launch("ti8_quant_row");
+}
+
+extern "C" int ti8_quant_col_t(const void* x, int64_t ldx, int8_t* qT, int64_t ldqt, float* s, float* ws,
+                               int64_t R, int64_t C, int qflags, int inv_mode, ti8_stream_t stream) {
+    QMode mode;
+    if (int e = parse_mode(qflags, inv_mode, &mode)) return e;
+    if (!x || !qT || !s || !ws) return fail(TI8_ERR_NULL, "ti8_quant_col_t: x, qT, s and ws are required");
+    if (R <= 0 || C <= 0 || R % 128 || C % 128 || C > 0x7fffffffLL)
+        return fail(TI8_ERR_SHAPE, "ti8_quant_col_t: need R%%128==0 and C%%128==0; got R=%lld C=%lld", (long long)R, (long long)C);
+    if (ldx < C || ldqt < R) return fail(TI8_ERR_SHAPE, "ti8_quant_col_t: leading dimension smaller than the row length");
+    if (!aligned16(x) || !aligned16(qT) || (ldx % 8) || (ldqt % 16))
+        return fail(TI8_ERR_ALIGN, "ti8_quant_col_t: pointers must be 16-byte aligned and strides multiples of 16 bytes");
+    const int64_t ntiles = (R / 128) * (C / 128);
+    if (ntiles > 0x7fffffffLL || R / 128 > 65535) return fail(TI8_ERR_SHAPE, "ti8_quant_col_t: too many tiles");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uint16_t* xp = static_cast<const uint16_t*>(x);
+    unsigned int* wsu = reinterpret_cast<unsigned int*>(ws);
+    hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((C + 255) / 256)), dim3(256), 0, st, wsu, (int)C, 0u);
+    hipLaunchKernelGGL(col_absmax_kernel, dim3((unsigned)((C + 255) / 256), (unsigned)(R / 128)), dim3(256), 0, st, xp,
+                       ldx, wsu, R, (int)C);
+    hipLaunchKernelGGL(quant_col_t_kernel, dim3((unsigned)ntiles), dim3(256), 0, st, xp, ldx, qT, ldqt, s, ws,
+                       (int)(C / 128), mode);
+    return check_launch("ti8_quant_col_t");
+}

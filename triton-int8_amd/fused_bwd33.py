@@ -1,0 +1,28 @@
+""""Fused" quantise + GEMM, 3-D x 3-D: drop-in for triton/fused_triton_bwd33.py.
+
+Both operands are scaled per 128x128 tile with the fused formula (additive 1e-5, no
+clamp).  The reference autotunes its tile shape, and BLOCK_K in {64, 128} changes the
+quantisation groups (triton/fused_triton_bwd33.py:10-23); this implementation fixes
+the 128x128x128 configuration its host wrapper names (:65-67).
+"""
+import torch
+
+from . import ops
+from ._common import calc_diff
+from ._lib import COMBINE_DIV_PROD, INV_MULTIPLIER, SCALE_BLOCK128
+
+__all__ = ["fused_int8_gemm", "bwd_33", "calc_diff"]
+
+
+def fused_int8_gemm(A_bf, B_bf, strict=False):
+    """bf16 [B,M,K] x bf16 [B,N,K] -> bf16 [B,M,N] (triton/fused_triton_bwd33.py:63-86)."""
+    if A_bf.dim() != 3 or B_bf.dim() != 3:
+        raise ValueError("A_bf must be [B, M, K] and B_bf [B, N, K]")
+    qa, sa = ops.quant_block(A_bf, clamp=False, eps_add=True, inv_mode=INV_MULTIPLIER, out="contiguous")
+    qb, sb = ops.quant_block(B_bf, clamp=False, eps_add=True, inv_mode=INV_MULTIPLIER, out="contiguous")
+    return ops.gemm_i8_nt(qa, qb, sa, SCALE_BLOCK128, sb, SCALE_BLOCK128, combine=COMBINE_DIV_PROD, strict=strict)
+
+
+def bwd_33(a: torch.Tensor, b: torch.Tensor):
+    """triton/fused_triton_bwd33.py:94-98."""
+    return fused_int8_gemm(A_bf=a.cuda(), B_bf=b.cuda())

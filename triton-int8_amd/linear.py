@@ -1,0 +1,217 @@
+"""INT8 linear layer built on the reference's two entry points.
+
+The reference stops at ``fwd_32`` / ``bwd_33`` (NT GEMMs that contract over the last
+dim of both operands) and never shows how a linear layer maps onto them.  The wiring
+used here is
+
+    Y  = fwd_32(X [B,M,K],       W   [N,K])
+    dX = fwd_32(dY[B,M,N],       W^T [K,N])
+    dW = bwd_33(dY^T [1,N,B*M],  X^T [1,K,B*M])[0]
+
+``scheme``
+  "block_channel"   reference literal (triton/block_channel_fwd32.py:221-222,
+                    triton/block_channel_bwd33.py:153-154): the 3-D operand per 128x128
+                    block, the 2-D operand per row; bwd_33 both per block.
+  "row_block"       "per-token activations, per-128x128-block weights": the first operand
+                    of every GEMM per row, the second per block.
+  "double_channel"  per-row scales on both operands, int32 accumulation over the whole K
+                    (triton/double-channle_fwd32.py), optional full-length Hadamard.
+``hadamard=128`` ("block_channel" / "row_block"): both operands of every GEMM are rotated
+by a block-diagonal H_128 along the contraction dim before quantisation and the result is
+multiplied by 2^-7 (exact) in the GEMM epilogue.
+
+MI355X-specific data flow: a 128x128 block quantisation commutes with transposition, so
+X and dY are each read ONCE by a quantiser that writes both the int8 tensor and its
+transpose (the K-contiguous operand of the dW GEMM); W^T is quantised per row by a
+column-absmax kernel that never materialises W^T in bf16.
+"""
+import torch
+
+from . import ops
+from ._lib import (COMBINE_MUL_MUL, INV_AMAX_DIV_127, INV_RCP_OF_SCALE, SCALE_BLOCK128, SCALE_ROW)
+
+__all__ = ["linear_forward", "linear_backward", "linear_fwd_bwd", "Int8LinearFunction", "Int8Linear", "SCHEMES"]
+
+SCHEMES = ("block_channel", "row_block", "double_channel")
+
+
+def _check(scheme, hadamard):
+    if scheme not in SCHEMES:
+        raise ValueError(f"unknown scheme {scheme!r}; expected one of {SCHEMES}")
+    if scheme == "double_channel" and hadamard not in (None, "full"):
+        raise ValueError("double_channel supports hadamard=None or 'full'")
+    if scheme != "double_channel" and hadamard not in (None, 128):
+        raise ValueError(f"{scheme} supports hadamard=None or 128")
+
+
+def _h128(x2d):
+    return ops.fwht(x2d, 128)
+
+
+def _gemm_bc(a_q, a_s, a_mode, b_q, b_s, b_mode, out_scale=1.0):
+    """2-D operands through the batched block-channel GEMM (batch of one)."""
+    a_s3 = a_s.reshape(1, -1) if a_mode == SCALE_ROW else a_s[None]
+    return ops.gemm_i8_nt(a_q[None], b_q, a_s3, a_mode, b_s, b_mode, combine=COMBINE_MUL_MUL,
+                          out_scale=out_scale)[0]
+
+
+def _gemm_dc(a_q, a_s, b_q, b_s, post_scale=0.0):
+    return ops.gemm_i8_nt(a_q[None], b_q, a_s.reshape(1, -1), SCALE_ROW, b_s, SCALE_ROW, acc_i32_full=True,
+                          post_scale=post_scale)[0]
+
+
+def linear_forward(X2, W, scheme="block_channel", hadamard=None):
+    """X2 bf16 [T, K] (tokens flattened), W bf16 [N, K] -> (Y bf16 [T, N], saved) where
+    ``saved`` holds what the backward can reuse (quantised X^T and its scales)."""
+    _check(scheme, hadamard)
+    saved = {}
+    if scheme == "block_channel":
+        if hadamard == 128:
+            q, s = ops.quant_block(_h128(X2)[None], clamp=True)
+            wq, ws = ops.quant_row(_h128(W), clamp=True)
+            return _gemm_bc(q[0], s[0], SCALE_BLOCK128, wq, ws, SCALE_ROW, 2.0 ** -7), saved
+        q, qT, s = ops.quant_block(X2[None], clamp=True, with_transpose=True)
+        saved["XqT"], saved["Xs"] = qT[0], s[0]
+        wq, ws = ops.quant_row(W, clamp=True)
+        return _gemm_bc(q[0], s[0], SCALE_BLOCK128, wq, ws, SCALE_ROW), saved
+    if scheme == "row_block":
+        xs_in, w_in = (_h128(X2), _h128(W)) if hadamard == 128 else (X2, W)
+        q, s = ops.quant_row(xs_in, clamp=True)
+        if hadamard == 128:
+            wq, ws = ops.quant_block(w_in[None], clamp=True)
+            return _gemm_bc(q, s, SCALE_ROW, wq[0], ws[0], SCALE_BLOCK128, 2.0 ** -7), saved
+        wq, wqT, ws = ops.quant_block(w_in[None], clamp=True, with_transpose=True)
+        saved["WqT"], saved["Ws"] = wqT[0], ws[0]
+        return _gemm_bc(q, s, SCALE_ROW, wq[0], ws[0], SCALE_BLOCK128), saved
+    # double_channel
+    K = X2.shape[1]
+    if hadamard == "full":
+        q, s = ops.quant_row(ops.fwht(X2), clamp=True, inv_mode=INV_AMAX_DIV_127)
+        wq, ws = ops.quant_row(ops.fwht(W), clamp=True, inv_mode=INV_AMAX_DIV_127)
+        return _gemm_dc(q, s, wq, ws, 1.0 / K), saved
+    q, s = ops.quant_row(X2, clamp=True, inv_mode=INV_AMAX_DIV_127)
+    wq, ws = ops.quant_row(W, clamp=True, inv_mode=INV_AMAX_DIV_127)
+    return _gemm_dc(q, s, wq, ws), saved
+
+
+def linear_backward(dY2, X2, W, scheme="block_channel", hadamard=None, saved=None):
+    """dY2 bf16 [T, N], X2 bf16 [T, K], W bf16 [N, K] -> (dX bf16 [T, K], dW bf16 [N, K])."""
+    _check(scheme, hadamard)
+    saved = saved or {}
+    T, N = dY2.shape
+    K = X2.shape[1]
+    if scheme == "block_channel":
+        if hadamard == 128:
+            # H_128 along N for dX, along the tokens for dW: two differently rotated copies
+            dq, ds = ops.quant_block(_h128(dY2)[None], clamp=True)
+            wtq, wts = ops.quant_row(_h128(W.t().contiguous()), clamp=True)
+            dX = _gemm_bc(dq[0], ds[0], SCALE_BLOCK128, wtq, wts, SCALE_ROW, 2.0 ** -7)
+            dyt, dyts = ops.quant_block(_h128(dY2.t().contiguous())[None], clamp=False)
+            xt, xts = ops.quant_block(_h128(X2.t().contiguous())[None], clamp=False)
+            dW = ops.gemm_i8_nt(dyt, xt, dyts, SCALE_BLOCK128, xts, SCALE_BLOCK128, out_scale=2.0 ** -7)[0]
+            return dX, dW
+        dq, dqT, ds = ops.quant_block(dY2[None], clamp=True, with_transpose=True)
+        wtq, wts = ops.quant_col_t(W, clamp=True)                    # W^T [K,N] per row
+        dX = _gemm_bc(dq[0], ds[0], SCALE_BLOCK128, wtq, wts, SCALE_ROW)
+        if "XqT" in saved:
+            xqT, xs = saved["XqT"], saved["Xs"]
+        else:
+            _, xqT3, xs3 = ops.quant_block(X2[None], clamp=True, with_transpose=True)
+            xqT, xs = xqT3[0], xs3[0]
+        # scales of the transposed operands are the transposed scale grids
+        dW = ops.gemm_i8_nt(dqT, xqT[None], ds.transpose(1, 2), SCALE_BLOCK128, xs.t()[None], SCALE_BLOCK128)[0]
+        return dX, dW
+    if scheme == "row_block":
+        if hadamard == 128:
+            dq, ds = ops.quant_row(_h128(dY2), clamp=True)
+            wtq, wts = ops.quant_block(_h128(W.t().contiguous())[None], clamp=True)
+            dX = _gemm_bc(dq, ds, SCALE_ROW, wtq[0], wts[0], SCALE_BLOCK128, 2.0 ** -7)
+            dytq, dyts = ops.quant_row(_h128(dY2.t().contiguous()), clamp=True)
+            xtq, xts = ops.quant_block(_h128(X2.t().contiguous())[None], clamp=True)
+            dW = _gemm_bc(dytq, dyts, SCALE_ROW, xtq[0], xts[0], SCALE_BLOCK128, 2.0 ** -7)
+            return dX, dW
+        dq, ds = ops.quant_row(dY2, clamp=True)
+        if "WqT" in saved:
+            wqT, ws = saved["WqT"], saved["Ws"]
+        else:
+            _, wqT3, ws3 = ops.quant_block(W[None], clamp=True, with_transpose=True)
+            wqT, ws = wqT3[0], ws3[0]
+        dX = _gemm_bc(dq, ds, SCALE_ROW, wqT, ws.t(), SCALE_BLOCK128)
+        dytq, dyts = ops.quant_col_t(dY2, clamp=True)                # dY^T [N,T] per row
+        _, xqT, xs = ops.quant_block(X2[None], clamp=True, with_transpose=True)
+        dW = _gemm_bc(dytq, dyts, SCALE_ROW, xqT[0], xs[0].t(), SCALE_BLOCK128)
+        return dX, dW
+    # double_channel
+    if hadamard == "full":
+        dq, ds = ops.quant_row(ops.fwht(dY2), clamp=True, inv_mode=INV_AMAX_DIV_127)
+        wtq, wts = ops.quant_row(ops.fwht(W.t().contiguous()), clamp=True, inv_mode=INV_AMAX_DIV_127)
+        dX = _gemm_dc(dq, ds, wtq, wts, 1.0 / N)
+        dytq, dyts = ops.quant_row(ops.fwht(dY2.t().contiguous()), clamp=True, inv_mode=INV_AMAX_DIV_127)
+        xtq, xts = ops.quant_row(ops.fwht(X2.t().contiguous()), clamp=True, inv_mode=INV_AMAX_DIV_127)
+        dW = _gemm_dc(dytq, dyts, xtq, xts, 1.0 / T)
+        return dX, dW
+    dq, ds = ops.quant_row(dY2, clamp=True, inv_mode=INV_AMAX_DIV_127)
+    wtq, wts = ops.quant_col_t(W, clamp=True, inv_mode=INV_AMAX_DIV_127)
+    dX = _gemm_dc(dq, ds, wtq, wts)
+    dytq, dyts = ops.quant_col_t(dY2, clamp=True, inv_mode=INV_AMAX_DIV_127)
+    xtq, xts = ops.quant_col_t(X2, clamp=True, inv_mode=INV_AMAX_DIV_127)
+    dW = _gemm_dc(dytq, dyts, xtq, xts)
+    return dX, dW
+
+
+def linear_fwd_bwd(X, W, dY, scheme="block_channel", hadamard=None):
+    """One forward + backward of the layer: returns (Y, dX, dW) for X [B,M,K] or [M,K]."""
+    lead = X.shape[:-1]
+    K, N = X.shape[-1], W.shape[0]
+    X2, dY2 = X.reshape(-1, K), dY.reshape(-1, N)
+    Y, saved = linear_forward(X2, W, scheme, hadamard)
+    dX, dW = linear_backward(dY2, X2, W, scheme, hadamard, saved)
+    return Y.reshape(*lead, N), dX.reshape(*lead, K), dW
+
+
+class Int8LinearFunction(torch.autograd.Function):
+    """y = x W^T (+ bias) with every GEMM of forward and backward on the INT8 path."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, scheme, hadamard):
+        K, N = x.shape[-1], weight.shape[0]
+        x2 = x.reshape(-1, K)
+        y, saved = linear_forward(x2, weight, scheme, hadamard)
+        ctx.scheme, ctx.hadamard, ctx.saved_q = scheme, hadamard, saved
+        ctx.has_bias = bias is not None
+        ctx.save_for_backward(x2, weight)
+        if bias is not None:
+            y = y + bias
+        return y.reshape(*x.shape[:-1], N)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x2, weight = ctx.saved_tensors
+        N = weight.shape[0]
+        dy2 = dy.reshape(-1, N).contiguous()
+        dx, dw = linear_backward(dy2, x2, weight, ctx.scheme, ctx.hadamard, ctx.saved_q)
+        db = dy2.sum(dim=0).to(dy.dtype) if ctx.has_bias else None
+        return dx.reshape(*dy.shape[:-1], x2.shape[1]), dw, db, None, None
+
+
+class Int8Linear(torch.nn.Module):
+    """``torch.nn.Linear`` whose three GEMMs (Y, dX, dW) run through the INT8 path.
+    in_features, out_features and the number of tokens must be multiples of 128."""
+
+    def __init__(self, in_features, out_features, bias=False, scheme="block_channel", hadamard=None,
+                 device=None, dtype=torch.bfloat16):
+        super().__init__()
+        _check(scheme, hadamard)
+        if in_features % 128 or out_features % 128:
+            raise ValueError("in_features and out_features must be multiples of 128")
+        self.in_features, self.out_features = in_features, out_features
+        self.scheme, self.hadamard = scheme, hadamard
+        self.weight = torch.nn.Parameter(torch.empty(out_features, in_features, device=device, dtype=dtype))
+        self.bias = torch.nn.Parameter(torch.zeros(out_features, device=device, dtype=dtype)) if bias else None
+        torch.nn.init.normal_(self.weight, std=0.02)
+
+    def forward(self, x):
+        return Int8LinearFunction.apply(x, self.weight, self.bias, self.scheme, self.hadamard)
+
+    def extra_repr(self):
+        return f"in_features={self.in_features}, out_features={self.out_features}, scheme={self.scheme}, hadamard={self.hadamard}"

@@ -1,0 +1,214 @@
+"""Host wrappers (allocate outputs, derive strides, pick the stream) around the C ABI.
+
+Every function takes and returns torch tensors on a HIP device, enqueues on the
+current torch stream and never synchronises.  Arguments the kernels cannot take
+(wrong dtype/device, sizes that are not multiples of the tile) raise ``ValueError``
+here, before anything is launched.
+"""
+import torch
+
+from . import _lib
+from ._lib import (COMBINE_DIV_PROD, COMBINE_MUL_MUL, COMBINE_MUL_PROD, GEMM_STRICT, INV_AMAX_DIV_127,
+                   INV_AMAX_MUL_RCP127, INV_MULTIPLIER, INV_RCP_OF_SCALE, Q_CLAMP, Q_EPS_ADD, Q_SCALE_BF16,
+                   SCALE_BLOCK128, SCALE_BLOCK_K256, SCALE_ROW, SCALE_ROW_K128)
+
+__all__ = ["quant_block", "quant_row", "quant_col_t", "fwht", "gemm_i8_nt", "gemm_i8_nt_i32"]
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _need(cond, msg):
+    if not cond:
+        raise ValueError(msg)
+
+
+def _check_bf16(x, name):
+    _need(isinstance(x, torch.Tensor) and x.is_cuda, f"{name} must be a tensor on the GPU")
+    _need(x.dtype == torch.bfloat16, f"{name} must be bfloat16, got {x.dtype}")
+
+
+def _qflags(clamp, eps_add, scale_bf16):
+    return (Q_CLAMP if clamp else 0) | (Q_EPS_ADD if eps_add else 0) | (Q_SCALE_BF16 if scale_bf16 else 0)
+
+
+def quant_block(x, *, clamp=True, group_c=128, eps_add=False, scale_bf16=False, inv_mode=INV_RCP_OF_SCALE,
+                out="like", with_transpose=False):
+    """Per-128 x group_c-block absmax quantisation of ``x`` [B, M, N] (bf16).
+
+    ``x`` may be row-major (last stride 1) or a transposed view of a row-major
+    tensor (stride(1) == 1); it is read in place either way.  ``out``:
+      "like"        q has the strides of ``x`` (what ``torch.empty_like`` gives)
+      "contiguous"  q is contiguous in the logical [B, M, N] orientation
+    ``with_transpose`` additionally returns ``qT`` = contiguous [B, N, M] int8 holding
+    ``q`` transposed, written by the same kernel from the same registers.
+    Returns ``(q, s)`` or ``(q, qT, s)``; ``s`` is fp32 [B, M/128, N/group_c]."""
+    _check_bf16(x, "x")
+    _need(x.dim() == 3, "x must be [B, M, N]")
+    B, M, N = x.shape
+    _need(B > 0 and M > 0 and N > 0, "empty tensors are not supported")
+    if x.stride(2) == 1 or N == 1:
+        xc, transposed = x, False
+    elif x.stride(1) == 1:
+        xc, transposed = x.transpose(1, 2), True
+    else:
+        xc, transposed = x.contiguous(), False
+    if xc.stride(2) != 1 or (B > 1 and xc.stride(0) % 8) or xc.stride(1) % 8 or xc.data_ptr() % 16:
+        xc = xc.contiguous()
+    _need(group_c in (128, 256), "group_c must be 128 or 256")
+    _need(out in ("like", "contiguous"), "out must be 'like' or 'contiguous'")
+    _need(not (transposed or with_transpose) or group_c == 128, "transposed layouts need 128 x 128 blocks")
+    _need(M % 128 == 0 and N % (group_c if not transposed else 128) == 0,
+          f"block quantisation needs M % 128 == 0 and N % {group_c} == 0, got M={M} N={N}")
+    R, C = xc.shape[1], xc.shape[2]          # canonical (row-major) view of the memory
+    dev = x.device
+    s = torch.empty((B, M // 128, N // group_c), dtype=torch.float32, device=dev)
+    if transposed:   # canonical tile (rb, cb) is logical tile (mb = cb, nb = rb)
+        ssr, ssc = s.stride(2), s.stride(1)
+    else:
+        ssr, ssc = s.stride(1), s.stride(2)
+    # which of the kernel's two outputs are needed: qc in the memory ("canonical")
+    # orientation [B, R, C], qct in the transposed one [B, C, R]
+    if transposed:
+        want_canon, want_canon_t = (out == "like" or with_transpose), (out == "contiguous")
+    else:
+        want_canon, want_canon_t = True, with_transpose
+    qc = torch.empty((B, R, C), dtype=torch.int8, device=dev) if want_canon else None
+    qct = torch.empty((B, C, R), dtype=torch.int8, device=dev) if want_canon_t else None
+    _lib.call("ti8_quant_block", xc.data_ptr(), xc.stride(0), xc.stride(1),
+              qc.data_ptr() if qc is not None else None, R * C, C,
+              qct.data_ptr() if qct is not None else None, R * C, R,
+              s.data_ptr(), s.stride(0), ssr, ssc, B, R, C, group_c,
+              _qflags(clamp, eps_add, scale_bf16), inv_mode, _stream())
+    if not transposed:
+        q = qc
+        qT = qct
+    else:
+        q = qct if out == "contiguous" else qc.transpose(1, 2)
+        qT = qc  # canonical orientation IS the logical transpose
+    return (q, qT, s) if with_transpose else (q, s)
+
+
+def quant_row(x, *, clamp=True, group=0, eps_add=False, scale_bf16=False, inv_mode=INV_RCP_OF_SCALE):
+    """Per-row (``group=0``) or per-(row, 128 columns) absmax quantisation of the last dim.
+    ``x``: bf16 [..., cols].  Returns ``(q, s)`` with ``s`` fp32 [...] or [..., cols/128]."""
+    _check_bf16(x, "x")
+    _need(x.dim() >= 1 and x.numel() > 0, "x must be a non-empty tensor")
+    cols = x.shape[-1]
+    _need(cols % 128 == 0 and cols <= 32768, f"per-row quantisation needs cols % 128 == 0 and cols <= 32768, got {cols}")
+    x2 = x.reshape(-1, cols)
+    if x2.stride(1) != 1 or x2.stride(0) % 8 or x2.data_ptr() % 16:
+        x2 = x2.contiguous()
+    rows = x2.shape[0]
+    q = torch.empty((rows, cols), dtype=torch.int8, device=x.device)
+    s = torch.empty((rows, cols // 128) if group else (rows,), dtype=torch.float32, device=x.device)
+    _lib.call("ti8_quant_row", x2.data_ptr(), x2.stride(0), q.data_ptr(), cols, s.data_ptr(), rows, cols, group,
+              _qflags(clamp, eps_add, scale_bf16), inv_mode, _stream())
+    lead = x.shape[:-1]
+    return q.reshape(*lead, cols), s.reshape(*lead, cols // 128) if group else s.reshape(*lead)
+
+
+def quant_col_t(x, *, clamp=True, inv_mode=INV_RCP_OF_SCALE):
+    """Per-column absmax quantisation of ``x`` [R, C] with transposed output: the per-row
+    quantiser applied to ``x.T``.  Returns ``(qT int8 [C, R], s fp32 [C])``."""
+    _check_bf16(x, "x")
+    _need(x.dim() == 2, "x must be [R, C]")
+    R, C = x.shape
+    _need(R % 128 == 0 and C % 128 == 0, f"column quantisation needs R % 128 == 0 and C % 128 == 0, got {R}x{C}")
+    if x.stride(1) != 1 or x.stride(0) % 8 or x.data_ptr() % 16:
+        x = x.contiguous()
+    qT = torch.empty((C, R), dtype=torch.int8, device=x.device)
+    s = torch.empty((C,), dtype=torch.float32, device=x.device)
+    ws = torch.empty((C,), dtype=torch.float32, device=x.device)
+    _lib.call("ti8_quant_col_t", x.data_ptr(), x.stride(0), qT.data_ptr(), R, s.data_ptr(), ws.data_ptr(), R, C,
+              _qflags(clamp, False, False), inv_mode, _stream())
+    return qT, s
+
+
+def fwht(x, n=None, scale=1.0):
+    """Un-normalised Walsh-Hadamard transform over groups of ``n`` (default: all) of the last dim."""
+    _check_bf16(x, "x")
+    cols = x.shape[-1]
+    n = cols if n is None else n
+    _need(n >= 128 and n <= 32768 and (n & (n - 1)) == 0, f"n must be a power of two in [128, 32768], got {n}")
+    _need(cols % n == 0, f"last dim {cols} is not a multiple of n={n}")
+    x2 = x.reshape(-1, cols)
+    if x2.stride(1) != 1 or x2.stride(0) % 8 or x2.data_ptr() % 16:
+        x2 = x2.contiguous()
+    y = torch.empty((x2.shape[0], cols), dtype=torch.bfloat16, device=x.device)
+    _lib.call("ti8_fwht", x2.data_ptr(), x2.stride(0), y.data_ptr(), cols, x2.shape[0], cols, n, float(scale), _stream())
+    return y.reshape(x.shape)
+
+
+def _k_contig(t):
+    if t.stride(-1) != 1 or any(st % 16 for st in t.stride()[:-1]) or t.data_ptr() % 16:
+        t = t.contiguous()
+    return t
+
+
+def _scale_desc(s, mode, rows, nkb, batch, batched, who):
+    """(ptr, batch stride, row stride, k stride) of a scale tensor for operand `who`."""
+    _need(s.dtype == torch.float32 and s.is_cuda, f"{who} scale must be a float32 GPU tensor")
+    if mode == SCALE_ROW:
+        shape = (batch, rows) if batched else (rows,)
+        _need(s.numel() == batch * rows if batched else s.numel() == rows,
+              f"{who} per-row scale must have {shape} elements, got {tuple(s.shape)}")
+        v = s.reshape(shape)
+        return v, (v.stride(0) if batched else 0), v.stride(-1), 0
+    if mode == SCALE_BLOCK128:
+        shape = (rows // 128, nkb)
+    elif mode == SCALE_ROW_K128:
+        shape = (rows, nkb)
+    else:
+        shape = (rows // 128, nkb // 2)
+    full = ((batch,) + shape) if batched else shape
+    _need(tuple(s.shape) == full or (not batched and tuple(s.shape) == (1,) + shape),
+          f"{who} scale must have shape {full}, got {tuple(s.shape)}")
+    v = s.reshape(full)
+    return v, (v.stride(0) if batched else 0), v.stride(-2), v.stride(-1)
+
+
+def gemm_i8_nt(A, B, sA, modeA, sB, modeB, *, acc_i32_full=False, combine=COMBINE_MUL_MUL, out_scale=1.0,
+               post_scale=0.0, strict=False, out=None):
+    """C[b] = dequant(A[b] @ B[b]^T): A int8 [batch, M, K]; B int8 [N, K] (shared) or [batch, N, K]."""
+    _need(A.dtype == torch.int8 and B.dtype == torch.int8 and A.is_cuda and B.is_cuda, "A and B must be int8 GPU tensors")
+    _need(A.dim() == 3 and B.dim() in (2, 3), "A must be [batch, M, K]; B [N, K] or [batch, N, K]")
+    batch, M, K = A.shape
+    N = B.shape[-2]
+    _need(B.shape[-1] == K, f"K mismatch: A has {K}, B has {B.shape[-1]}")
+    _need(B.dim() == 2 or B.shape[0] == batch, "batch mismatch between A and B")
+    _need(M % 128 == 0 and N % 128 == 0 and K % 128 == 0 and batch > 0,
+          f"M, N, K must be positive multiples of 128, got M={M} N={N} K={K}")
+    A, B = _k_contig(A), _k_contig(B)
+    nkb = K // 128
+    sAv, sa_bs, sa_rs, sa_ks = _scale_desc(sA, modeA, M, nkb, batch, True, "A")
+    sBv, sb_bs, sb_rs, sb_ks = _scale_desc(sB, modeB, N, nkb, batch, B.dim() == 3, "B")
+    if out is None:
+        out = torch.empty((batch, M, N), dtype=torch.bfloat16, device=A.device)
+    else:
+        _need(out.shape == (batch, M, N) and out.dtype == torch.bfloat16 and out.stride(2) == 1, "bad `out` tensor")
+    _lib.call("ti8_gemm_i8_nt", A.data_ptr(), A.stride(0), A.stride(1),
+              B.data_ptr(), B.stride(0) if B.dim() == 3 else 0, B.stride(-2),
+              out.data_ptr(), out.stride(0), out.stride(1),
+              sAv.data_ptr(), modeA, sa_bs, sa_rs, sa_ks, sBv.data_ptr(), modeB, sb_bs, sb_rs, sb_ks,
+              batch, M, N, K, 1 if acc_i32_full else 0, combine, float(out_scale), float(post_scale),
+              GEMM_STRICT if strict else 0, _stream())
+    return out
+
+
+def gemm_i8_nt_i32(A, B):
+    """Raw int32 accumulators of A[b] @ B[b]^T over the whole K."""
+    _need(A.dtype == torch.int8 and B.dtype == torch.int8 and A.is_cuda and B.is_cuda, "A and B must be int8 GPU tensors")
+    _need(A.dim() == 3 and B.dim() in (2, 3), "A must be [batch, M, K]; B [N, K] or [batch, N, K]")
+    batch, M, K = A.shape
+    N = B.shape[-2]
+    _need(B.shape[-1] == K and (B.dim() == 2 or B.shape[0] == batch), "shape mismatch between A and B")
+    _need(M % 128 == 0 and N % 128 == 0 and K % 128 == 0 and batch > 0,
+          f"M, N, K must be positive multiples of 128, got M={M} N={N} K={K}")
+    A, B = _k_contig(A), _k_contig(B)
+    C = torch.empty((batch, M, N), dtype=torch.int32, device=A.device)
+    _lib.call("ti8_gemm_i8_nt_i32", A.data_ptr(), A.stride(0), A.stride(1),
+              B.data_ptr(), B.stride(0) if B.dim() == 3 else 0, B.stride(-2),
+              C.data_ptr(), C.stride(0), C.stride(1), batch, M, N, K, _stream())
+    return C
