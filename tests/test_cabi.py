@@ -1,0 +1,98 @@
+"""The C ABI library loads without a GPU, exports every symbol include/ti8.h declares,
+and rejects bad arguments on the host (status code + message) before launching anything."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from conftest import ROOT
+
+HEADER = os.path.join(ROOT, "include", "ti8.h")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    import triton_int8_amd
+    return triton_int8_amd._lib.lib()
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ti8_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported(lib):
+    names = declared_functions()
+    assert {"ti8_quant_block", "ti8_quant_row", "ti8_quant_col_t", "ti8_fwht", "ti8_gemm_i8_nt",
+            "ti8_gemm_i8_nt_i32", "ti8_version", "ti8_last_error", "ti8_arch"} <= set(names)
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in ti8.h but not exported by libti8.so"
+    import triton_int8_amd
+    assert sorted(triton_int8_amd._lib.EXPORTS) == names       # the binding covers the whole header
+
+
+def test_version_and_arch(lib):
+    assert lib.ti8_version() >= 100
+    assert lib.ti8_arch() == b"gfx950"
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    import triton_int8_amd
+    L = triton_int8_amd._lib
+    monkeypatch.setattr(L, "_lib", None)
+    monkeypatch.setattr(L, "LIB_PATH", "/nonexistent/libti8.so")
+    with pytest.raises(ImportError, match="no fallback"):
+        L.lib()
+
+
+FAKE = 0x10000  # a 16-byte aligned non-null "device pointer"; validation never dereferences it
+
+
+@pytest.mark.parametrize("call,code,msg", [
+    (("ti8_quant_block", None, 0, 128, FAKE, 0, 128, None, 0, 0, FAKE, 0, 1, 1, 1, 128, 128, 128, 0, 0, None), 1, "required"),
+    (("ti8_quant_block", FAKE, 0, 128, FAKE, 0, 128, None, 0, 0, FAKE, 0, 1, 1, 1, 100, 128, 128, 0, 0, None), 2, "R%128"),
+    (("ti8_quant_block", FAKE, 0, 128, FAKE, 0, 128, None, 0, 0, FAKE, 0, 1, 1, 1, 128, 128, 64, 0, 0, None), 4, "group_c"),
+    (("ti8_quant_block", FAKE, 0, 128, FAKE, 0, 128, FAKE, 0, 128, FAKE, 0, 1, 1, 1, 128, 256, 256, 0, 0, None), 4, "transposed"),
+    (("ti8_quant_block", FAKE + 2, 0, 128, FAKE, 0, 128, None, 0, 0, FAKE, 0, 1, 1, 1, 128, 128, 128, 0, 0, None), 3, "aligned"),
+    (("ti8_quant_block", FAKE, 0, 128, FAKE, 0, 128, None, 0, 0, FAKE, 0, 1, 1, 1, 128, 128, 128, 64, 0, None), 4, "flag"),
+    (("ti8_quant_row", FAKE, 4096, FAKE, 4096, FAKE, 4, 65536, 0, 0, 0, None), 2, "cols<=32768"),
+    (("ti8_quant_row", FAKE, 4096, FAKE, 4096, FAKE, 4, 4096, 64, 0, 0, None), 4, "group"),
+    (("ti8_quant_row", FAKE, 4096, FAKE, 4096, FAKE, 4, 4096, 0, 0, 7, None), 4, "inv_mode"),
+    (("ti8_quant_col_t", FAKE, 256, FAKE, 128, FAKE, None, 128, 256, 0, 0, None), 1, "required"),
+    (("ti8_quant_col_t", FAKE, 256, FAKE, 128, FAKE, FAKE, 100, 256, 0, 0, None), 2, "R%128"),
+    (("ti8_fwht", FAKE, 384, FAKE, 384, 4, 384, 384, 1.0, None), 2, "power of two"),
+    (("ti8_fwht", FAKE, 256, FAKE, 256, 4, 256, 64, 1.0, None), 2, "power of two"),
+    (("ti8_gemm_i8_nt", FAKE, 0, 128, FAKE, 0, 128, FAKE, 0, 128, FAKE, 0, 0, 1, 0, FAKE, 0, 0, 1, 0,
+      1, 128, 128, 100, 0, 0, 1.0, 0.0, 0, None), 2, "multiples of 128"),
+    (("ti8_gemm_i8_nt", FAKE, 0, 128, FAKE, 0, 128, FAKE, 0, 128, None, 0, 0, 1, 0, FAKE, 0, 0, 1, 0,
+      1, 128, 128, 128, 0, 0, 1.0, 0.0, 0, None), 1, "scale pointer"),
+    (("ti8_gemm_i8_nt", FAKE, 0, 128, FAKE, 0, 128, FAKE, 0, 128, FAKE, 1, 0, 1, 1, FAKE, 0, 0, 1, 0,
+      1, 128, 128, 128, 1, 0, 1.0, 0.0, 0, None), 4, "per-row scales"),
+    (("ti8_gemm_i8_nt", FAKE, 0, 128, FAKE, 0, 128, FAKE, 0, 128, FAKE, 0, 0, 1, 0, FAKE, 0, 0, 1, 0,
+      1, 128, 128, 128, 0, 9, 1.0, 0.0, 0, None), 4, "combine"),
+    (("ti8_gemm_i8_nt_i32", FAKE, 0, 64, FAKE, 0, 128, FAKE, 0, 128, 1, 128, 128, 128, None), 2, "leading dimension"),
+])
+def test_argument_validation(lib, call, code, msg):
+    import triton_int8_amd
+    name, args = call[0], call[1:]
+    rc = getattr(lib, name)(*args)
+    assert rc == code, lib.ti8_last_error()
+    assert msg in lib.ti8_last_error().decode()
+    with pytest.raises(triton_int8_amd._lib.Ti8Error):
+        triton_int8_amd._lib.call(name, *args)
+
+
+def test_python_surface_rejects_bad_inputs_without_gpu():
+    import torch
+    import triton_int8_amd as T
+    x = torch.zeros(1, 128, 128, dtype=torch.bfloat16)          # CPU tensor
+    with pytest.raises(ValueError, match="GPU"):
+        T.ops.quant_block(x)
+    with pytest.raises(ValueError):
+        T.linear.linear_forward(x[0], x[0], scheme="nope")
+    with pytest.raises(AssertionError):
+        T.block_channel_fwd32.triton_per_token_quant(torch.zeros(4, 100, dtype=torch.bfloat16))
+    with pytest.raises(ValueError, match="bfloat16"):
+        T.block_channel_fwd32.triton_gemm(None, None, None, None, out_dtype=torch.float16)

@@ -99,7 +99,7 @@ def test_invariants(seed):
     # reconstruction error is at most half a step (plus fp32 rounding of the product)
     sx = s.repeat_interleave(128, 1).repeat_interleave(128, 2)
     err = (x.float() - q.float() * sx).abs()
-    assert bool((err <= sx * 0.5 * (1 + 1e-5) + 1e-12).all())
+    assert bool((err <= sx * (0.5 + 1e-4)).all())  # half a step + fp32 rounding of x*scale, 1/scale
     # a 128x128 block quantisation commutes with transposition
     qt, st = obb.triton_per_block_quant(x.transpose(1, 2))
     assert torch.equal(qt, q.transpose(1, 2)) and torch.equal(st, s.transpose(1, 2))
