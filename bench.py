@@ -1,0 +1,180 @@
+#!/usr/bin/env python3
+"""Benchmark of the INT8 linear layer (forward + backward) on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--scheme block_channel]
+
+One step = one pass of the hot path over one batch of synthetic input resident in HBM:
+Y = X W^T, dX = dY W, dW = dY^T X, every operand quantised to int8 on the way (all
+quantiser launches are inside the timed region).  The workload is BASELINE.json's
+config 2: X 8192x4096 bf16 ~N(0,1) with 1% of the input channels x20, W 4096x4096
+~N(0,0.02), dY 8192x4096 ~N(0,1e-3), seed 1, block-channel scheme.
+
+Prints ONE JSON line.  `value` = 6*M*N*K int8 operations (three GEMMs) divided by the
+mean wall-clock time of a step, in TOPS.  `roofline` describes the dominant kernel (the
+i8 MFMA GEMM): 2*M*N*K operations per launch over its mean launch duration, measured with
+HIP events on the launch stream in a second pass of K steps (so the events do not sit in
+the region `value` is timed on).  `cpu_baseline` is the torch-CPU oracle of the same path
+timed once on the host cores on a bounded sample; it is a reported baseline, not a target.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+METRIC = "INT8 linear fwd+bwd TOPS & % INT8 MFMA peak at 8192x4096x4096"
+INT8_PEAK_TOPS = 5000.0   # MI355X dense int8 MFMA peak, 5.0 POP/s
+HBM_PEAK_GBS = 8000.0     # MI355X HBM3E, 8 TB/s
+M, K, N = 8192, 4096, 4096
+
+
+def make_inputs(m=M, k=K, n=N, seed=1):
+    g = torch.Generator().manual_seed(seed)
+    X = torch.randn(m, k, generator=g)
+    outl = torch.randperm(k, generator=g)[: (k + 99) // 100]
+    X[:, outl] *= 20.0
+    W = torch.randn(n, k, generator=g) * 0.02
+    dY = torch.randn(m, n, generator=g) * 1e-3
+    return X.to(torch.bfloat16), W.to(torch.bfloat16), dY.to(torch.bfloat16)
+
+
+def event_time_ms(fn, reps):
+    """Mean duration of fn() over `reps` launches, HIP events on the current stream."""
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+    for a, b in evs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    return sum(a.elapsed_time(b) for a, b in evs) / reps
+
+
+def cpu_baseline(scheme):
+    """The torch-CPU oracle of the same path on the host cores, bounded sample."""
+    from oracle import linear as olin
+    m, reps = M, 3
+    X, W, dY = make_inputs(m=m)
+    olin.linear_fwd_bwd(X[:512], W, dY[:512], scheme)   # warm the thread pool / sgemm
+    t0 = time.time()
+    for _ in range(reps):
+        olin.linear_fwd_bwd(X, W, dY, scheme)
+    dt = (time.time() - t0) / reps
+    return {"value": round(6.0 * m * N * K / dt / 1e12, 4), "unit": "TOPS", "cores": torch.get_num_threads(),
+            "kind": "port", "host_cpus": os.cpu_count(), "seconds_per_step": round(dt, 2),
+            "sample": f"{reps} full steps of config 2 (fwd+bwd: Y, dX, dW incl. quantisation, {m} tokens x K={K} x N={N}, "
+                      f"same seed and distributions) through the torch-CPU oracle (fp32 sgemm per 128-deep K block, exact)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--scheme", default="block_channel", choices=["block_channel", "row_block", "double_channel"])
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU baseline leg (profiling runs)")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build runs on ONE GPU only (the path has no collectives yet); use --gpus 1")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
+
+    import triton_int8_amd as T
+    from triton_int8_amd import ops
+    from triton_int8_amd._lib import SCALE_BLOCK128, SCALE_ROW
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    X, W, dY = (t.to(dev) for t in make_inputs())
+
+    def step():
+        return T.linear_fwd_bwd(X, W, dY, args.scheme)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    tops = 6.0 * M * N * K / dt / 1e12
+
+    # ---- dominant kernel: the three GEMM launches of a step, timed alone with HIP events
+    if args.scheme == "double_channel":
+        xq, xs = ops.quant_row(X, clamp=True, inv_mode=1)
+        wq, ws = ops.quant_row(W, clamp=True, inv_mode=1)
+        dq, ds = ops.quant_row(dY, clamp=True, inv_mode=1)
+        wtq, wts = ops.quant_col_t(W, clamp=True, inv_mode=1)
+        dtq, dts = ops.quant_col_t(dY, clamp=True, inv_mode=1)
+        xtq, xts = ops.quant_col_t(X, clamp=True, inv_mode=1)
+        gemms = [lambda: ops.gemm_i8_nt(xq[None], wq, xs[None], SCALE_ROW, ws, SCALE_ROW, acc_i32_full=True),
+                 lambda: ops.gemm_i8_nt(dq[None], wtq, ds[None], SCALE_ROW, wts, SCALE_ROW, acc_i32_full=True),
+                 lambda: ops.gemm_i8_nt(dtq[None], xtq, dts[None], SCALE_ROW, xts, SCALE_ROW, acc_i32_full=True)]
+        kernel = "gemm_i8_kernel<256,256,2,2,EPI_ROWS>"
+    else:
+        xq, xqT, xs = ops.quant_block(X[None], clamp=True, with_transpose=True)
+        dq, dqT, ds = ops.quant_block(dY[None], clamp=True, with_transpose=True)
+        if args.scheme == "block_channel":
+            wq, ws = ops.quant_row(W, clamp=True)
+            wtq, wts = ops.quant_col_t(W, clamp=True)
+            gemms = [lambda: ops.gemm_i8_nt(xq, wq, xs, SCALE_BLOCK128, ws, SCALE_ROW),
+                     lambda: ops.gemm_i8_nt(dq, wtq, ds, SCALE_BLOCK128, wts, SCALE_ROW),
+                     lambda: ops.gemm_i8_nt(dqT, xqT, ds.transpose(1, 2), SCALE_BLOCK128, xs.transpose(1, 2), SCALE_BLOCK128)]
+        else:
+            xrq, xrs = ops.quant_row(X, clamp=True)
+            drq, drs = ops.quant_row(dY, clamp=True)
+            wq, wqT, ws = ops.quant_block(W[None], clamp=True, with_transpose=True)
+            dtq, dts = ops.quant_col_t(dY, clamp=True)
+            gemms = [lambda: ops.gemm_i8_nt(xrq[None], wq[0], xrs[None], SCALE_ROW, ws[0], SCALE_BLOCK128),
+                     lambda: ops.gemm_i8_nt(drq[None], wqT[0], drs[None], SCALE_ROW, ws[0].t(), SCALE_BLOCK128),
+                     lambda: ops.gemm_i8_nt(dtq[None], xqT[0], dts[None], SCALE_ROW, xs[0].t(), SCALE_BLOCK128)]
+        kernel = "gemm_i8_kernel<256,128,2,2,EPI_PROMOTE>"
+    for f in gemms:
+        f()
+    gemm_ms = [event_time_ms(f, args.steps) for f in gemms]
+    avg_ms = sum(gemm_ms) / len(gemm_ms)
+    achieved = 2.0 * M * N * K / (avg_ms * 1e-3) / 1e12
+
+    # ---- secondary: the activation quantiser against HBM, and the bf16 GEMM the reference
+    # times beside its int8 path (test.py:34-38)
+    q_ms = event_time_ms(lambda: ops.quant_block(X[None], clamp=True, with_transpose=True), args.steps)
+    q_bytes = 4.0 * M * K  # 2 B read + 1 B int8 + 1 B transposed int8 per element
+    q1_ms = event_time_ms(lambda: ops.quant_block(X[None], clamp=True), args.steps)
+    bf16_fns = (lambda: X @ W.t(), lambda: dY @ W, lambda: dY.t() @ X)
+    for f in bf16_fns:
+        f()
+        f()
+    bf16_ms = sum(event_time_ms(f, args.steps) for f in bf16_fns)
+
+    out = {
+        "metric": METRIC, "value": round(tops, 2), "unit": "TOPS", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+        "config": {"workload": f"config 2: {args.scheme} INT8 linear fwd+bwd (Y, dX, dW + all quantisers), "
+                               f"tokens={M} K={K} N={N}, seed 1, X~N(0,1) 1% channels x20, W~N(0,0.02), dY~N(0,1e-3)",
+                   "scheme": args.scheme, "M": M, "K": K, "N": N},
+        "pct_int8_peak": round(100.0 * tops / INT8_PEAK_TOPS, 2),
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": INT8_PEAK_TOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / INT8_PEAK_TOPS, 4), "traffic": None, "kernel": kernel,
+                     "ops_per_launch": 2 * M * N * K, "launch_ms": [round(t, 4) for t in gemm_ms],
+                     "note": "int8 multiply-adds counted as 2*M*N*K operations per launch; peak is the dense int8 MFMA rate"},
+        "quant_roofline": {"bound": "hbm", "kernel": "quant_block_kernel<1,true,true>",
+                           "achieved": round(q_bytes / (q_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                           "frac": round(q_bytes / (q_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "launch_ms": round(q_ms, 4),
+                           "bytes_per_launch": int(q_bytes),
+                           "single_output_GBs": round(3.0 * M * K / (q1_ms * 1e-3) / 1e9, 1)},
+        "bf16_matmul_ms_per_step": round(bf16_ms, 4),
+        "bf16_matmul_tflops": round(6.0 * M * N * K / (bf16_ms * 1e-3) / 1e12, 1),
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(args.scheme)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()
