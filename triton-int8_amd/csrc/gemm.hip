@@ -14,6 +14,7 @@
 // for both operands, which is all an NT dot product needs); result register r of lane
 // l is C[8*(r/4) + 4*(l/32) + r%4][l % 32] with rows from A and columns from B.
 #include "ti8_common.h"
+#include <type_traits>
 
 namespace ti8 {
 
@@ -36,7 +37,9 @@ struct GemmArgs {
     float out_scale, post_scale;
 };
 
-enum { EPI_I32 = 0, EPI_ROWS = 1, EPI_PROMOTE = 2, EPI_STRICT = 3 };
+enum { EPI_I32 = 0, EPI_ROWS = 1, EPI_PROMOTE = 2, EPI_STRICT = 3, EPI_PROMOTE_DIV = 4 };
+
+__constant__ float k_one = 1.0f;  // stands in for the in-loop factor of an operand scaled per row
 
 
 // scale of operand row `row` at K block kb
@@ -50,17 +53,45 @@ __device__ __forceinline__ float scale_at(const ScaleDesc& d, int64_t batch, int
 }
 
 // One wave's share of a K tile: NI global->LDS instructions of 64 x 16 bytes; instruction i
-// fills the 1 KiB slab at lds + i*1024 (lane l lands at byte 16*l of the slab).
+// fills the 1 KiB slab at lds + i*1024 (lane l lands at byte 16*l of the slab) from
+// base + i*stride8 (wave-uniform: 8 rows further per instruction) + voff[(t0 + i) & 1] (per lane).
 template <int NI>
-__device__ __forceinline__ void issue_tile_loads(const int8_t* const (&gp)[NI], int koff, int8_t* lds) {
+__device__ __forceinline__ void issue_tile_loads(const int8_t* base, int64_t stride8, const uint32_t (&voff)[2], int t0,
+                                                 int8_t* lds) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the builtin only exists in the device pass
 #pragma unroll
-    for (int i = 0; i < NI; ++i) __builtin_amdgcn_global_load_lds(gp[i] + koff, lds + i * 1024, 16, 0, 0);
+    for (int i = 0; i < NI; ++i)
+        __builtin_amdgcn_global_load_lds(base + i * stride8 + voff[(t0 + i) & 1], lds + i * 1024, 16, 0, 0);
 #else
-    (void)gp; (void)koff; (void)lds;
+    (void)base; (void)stride8; (void)voff; (void)t0; (void)lds;
 #endif
 }
 
+// Interleaving hint for one k-step: TM*TN MFMAs, with up to NDS LDS reads, NVM global->LDS
+// loads and NVA*TM*TN VALU ops slotted one group per MFMA so that the matrix pipe never waits
+// behind a burst of memory or vector instructions.
+template <int NMFMA, int NDS, int NVM, int NVA>
+__device__ __forceinline__ void interleave_hint() {
+#if defined(__HIP_DEVICE_COMPILE__)
+#pragma unroll
+    for (int q = 0; q < NMFMA; ++q) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                   // 1 MFMA
+        if (NVA > 0) __builtin_amdgcn_sched_group_barrier(0x002, NVA, 0);    // NVA VALU
+        if (q < NDS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);      // 1 DS read
+        if (q < NVM) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);      // 1 VMEM read
+    }
+#endif
+}
+
+// Software pipeline of the main loop (per workgroup, K tile kt, LDS buffers cur = kt & 1):
+//   k-step 0: MFMA on fragments(kt, 0) | read fragments(kt, 1) | issue B half of tile kt+1
+//   k-step 1: MFMA on fragments(kt, 1) | read fragments(kt, 2)
+//   k-step 2: MFMA on fragments(kt, 2) | read fragments(kt, 3)
+//             wait: own loads of tile kt+1 landed, own LDS reads of buffer cur returned; BARRIER
+//   k-step 3: MFMA on fragments(kt, 3) | read fragments(kt+1, 0) | issue A half of tile kt+2
+//             into buffer cur (every wave is past its last read of it)
+// so there is one barrier per K tile, it sits where the next fragments are already in
+// registers, and a tile's loads have a full K tile of MFMA time to land.
 template <int BM, int BN, int WM, int WN, int EPI>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g) {
     constexpr int NW = WM * WN;
@@ -69,7 +100,10 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
     constexpr int A_INSTR = BM / 8 / NW;  // global->LDS wave instructions per K tile per wave
     constexpr int B_INSTR = BN / 8 / NW;
     constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128;
-    constexpr bool PROMOTE = (EPI == EPI_PROMOTE || EPI == EPI_STRICT);
+    constexpr bool FAST = (EPI == EPI_PROMOTE || EPI == EPI_PROMOTE_DIV);
+    constexpr bool DIV = (EPI == EPI_PROMOTE_DIV);  // acc += d / (sa*sb): multiply by the reciprocal
+    constexpr bool PROMOTE = (FAST || EPI == EPI_STRICT);
+    constexpr int NSET = FAST ? 2 : 1;  // int32 accumulator sets (two: promote one while filling the other)
     static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "tile/wave mismatch");
 
     extern __shared__ __attribute__((aligned(1024))) int8_t smem[];
@@ -78,7 +112,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
     int8_t* const ldsB = smem + 2 * A_BYTES;
 
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: keep it in an SGPR
     const int wm = wave / WN, wn = wave % WN;
 
     // ---- tile assignment: XCD-aware remap, then groups of 8 tile rows -----------------
@@ -99,124 +133,226 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
     const int8_t* Bb = g.B + (int64_t)batch * g.bsb;
 
     // ---- global -> LDS mapping --------------------------------------------------------
-    // wave instruction t covers tile rows 8t..8t+7; lane l writes LDS chunk l of that 1 KiB
-    // slab = (row 8t + l/8, physical chunk l%8), which holds logical chunk (l%8) ^ (l/8).
+    // wave instruction t covers tile rows 8t..8t+7; lane l lands at byte 16*l of that 1 KiB
+    // slab = (row 8t + l/8, physical chunk l%8).  Physical chunk p of row r holds logical
+    // chunk p ^ (r & 7) ^ ((r >> 3) & 1): the 16 rows a quarter-wave reads at one k offset
+    // then sit in 16 distinct 16-byte bank groups.
+    // Address = (uniform row base of the instruction, SGPRs) + (per-lane 32-bit offset, one
+    // VGPR per parity of t): keeps the loop's address registers to four VGPRs.
     const int ld_row = lane >> 3;
-    const int ld_chunk = (lane & 7) ^ ld_row;
-    const int8_t* gA[A_INSTR];
-    const int8_t* gB[B_INSTR];
+    uint32_t voffA[2], voffB[2];
 #pragma unroll
-    for (int i = 0; i < A_INSTR; ++i) {
-        const int r = min(m0 + (wave * A_INSTR + i) * 8 + ld_row, g.M - 1);
-        gA[i] = Ab + (int64_t)r * g.lda + ld_chunk * 16;
+    for (int p = 0; p < 2; ++p) {
+        const int ch = (lane & 7) ^ ld_row ^ p;
+        voffA[p] = (uint32_t)(ld_row * (int)g.lda + ch * 16);
+        voffB[p] = (uint32_t)(ld_row * (int)g.ldb + ch * 16);
     }
-#pragma unroll
-    for (int i = 0; i < B_INSTR; ++i) {
-        const int r = min(n0 + (wave * B_INSTR + i) * 8 + ld_row, g.N - 1);
-        gB[i] = Bb + (int64_t)r * g.ldb + ld_chunk * 16;
-    }
+    // a wave's instructions cover A_INSTR*8 consecutive tile rows (a divisor of 128): if they
+    // start past M (a multiple of 128) they re-read the valid half; those results are masked
+    static_assert(128 % (A_INSTR * 8) == 0 && 128 % (B_INSTR * 8) == 0, "a wave's rows must not straddle a 128-row boundary");
+    int rA0 = m0 + wave * A_INSTR * 8, rB0 = n0 + wave * B_INSTR * 8;
+    if (rA0 >= g.M) rA0 -= 128;
+    if (rB0 >= g.N) rB0 -= 128;
+    const int8_t* const baseA = Ab + (int64_t)rA0 * g.lda;  // wave-uniform
+    const int8_t* const baseB = Bb + (int64_t)rB0 * g.ldb;
+    const int64_t strideA8 = 8 * g.lda, strideB8 = 8 * g.ldb;
+    int8_t* const wA = ldsA + wave * A_INSTR * 1024;  // this wave's share of the A buffer
+    int8_t* const wB = ldsB + wave * B_INSTR * 1024;
 
     // ---- LDS -> register mapping ------------------------------------------------------
     const int fr_row = lane & 31;
     const int fr_half = lane >> 5;
-    const int sw = lane & 7;  // row & 7 (every block starts on a multiple of 8 rows)
+    const int sw = (lane & 7) ^ ((lane >> 3) & 1);
     const int a_row_off = (wm * TM * 32 + fr_row) * 128;
     const int b_row_off = (wn * TN * 32 + fr_row) * 128;
+    int choff[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) choff[ks] = ((ks * 2 + fr_half) ^ sw) * 16;
 
-    v16i acc[TM][TN];
+    v16i acc[NSET][TM][TN];
     float accf[PROMOTE ? TM : 1][PROMOTE ? TN : 1][16];
+    const v16i vzero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+    for (int s = 0; s < NSET; ++s)
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
-            if (PROMOTE) {
+            for (int j = 0; j < TN; ++j) acc[s][i][j] = vzero;
+    if (PROMOTE) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) accf[i][j][r] = 0.0f;
-            }
+    }
+
+    // per-K-tile scale factors of the fast promotion: fa per 32-row block (wave-uniform),
+    // fb per lane (its column).  Operands with per-row scales contribute in the epilogue.
+    // In-loop factor of K tile kt = pfa[i][(kt >> sha) * ksa] * pfb[j][(kt >> shb) * ksb]; an
+    // operand scaled per row reads the constant 1 with stride 0, so the loop has no branches.
+    const float* pfa[TM];
+    const float* pfb[TN];
+    int ksa = 0, ksb = 0, sha = 0, shb = 0;
+    if (FAST) {
+        const bool a_in = g.sa.mode != TI8_SCALE_ROW, b_in = g.sb.mode != TI8_SCALE_ROW;
+        ksa = a_in ? (int)g.sa.ks : 0;
+        ksb = b_in ? (int)g.sb.ks : 0;
+        sha = g.sa.mode == TI8_SCALE_BLOCK_K256 ? 1 : 0;
+        shb = g.sb.mode == TI8_SCALE_BLOCK_K256 ? 1 : 0;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const int row = min(m0 + (wm * TM + i) * 32, g.M - 1);
+            pfa[i] = a_in ? g.sa.p + batch * g.sa.bs + (int64_t)(g.sa.mode == TI8_SCALE_ROW_K128 ? row : row >> 7) * g.sa.rs : &k_one;
         }
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int col = min(n0 + (wn * TN + j) * 32 + fr_row, g.N - 1);
+            pfb[j] = b_in ? g.sb.p + batch * g.sb.bs + (int64_t)(g.sb.mode == TI8_SCALE_ROW_K128 ? col : col >> 7) * g.sb.rs : &k_one;
+        }
+    }
+    float fa[TM], fb[TN];      // factors of the K tile being promoted
+    float fa_n[TM], fb_n[TN];  // factors of the K tile being accumulated (loaded one tile ahead)
+#pragma unroll
+    for (int i = 0; i < TM; ++i) fa[i] = fa_n[i] = 1.0f;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) fb[j] = fb_n[j] = 1.0f;
+    auto load_factors = [&](int kt) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa_n[i] = pfa[i][(kt >> sha) * ksa];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb_n[j] = pfb[j][(kt >> shb) * ksb];
+    };
+    auto rotate_factors = [&]() {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[i] = fa_n[i];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb[j] = fb_n[j];
+    };
+    // accf += f32(acc[set]) * factor, block row i only (one quarter of the work per k-step)
+    auto promote_row = [&](int set, int i) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            float f = fa[i] * fb[j];
+            if (DIV) f = 1.0f / f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                accf[i][j][r] = __builtin_fmaf(static_cast<float>(acc[set][i][j][r]), f, accf[i][j][r]);
+        }
+    };
+
+    v4i a[2][TM], b[2][TN];
+    auto load_frags = [&](int set, const int8_t* sA, const int8_t* sB, int ks) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) a[set][i] = *reinterpret_cast<const v4i*>(sA + i * 4096 + choff[ks]);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) b[set][j] = *reinterpret_cast<const v4i*>(sB + j * 4096 + choff[ks]);
+    };
+    auto mfmas = [&](int fset, int aset, bool first) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                acc[aset][i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[fset][i], b[fset][j],
+                                                                       first ? vzero : acc[aset][i][j], 0, 0, 0);
+    };
 
     const int nk = g.K >> 7;
-    issue_tile_loads<A_INSTR>(gA, 0, ldsA + wave * A_INSTR * 1024);
-    issue_tile_loads<B_INSTR>(gB, 0, ldsB + wave * B_INSTR * 1024);
-    __builtin_amdgcn_s_waitcnt(0x0f70 & 0);  // vmcnt(0) (all counters to zero)
+    // prologue: tile 0 complete, A half of tile 1 in flight, fragments (0, 0) in registers
+    const int tA0 = wave * A_INSTR, tB0 = wave * B_INSTR;
+    issue_tile_loads<A_INSTR>(baseA, strideA8, voffA, tA0, wA);
+    issue_tile_loads<B_INSTR>(baseB, strideB8, voffB, tB0, wB);
+    __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
+    const int klast = (nk - 1) * 128;  // loads past the last K tile re-read it into a free buffer: no branches in the loop
+    issue_tile_loads<A_INSTR>(baseA + min(128, klast), strideA8, voffA, tA0, wA + A_BYTES);
+    load_frags(0, ldsA + a_row_off, ldsB + b_row_off, 0);
 
-    for (int kt = 0; kt < nk; ++kt) {
-        const int buf = kt & 1;
-        if (kt + 1 < nk) {
-            issue_tile_loads<A_INSTR>(gA, (kt + 1) * 128, ldsA + (buf ^ 1) * A_BYTES + wave * A_INSTR * 1024);
-            issue_tile_loads<B_INSTR>(gB, (kt + 1) * 128, ldsB + (buf ^ 1) * B_BYTES + wave * B_INSTR * 1024);
-        }
-
-        const int8_t* sA = ldsA + buf * A_BYTES + a_row_off;
-        const int8_t* sB = ldsB + buf * B_BYTES + b_row_off;
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-            const int choff = ((ks * 2 + fr_half) ^ sw) * 16;
-            v4i a[TM], b[TN];
-#pragma unroll
-            for (int i = 0; i < TM; ++i) a[i] = *reinterpret_cast<const v4i*>(sA + i * 32 * 128 + choff);
-#pragma unroll
-            for (int j = 0; j < TN; ++j) b[j] = *reinterpret_cast<const v4i*>(sB + j * 32 * 128 + choff);
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[j], acc[i][j], 0, 0, 0);
-        }
-
-        if (EPI == EPI_PROMOTE) {
-            // in-loop factor: scalar per 128-row block of A (unless A is per-row) times the
-            // per-column value of B (unless B is per-row); per-row parts wait for the epilogue
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                const int mrow = min(m0 + (wm * TM + i) * 32, g.M - 1);
-                const float fa = (g.sa.mode == TI8_SCALE_ROW) ? 1.0f : scale_at(g.sa, batch, mrow, kt);
-#pragma unroll
-                for (int j = 0; j < TN; ++j) {
-                    const int ncol = min(n0 + (wn * TN + j) * 32 + fr_row, g.N - 1);
-                    const float fb = (g.sb.mode == TI8_SCALE_ROW) ? 1.0f : scale_at(g.sb, batch, ncol, kt);
-                    float f = fa * fb;
-                    if (g.combine == TI8_COMBINE_DIV_PROD) f = 1.0f / f;
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        accf[i][j][r] = __builtin_fmaf(static_cast<float>(acc[i][j][r]), f, accf[i][j][r]);
-                        acc[i][j][r] = 0;
-                    }
-                }
-            }
-        } else if (EPI == EPI_STRICT) {
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j) {
-                    const int ncol = min(n0 + (wn * TN + j) * 32 + fr_row, g.N - 1);
-                    const float sb = scale_at(g.sb, batch, ncol, kt);
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int mrow = min(m0 + (wm * TM + i) * 32 + 8 * (r >> 2) + 4 * fr_half + (r & 3), g.M - 1);
-                        const float sa = scale_at(g.sa, batch, mrow, kt);
-                        const float d = static_cast<float>(acc[i][j][r]);
-                        float t;
-                        if (g.combine == TI8_COMBINE_MUL_MUL) {
-                            t = d * sa;
-                            t = t * sb;
-                        } else if (g.combine == TI8_COMBINE_MUL_PROD) {
-                            t = d * (sa * sb);
-                        } else {
-                            t = d / (sa * sb);
-                        }
-                        accf[i][j][r] = accf[i][j][r] + t;  // separate rounding: contraction is off
-                        acc[i][j][r] = 0;
-                    }
-                }
-        }
-
-        __builtin_amdgcn_s_waitcnt(0);
+    // one K tile; SET = int32 accumulator set it fills, PREV = promote the other set meanwhile
+    auto ktile = [&](int kt, auto set_c, auto prev_c) {
+        constexpr int SET = decltype(set_c)::value;
+        constexpr bool PREV = decltype(prev_c)::value;
+        constexpr int NVA = PREV ? 32 / TM : 0;  // VALU ops per MFMA slot: 2 per element, TN*16 elements per k-step
+        const int cur = kt & 1;
+        const int8_t* sA = ldsA + cur * A_BYTES + a_row_off;
+        const int8_t* sB = ldsB + cur * B_BYTES + b_row_off;
+        if (FAST) load_factors(kt);  // consumed one K tile later; they land before this tile's barrier
+        // k-step 0
+        issue_tile_loads<B_INSTR>(baseB + min((kt + 1) * 128, klast), strideB8, voffB, tB0, wB + (cur ^ 1) * B_BYTES);
+        load_frags(1, sA, sB, 1);
+        mfmas(0, SET, FAST);
+        if (PREV) promote_row(SET ^ (NSET - 1), 0);
+        interleave_hint<TM * TN, TM + TN, B_INSTR, NVA>();
+        // k-step 1
+        load_frags(0, sA, sB, 2);
+        mfmas(1, SET, false);
+        if (PREV && TM > 1) promote_row(SET ^ (NSET - 1), 1 % TM);
+        interleave_hint<TM * TN, TM + TN, 0, NVA>();
+        // k-step 2
+        load_frags(1, sA, sB, 3);
+        mfmas(0, SET, false);
+        if (PREV && TM > 2) promote_row(SET ^ (NSET - 1), 2 % TM);
+        interleave_hint<TM * TN, TM + TN, 0, NVA>();
+        __builtin_amdgcn_s_waitcnt(0);  // tile kt+1 landed; every read of buffer `cur` returned
         __syncthreads();
+        // k-step 3
+        issue_tile_loads<A_INSTR>(baseA + min((kt + 2) * 128, klast), strideA8, voffA, tA0, wA + cur * A_BYTES);
+        load_frags(0, ldsA + (cur ^ 1) * A_BYTES + a_row_off, ldsB + (cur ^ 1) * B_BYTES + b_row_off, 0);
+        mfmas(1, SET, false);
+        if (PREV && TM > 3) promote_row(SET ^ (NSET - 1), 3 % TM);
+        interleave_hint<TM * TN, TM + TN, A_INSTR, NVA>();
+        if (FAST) rotate_factors();
+    };
+    using std::integral_constant;
+    if (FAST) {
+        static_assert(!FAST || TM == 4, "the fast promotion spreads its four block rows over the four k-steps");
+        // two K tiles per trip so that the accumulator set is a compile-time index
+        ktile(0, integral_constant<int, 0>{}, integral_constant<bool, false>{});
+        int kt = 1;
+        for (; kt + 1 < nk; kt += 2) {
+            ktile(kt, integral_constant<int, NSET - 1>{}, integral_constant<bool, true>{});   // fills set 1, promotes set 0
+            ktile(kt + 1, integral_constant<int, 0>{}, integral_constant<bool, true>{});      // fills set 0, promotes set 1
+        }
+        if (kt < nk) {  // odd tail: one more tile into set 1, then drain it
+            ktile(kt, integral_constant<int, NSET - 1>{}, integral_constant<bool, true>{});
+#pragma unroll
+            for (int i = 0; i < TM; ++i) promote_row(NSET - 1, i);
+        } else {
+#pragma unroll
+            for (int i = 0; i < TM; ++i) promote_row(0, i);
+        }
+    } else {
+        for (int kt = 0; kt < nk; ++kt) {
+            ktile(kt, integral_constant<int, 0>{}, integral_constant<bool, false>{});
+            if (EPI == EPI_STRICT) {
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) {
+                        const float sb = scale_at(g.sb, batch, min(n0 + (wn * TN + j) * 32 + fr_row, g.N - 1), kt);
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) {
+                            const int mrow = min(m0 + (wm * TM + i) * 32 + 8 * (r >> 2) + 4 * fr_half + (r & 3), g.M - 1);
+                            const float sa = scale_at(g.sa, batch, mrow, kt);
+                            const float d = static_cast<float>(acc[0][i][j][r]);
+                            float t;
+                            if (g.combine == TI8_COMBINE_MUL_MUL) {
+                                t = d * sa;
+                                t = t * sb;
+                            } else if (g.combine == TI8_COMBINE_MUL_PROD) {
+                                t = d * (sa * sb);
+                            } else {
+                                t = d / (sa * sb);
+                            }
+                            accf[i][j][r] = accf[i][j][r] + t;  // separate rounding: contraction is off
+                            acc[0][i][j][r] = 0;
+                        }
+                    }
+            }
+        }
     }
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
 
     // ---- epilogue ---------------------------------------------------------------------
     // Each wave moves its accumulators through a private 16 KiB LDS slab, 32 tile rows at
@@ -232,11 +368,11 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
     const int rb_row = lane / LPR;
     const int ncol0 = n0 + wn * WCOLS + rb_col;          // first of this lane's 4 columns
     float coln[4] = {1.0f, 1.0f, 1.0f, 1.0f};
-    if (EPI == EPI_ROWS || (EPI == EPI_PROMOTE && g.sb.mode == TI8_SCALE_ROW)) {
+    if (EPI == EPI_ROWS || (FAST && g.sb.mode == TI8_SCALE_ROW)) {
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             coln[c] = scale_at(g.sb, batch, min(ncol0 + c, g.N - 1), 0);
-            if (EPI == EPI_PROMOTE && g.combine == TI8_COMBINE_DIV_PROD) coln[c] = 1.0f / coln[c];
+            if (DIV) coln[c] = 1.0f / coln[c];
         }
     }
 #pragma unroll
@@ -247,7 +383,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
             for (int r = 0; r < 16; ++r) {
                 const int rr = 8 * (r >> 2) + 4 * fr_half + (r & 3);
                 const uint32_t bits = PROMOTE ? __float_as_uint(accf[PROMOTE ? i : 0][PROMOTE ? j : 0][r])
-                                              : static_cast<uint32_t>(acc[i][j][r]);
+                                              : static_cast<uint32_t>(acc[0][i][j][r]);
                 slab[rr * WCOLS + j * 32 + fr_row] = bits;
             }
         // same wave reads what it wrote: an LDS counter wait is enough, no barrier
@@ -276,16 +412,16 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
                 }
             } else {
                 float rowm = 1.0f;
-                const bool row_part = (EPI == EPI_PROMOTE && g.sa.mode == TI8_SCALE_ROW);
+                const bool row_part = (FAST && g.sa.mode == TI8_SCALE_ROW);
                 if (row_part) {
                     rowm = scale_at(g.sa, batch, m, 0);
-                    if (g.combine == TI8_COMBINE_DIV_PROD) rowm = 1.0f / rowm;
+                    if (DIV) rowm = 1.0f / rowm;
                 }
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
                     float v = __uint_as_float(wb[c]);
                     if (row_part) v = v * rowm;
-                    if (EPI == EPI_PROMOTE && g.sb.mode == TI8_SCALE_ROW) v = v * coln[c];
+                    if (FAST && g.sb.mode == TI8_SCALE_ROW) v = v * coln[c];
                     if (g.out_scale != 1.0f) v = v * g.out_scale;
                     t[c] = v;
                 }
@@ -371,9 +507,10 @@ extern "C" int ti8_gemm_i8_nt(const int8_t* A, int64_t bsa, int64_t lda, const i
     a.strict = (gemm_flags & TI8_GEMM_STRICT) ? 1 : 0;
     a.out_scale = out_scale; a.post_scale = post_scale;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (acc_i32_full) return launch<256, 256, 2, 2, EPI_ROWS>(a, batch, st);
+    if (acc_i32_full) return launch<256, 256, 2, 4, EPI_ROWS>(a, batch, st);
     const bool a_loop_per_row = (modeA == TI8_SCALE_ROW_K128);  // would need a per-register factor
     if (a.strict || a_loop_per_row) return launch<128, 128, 2, 2, EPI_STRICT>(a, batch, st);
+    if (combine == TI8_COMBINE_DIV_PROD) return launch<256, 128, 2, 2, EPI_PROMOTE_DIV>(a, batch, st);
     return launch<256, 128, 2, 2, EPI_PROMOTE>(a, batch, st);
 }
 
@@ -390,5 +527,5 @@ extern "C" int ti8_gemm_i8_nt_i32(const int8_t* A, int64_t bsa, int64_t lda, con
     a.M = (int)M; a.N = (int)N; a.K = (int)K;
     a.tiles_m = a.tiles_n = 0;
     a.combine = 0; a.strict = 0; a.out_scale = 1.0f; a.post_scale = 0.0f;
-    return launch<256, 256, 2, 2, EPI_I32>(a, batch, static_cast<hipStream_t>(stream));
+    return launch<256, 256, 2, 4, EPI_I32>(a, batch, static_cast<hipStream_t>(stream));
 }
