@@ -37,9 +37,9 @@ struct GemmArgs {
     float out_scale, post_scale;
 };
 
-enum { EPI_I32 = 0, EPI_ROWS = 1, EPI_PROMOTE = 2, EPI_STRICT = 3, EPI_PROMOTE_DIV = 4 };
-
-__constant__ float k_one = 1.0f;  // stands in for the in-loop factor of an operand scaled per row
+// EPI_PROMOTE: the per-K-tile factor is uniform over a wave's 128 x 64 tile (block or per-row scales
+// on both operands); EPI_PROMOTE_LANE: operand B carries one scale per (column, K tile).
+enum { EPI_I32 = 0, EPI_ROWS = 1, EPI_PROMOTE = 2, EPI_STRICT = 3, EPI_PROMOTE_LANE = 4 };
 
 
 // scale of operand row `row` at K block kb
@@ -100,8 +100,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
     constexpr int A_INSTR = BM / 8 / NW;  // global->LDS wave instructions per K tile per wave
     constexpr int B_INSTR = BN / 8 / NW;
     constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128;
-    constexpr bool FAST = (EPI == EPI_PROMOTE || EPI == EPI_PROMOTE_DIV);
-    constexpr bool DIV = (EPI == EPI_PROMOTE_DIV);  // acc += d / (sa*sb): multiply by the reciprocal
+    constexpr bool FAST = (EPI == EPI_PROMOTE || EPI == EPI_PROMOTE_LANE);
+    constexpr bool LANEB = (EPI == EPI_PROMOTE_LANE);
     constexpr bool PROMOTE = (FAST || EPI == EPI_STRICT);
     constexpr int NSET = FAST ? 2 : 1;  // int32 accumulator sets (two: promote one while filling the other)
     static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "tile/wave mismatch");
@@ -187,45 +187,57 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
                 for (int r = 0; r < 16; ++r) accf[i][j][r] = 0.0f;
     }
 
-    // per-K-tile scale factors of the fast promotion: fa per 32-row block (wave-uniform),
-    // fb per lane (its column).  Operands with per-row scales contribute in the epilogue.
-    // In-loop factor of K tile kt = pfa[i][(kt >> sha) * ksa] * pfb[j][(kt >> shb) * ksb]; an
-    // operand scaled per row reads the constant 1 with stride 0, so the loop has no branches.
-    const float* pfa[TM];
-    const float* pfb[TN];
-    int ksa = 0, ksb = 0, sha = 0, shb = 0;
+    // ---- per-K-tile factors of the fast promotion ---------------------------------------
+    // accf += f32(dot_kt) * f_kt with f_kt = fa_kt * fb_kt (or its reciprocal for the fused
+    // kernels' division).  Operands scaled per row contribute 1 here and their row / column
+    // vector in the epilogue.  A wave's tile (128 rows x 64 columns) lies inside one 128 x 128
+    // scale block, so with block scales f_kt is wave-uniform: all nk (<= 256) values are
+    // fetched once before the loop, lane l of fvec[c] holding tile kt = 64 c + l, and the loop
+    // picks them with v_readlane -- no memory instruction for scales inside the loop.
+    const bool divide = FAST && g.combine == TI8_COMBINE_DIV_PROD;
+    const bool a_in = FAST && g.sa.mode != TI8_SCALE_ROW, b_in = FAST && g.sb.mode != TI8_SCALE_ROW;
+    const int sha = g.sa.mode == TI8_SCALE_BLOCK_K256 ? 1 : 0, shb = g.sb.mode == TI8_SCALE_BLOCK_K256 ? 1 : 0;
+    float fvec[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+    const float* pfb[TN];  // LANEB: this lane's column of B's scale grid
     if (FAST) {
-        const bool a_in = g.sa.mode != TI8_SCALE_ROW, b_in = g.sb.mode != TI8_SCALE_ROW;
-        ksa = a_in ? (int)g.sa.ks : 0;
-        ksb = b_in ? (int)g.sb.ks : 0;
-        sha = g.sa.mode == TI8_SCALE_BLOCK_K256 ? 1 : 0;
-        shb = g.sb.mode == TI8_SCALE_BLOCK_K256 ? 1 : 0;
+        static_assert(!FAST || (TM == 4 && TN <= 4), "fast promotion assumes a 128-row wave tile inside one scale block");
+        const int rowblk = min(m0 + wm * 128, g.M - 1) >> 7;
+        const float* pa = g.sa.p + batch * g.sa.bs + (int64_t)rowblk * g.sa.rs;
+        const int colblk = min(n0 + wn * TN * 32, g.N - 1) >> 7;
+        const float* pb = g.sb.p + batch * g.sb.bs + (int64_t)colblk * g.sb.rs;
+        const int nkt = g.K >> 7;
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            const int row = min(m0 + (wm * TM + i) * 32, g.M - 1);
-            pfa[i] = a_in ? g.sa.p + batch * g.sa.bs + (int64_t)(g.sa.mode == TI8_SCALE_ROW_K128 ? row : row >> 7) * g.sa.rs : &k_one;
+        for (int c = 0; c < 4; ++c) {
+            const int kt = min(c * 64 + lane, nkt - 1);
+            float f = a_in ? pa[(int64_t)(kt >> sha) * g.sa.ks] : 1.0f;
+            if (!LANEB && b_in) f = f * pb[(int64_t)(kt >> shb) * g.sb.ks];
+            if (!LANEB && divide) f = 1.0f / f;
+            fvec[c] = f;
         }
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
             const int col = min(n0 + (wn * TN + j) * 32 + fr_row, g.N - 1);
-            pfb[j] = b_in ? g.sb.p + batch * g.sb.bs + (int64_t)(g.sb.mode == TI8_SCALE_ROW_K128 ? col : col >> 7) * g.sb.rs : &k_one;
+            pfb[j] = g.sb.p + batch * g.sb.bs + (int64_t)col * g.sb.rs;
         }
     }
-    float fa[TM], fb[TN];      // factors of the K tile being promoted
-    float fa_n[TM], fb_n[TN];  // factors of the K tile being accumulated (loaded one tile ahead)
-#pragma unroll
-    for (int i = 0; i < TM; ++i) fa[i] = fa_n[i] = 1.0f;
+    float f_cur = 1.0f, f_nxt = 1.0f;   // wave-uniform factor of the tile being promoted / accumulated
+    float fb[TN], fb_n[TN];             // LANEB only: per-lane factors
 #pragma unroll
     for (int j = 0; j < TN; ++j) fb[j] = fb_n[j] = 1.0f;
     auto load_factors = [&](int kt) {
+        const int l = kt & 63, c = kt >> 6;
+        const float v0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fvec[0]), l));
+        const float v1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fvec[1]), l));
+        const float v2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fvec[2]), l));
+        const float v3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fvec[3]), l));
+        f_nxt = c == 0 ? v0 : (c == 1 ? v1 : (c == 2 ? v2 : v3));
+        if (LANEB) {
 #pragma unroll
-        for (int i = 0; i < TM; ++i) fa_n[i] = pfa[i][(kt >> sha) * ksa];
-#pragma unroll
-        for (int j = 0; j < TN; ++j) fb_n[j] = pfb[j][(kt >> shb) * ksb];
+            for (int j = 0; j < TN; ++j) fb_n[j] = pfb[j][(int64_t)kt * g.sb.ks];
+        }
     };
     auto rotate_factors = [&]() {
-#pragma unroll
-        for (int i = 0; i < TM; ++i) fa[i] = fa_n[i];
+        f_cur = f_nxt;
 #pragma unroll
         for (int j = 0; j < TN; ++j) fb[j] = fb_n[j];
     };
@@ -233,8 +245,12 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
     auto promote_row = [&](int set, int i) {
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-            float f = fa[i] * fb[j];
-            if (DIV) f = 1.0f / f;
+            float f = f_cur;
+            if (LANEB) {
+                f = f_cur * fb[j];
+                const float rf = 1.0f / f;
+                f = divide ? rf : f;
+            }
 #pragma unroll
             for (int r = 0; r < 16; ++r)
                 accf[i][j][r] = __builtin_fmaf(static_cast<float>(acc[set][i][j][r]), f, accf[i][j][r]);
@@ -372,7 +388,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             coln[c] = scale_at(g.sb, batch, min(ncol0 + c, g.N - 1), 0);
-            if (DIV) coln[c] = 1.0f / coln[c];
+            if (divide) coln[c] = 1.0f / coln[c];
         }
     }
 #pragma unroll
@@ -415,7 +431,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
                 const bool row_part = (FAST && g.sa.mode == TI8_SCALE_ROW);
                 if (row_part) {
                     rowm = scale_at(g.sa, batch, m, 0);
-                    if (DIV) rowm = 1.0f / rowm;
+                    if (divide) rowm = 1.0f / rowm;
                 }
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
@@ -508,9 +524,11 @@ extern "C" int ti8_gemm_i8_nt(const int8_t* A, int64_t bsa, int64_t lda, const i
     a.out_scale = out_scale; a.post_scale = post_scale;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (acc_i32_full) return launch<256, 256, 2, 4, EPI_ROWS>(a, batch, st);
-    const bool a_loop_per_row = (modeA == TI8_SCALE_ROW_K128);  // would need a per-register factor
-    if (a.strict || a_loop_per_row) return launch<128, 128, 2, 2, EPI_STRICT>(a, batch, st);
-    if (combine == TI8_COMBINE_DIV_PROD) return launch<256, 128, 2, 2, EPI_PROMOTE_DIV>(a, batch, st);
+    // the fast promotion keeps at most 256 per-K-tile factors in registers and cannot apply a
+    // factor that varies per row of A inside the loop: those cases take the literal kernel
+    const bool a_loop_per_row = (modeA == TI8_SCALE_ROW_K128);
+    if (a.strict || a_loop_per_row || K > 256 * 128) return launch<128, 128, 2, 2, EPI_STRICT>(a, batch, st);
+    if (modeB == TI8_SCALE_ROW_K128) return launch<256, 128, 2, 2, EPI_PROMOTE_LANE>(a, batch, st);
     return launch<256, 128, 2, 2, EPI_PROMOTE>(a, batch, st);
 }
 
