@@ -15,8 +15,11 @@ SOURCES = ["api.hip", "quant.hip", "fwht.hip", "gemm.hip"]
 # -ffp-contract=off: x*scale+0.5 must round twice (bit-exact quantisation); kernels
 #   that want an fma ask for one explicitly.
 # -packed-fp32-ops disabled: keep hipcc from forming v_pk_*_f32 from scalar float code.
+# -amdgpu-mfma-vgpr-form: MFMA accumulators in ordinary VGPRs, so the block-channel promotion
+#   (convert + fma on every 128-deep partial) reads them without v_accvgpr_read copies.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off",
-         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument",
+         "-mllvm", "-amdgpu-mfma-vgpr-form"]
 
 
 def build(verbose: bool = False) -> str:

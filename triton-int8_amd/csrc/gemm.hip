@@ -14,7 +14,7 @@
 // for both operands, which is all an NT dot product needs); result register r of lane
 // l is C[8*(r/4) + 4*(l/32) + r%4][l % 32] with rows from A and columns from B.
 #include "ti8_common.h"
-#include <type_traits>
+#include <stdlib.h>
 
 namespace ti8 {
 
@@ -103,7 +103,6 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
     constexpr bool FAST = (EPI == EPI_PROMOTE || EPI == EPI_PROMOTE_LANE);
     constexpr bool LANEB = (EPI == EPI_PROMOTE_LANE);
     constexpr bool PROMOTE = (FAST || EPI == EPI_STRICT);
-    constexpr int NSET = FAST ? 2 : 1;  // int32 accumulator sets (two: promote one while filling the other)
     static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "tile/wave mismatch");
 
     extern __shared__ __attribute__((aligned(1024))) int8_t smem[];
@@ -169,15 +168,13 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) choff[ks] = ((ks * 2 + fr_half) ^ sw) * 16;
 
-    v16i acc[NSET][TM][TN];
+    v16i acc[TM][TN];
     float accf[PROMOTE ? TM : 1][PROMOTE ? TN : 1][16];
     const v16i vzero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-    for (int s = 0; s < NSET; ++s)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j) acc[s][i][j] = vzero;
+        for (int j = 0; j < TN; ++j) acc[i][j] = vzero;
     if (PROMOTE) {
 #pragma unroll
         for (int i = 0; i < TM; ++i)
@@ -200,8 +197,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
     float fvec[4] = {1.0f, 1.0f, 1.0f, 1.0f};
     const float* pfb[TN];  // LANEB: this lane's column of B's scale grid
     if (FAST) {
-        static_assert(!FAST || (TM == 4 && TN <= 4), "fast promotion assumes a 128-row wave tile inside one scale block");
-        const int rowblk = min(m0 + wm * 128, g.M - 1) >> 7;
+        static_assert(!FAST || (128 % (TM * 32) == 0 && 128 % (TN * 32) == 0), "a wave tile must lie inside one 128 x 128 scale block");
+        const int rowblk = min(m0 + wm * TM * 32, g.M - 1) >> 7;
         const float* pa = g.sa.p + batch * g.sa.bs + (int64_t)rowblk * g.sa.rs;
         const int colblk = min(n0 + wn * TN * 32, g.N - 1) >> 7;
         const float* pb = g.sb.p + batch * g.sb.bs + (int64_t)colblk * g.sb.rs;
@@ -220,40 +217,20 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
             pfb[j] = g.sb.p + batch * g.sb.bs + (int64_t)col * g.sb.rs;
         }
     }
-    float f_cur = 1.0f, f_nxt = 1.0f;   // wave-uniform factor of the tile being promoted / accumulated
-    float fb[TN], fb_n[TN];             // LANEB only: per-lane factors
+    float f_cur = 1.0f;   // wave-uniform factor of the K tile being accumulated
+    float fb[TN];         // LANEB only: per-lane factors of that tile
 #pragma unroll
-    for (int j = 0; j < TN; ++j) fb[j] = fb_n[j] = 1.0f;
+    for (int j = 0; j < TN; ++j) fb[j] = 1.0f;
     auto load_factors = [&](int kt) {
         const int l = kt & 63, c = kt >> 6;
         const float v0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fvec[0]), l));
         const float v1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fvec[1]), l));
         const float v2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fvec[2]), l));
         const float v3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fvec[3]), l));
-        f_nxt = c == 0 ? v0 : (c == 1 ? v1 : (c == 2 ? v2 : v3));
-        if (LANEB) {
+        f_cur = c == 0 ? v0 : (c == 1 ? v1 : (c == 2 ? v2 : v3));
+        if (LANEB) {  // issued before this tile's loads; consumed after its barrier (which waits for them)
 #pragma unroll
-            for (int j = 0; j < TN; ++j) fb_n[j] = pfb[j][(int64_t)kt * g.sb.ks];
-        }
-    };
-    auto rotate_factors = [&]() {
-        f_cur = f_nxt;
-#pragma unroll
-        for (int j = 0; j < TN; ++j) fb[j] = fb_n[j];
-    };
-    // accf += f32(acc[set]) * factor, block row i only (one quarter of the work per k-step)
-    auto promote_row = [&](int set, int i) {
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            float f = f_cur;
-            if (LANEB) {
-                f = f_cur * fb[j];
-                const float rf = 1.0f / f;
-                f = divide ? rf : f;
-            }
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-                accf[i][j][r] = __builtin_fmaf(static_cast<float>(acc[set][i][j][r]), f, accf[i][j][r]);
+            for (int j = 0; j < TN; ++j) fb[j] = pfb[j][(int64_t)kt * g.sb.ks];
         }
     };
 
@@ -264,13 +241,32 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
 #pragma unroll
         for (int j = 0; j < TN; ++j) b[set][j] = *reinterpret_cast<const v4i*>(sB + j * 4096 + choff[ks]);
     };
-    auto mfmas = [&](int fset, int aset, bool first) {
+    auto mfmas = [&](int fset, bool first) {
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int j = 0; j < TN; ++j)
-                acc[aset][i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[fset][i], b[fset][j],
-                                                                       first ? vzero : acc[aset][i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[fset][i], b[fset][j], first ? vzero : acc[i][j], 0, 0, 0);
+    };
+    // Last k-step of a K tile in the fast promotion: the MFMA that completes a block's 128-deep
+    // dot product writes it to ordinary VGPRs (its accumulator input still comes from the
+    // accumulation registers), where convert + fma can consume it directly; the accumulation
+    // registers restart from zero in the next tile, so nothing is copied or cleared.
+    auto mfmas_promote = [&](int fset) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const v16i d = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[fset][i], b[fset][j], acc[i][j], 0, 0, 0);
+                float f = f_cur;
+                if (LANEB) {
+                    f = f_cur * fb[j];
+                    const float rf = 1.0f / f;
+                    f = divide ? rf : f;
+                }
+#pragma unroll
+                for (int r = 0; r < 16; ++r) accf[i][j][r] = __builtin_fmaf(static_cast<float>(d[r]), f, accf[i][j][r]);
+            }
     };
 
     const int nk = g.K >> 7;
@@ -284,62 +280,40 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
     issue_tile_loads<A_INSTR>(baseA + min(128, klast), strideA8, voffA, tA0, wA + A_BYTES);
     load_frags(0, ldsA + a_row_off, ldsB + b_row_off, 0);
 
-    // one K tile; SET = int32 accumulator set it fills, PREV = promote the other set meanwhile
-    auto ktile = [&](int kt, auto set_c, auto prev_c) {
-        constexpr int SET = decltype(set_c)::value;
-        constexpr bool PREV = decltype(prev_c)::value;
-        constexpr int NVA = PREV ? 32 / TM : 0;  // VALU ops per MFMA slot: 2 per element, TN*16 elements per k-step
+    auto ktile = [&](int kt) {
         const int cur = kt & 1;
         const int8_t* sA = ldsA + cur * A_BYTES + a_row_off;
         const int8_t* sB = ldsB + cur * B_BYTES + b_row_off;
-        if (FAST) load_factors(kt);  // consumed one K tile later; they land before this tile's barrier
+        if (FAST) load_factors(kt);
         // k-step 0
         issue_tile_loads<B_INSTR>(baseB + min((kt + 1) * 128, klast), strideB8, voffB, tB0, wB + (cur ^ 1) * B_BYTES);
         load_frags(1, sA, sB, 1);
-        mfmas(0, SET, FAST);
-        if (PREV) promote_row(SET ^ (NSET - 1), 0);
-        interleave_hint<TM * TN, TM + TN, B_INSTR, NVA>();
+        mfmas(0, FAST);
+        interleave_hint<TM * TN, TM + TN, B_INSTR, 0>();
         // k-step 1
         load_frags(0, sA, sB, 2);
-        mfmas(1, SET, false);
-        if (PREV && TM > 1) promote_row(SET ^ (NSET - 1), 1 % TM);
-        interleave_hint<TM * TN, TM + TN, 0, NVA>();
+        mfmas(1, false);
+        interleave_hint<TM * TN, TM + TN, 0, 0>();
         // k-step 2
         load_frags(1, sA, sB, 3);
-        mfmas(0, SET, false);
-        if (PREV && TM > 2) promote_row(SET ^ (NSET - 1), 2 % TM);
-        interleave_hint<TM * TN, TM + TN, 0, NVA>();
+        mfmas(0, false);
+        interleave_hint<TM * TN, TM + TN, 0, 0>();
         __builtin_amdgcn_s_waitcnt(0);  // tile kt+1 landed; every read of buffer `cur` returned
         __syncthreads();
         // k-step 3
         issue_tile_loads<A_INSTR>(baseA + min((kt + 2) * 128, klast), strideA8, voffA, tA0, wA + cur * A_BYTES);
         load_frags(0, ldsA + (cur ^ 1) * A_BYTES + a_row_off, ldsB + (cur ^ 1) * B_BYTES + b_row_off, 0);
-        mfmas(1, SET, false);
-        if (PREV && TM > 3) promote_row(SET ^ (NSET - 1), 3 % TM);
-        interleave_hint<TM * TN, TM + TN, A_INSTR, NVA>();
-        if (FAST) rotate_factors();
-    };
-    using std::integral_constant;
-    if (FAST) {
-        static_assert(!FAST || TM == 4, "the fast promotion spreads its four block rows over the four k-steps");
-        // two K tiles per trip so that the accumulator set is a compile-time index
-        ktile(0, integral_constant<int, 0>{}, integral_constant<bool, false>{});
-        int kt = 1;
-        for (; kt + 1 < nk; kt += 2) {
-            ktile(kt, integral_constant<int, NSET - 1>{}, integral_constant<bool, true>{});   // fills set 1, promotes set 0
-            ktile(kt + 1, integral_constant<int, 0>{}, integral_constant<bool, true>{});      // fills set 0, promotes set 1
-        }
-        if (kt < nk) {  // odd tail: one more tile into set 1, then drain it
-            ktile(kt, integral_constant<int, NSET - 1>{}, integral_constant<bool, true>{});
-#pragma unroll
-            for (int i = 0; i < TM; ++i) promote_row(NSET - 1, i);
+        if (FAST) {
+            mfmas_promote(1);
+            interleave_hint<TM * TN, TM + TN, A_INSTR, 32>();
         } else {
-#pragma unroll
-            for (int i = 0; i < TM; ++i) promote_row(0, i);
+            mfmas(1, false);
+            interleave_hint<TM * TN, TM + TN, A_INSTR, 0>();
         }
-    } else {
+    };
+    {
         for (int kt = 0; kt < nk; ++kt) {
-            ktile(kt, integral_constant<int, 0>{}, integral_constant<bool, false>{});
+            ktile(kt);
             if (EPI == EPI_STRICT) {
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
@@ -350,7 +324,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
                         for (int r = 0; r < 16; ++r) {
                             const int mrow = min(m0 + (wm * TM + i) * 32 + 8 * (r >> 2) + 4 * fr_half + (r & 3), g.M - 1);
                             const float sa = scale_at(g.sa, batch, mrow, kt);
-                            const float d = static_cast<float>(acc[0][i][j][r]);
+                            const float d = static_cast<float>(acc[i][j][r]);
                             float t;
                             if (g.combine == TI8_COMBINE_MUL_MUL) {
                                 t = d * sa;
@@ -361,7 +335,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
                                 t = d / (sa * sb);
                             }
                             accf[i][j][r] = accf[i][j][r] + t;  // separate rounding: contraction is off
-                            acc[0][i][j][r] = 0;
+                            acc[i][j][r] = 0;
                         }
                     }
             }
@@ -399,7 +373,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
             for (int r = 0; r < 16; ++r) {
                 const int rr = 8 * (r >> 2) + 4 * fr_half + (r & 3);
                 const uint32_t bits = PROMOTE ? __float_as_uint(accf[PROMOTE ? i : 0][PROMOTE ? j : 0][r])
-                                              : static_cast<uint32_t>(acc[0][i][j][r]);
+                                              : static_cast<uint32_t>(acc[i][j][r]);
                 slab[rr * WCOLS + j * 32 + fr_row] = bits;
             }
         // same wave reads what it wrote: an LDS counter wait is enough, no barrier
@@ -528,8 +502,13 @@ extern "C" int ti8_gemm_i8_nt(const int8_t* A, int64_t bsa, int64_t lda, const i
     // factor that varies per row of A inside the loop: those cases take the literal kernel
     const bool a_loop_per_row = (modeA == TI8_SCALE_ROW_K128);
     if (a.strict || a_loop_per_row || K > 256 * 128) return launch<128, 128, 2, 2, EPI_STRICT>(a, batch, st);
-    if (modeB == TI8_SCALE_ROW_K128) return launch<256, 128, 2, 2, EPI_PROMOTE_LANE>(a, batch, st);
-    return launch<256, 128, 2, 2, EPI_PROMOTE>(a, batch, st);
+    if (modeB == TI8_SCALE_ROW_K128) return launch<256, 128, 4, 2, EPI_PROMOTE_LANE>(a, batch, st);
+    static const int cfg = getenv("TI8_PROMOTE_CFG") ? atoi(getenv("TI8_PROMOTE_CFG")) : 0;
+    if (cfg == 1) return launch<256, 128, 2, 2, EPI_PROMOTE>(a, batch, st);
+    if (cfg == 2) return launch<128, 256, 2, 4, EPI_PROMOTE>(a, batch, st);
+    if (cfg == 3) return launch<256, 256, 4, 4, EPI_PROMOTE>(a, batch, st);
+    if (cfg == 4) return launch<128, 128, 2, 2, EPI_PROMOTE>(a, batch, st);
+    return launch<256, 128, 4, 2, EPI_PROMOTE>(a, batch, st);
 }
 
 extern "C" int ti8_gemm_i8_nt_i32(const int8_t* A, int64_t bsa, int64_t lda, const int8_t* B, int64_t bsb, int64_t ldb,
