@@ -115,7 +115,7 @@ def main():
         gemms = [lambda: ops.gemm_i8_nt(xq[None], wq, xs[None], SCALE_ROW, ws, SCALE_ROW, acc_i32_full=True),
                  lambda: ops.gemm_i8_nt(dq[None], wtq, ds[None], SCALE_ROW, wts, SCALE_ROW, acc_i32_full=True),
                  lambda: ops.gemm_i8_nt(dtq[None], xtq, dts[None], SCALE_ROW, xts, SCALE_ROW, acc_i32_full=True)]
-        kernel = "gemm_i8_kernel<256,256,2,2,EPI_ROWS>"
+        kernel = "gemm_i8_kernel<256,256,2,4,EPI_ROWS>"
     else:
         xq, xqT, xs = ops.quant_block(X[None], clamp=True, with_transpose=True)
         dq, dqT, ds = ops.quant_block(dY[None], clamp=True, with_transpose=True)
@@ -133,7 +133,7 @@ def main():
             gemms = [lambda: ops.gemm_i8_nt(xrq[None], wq[0], xrs[None], SCALE_ROW, ws[0], SCALE_BLOCK128),
                      lambda: ops.gemm_i8_nt(drq[None], wqT[0], drs[None], SCALE_ROW, ws[0].t(), SCALE_BLOCK128),
                      lambda: ops.gemm_i8_nt(dtq[None], xqT[0], dts[None], SCALE_ROW, xs[0].t(), SCALE_BLOCK128)]
-        kernel = "gemm_i8_kernel<256,128,2,2,EPI_PROMOTE>"
+        kernel = "gemm_i8_kernel<256,128,4,2,EPI_PROMOTE>"
     for f in gemms:
         f()
     gemm_ms = [event_time_ms(f, args.steps) for f in gemms]
@@ -145,11 +145,19 @@ def main():
     q_ms = event_time_ms(lambda: ops.quant_block(X[None], clamp=True, with_transpose=True), args.steps)
     q_bytes = 4.0 * M * K  # 2 B read + 1 B int8 + 1 B transposed int8 per element
     q1_ms = event_time_ms(lambda: ops.quant_block(X[None], clamp=True), args.steps)
+    # a plain device copy of X (64 MiB read + 64 MiB write): the reachable HBM rate on this box,
+    # and the known-size kernel the rocprofv3 FETCH_SIZE / WRITE_SIZE counters are calibrated on
+    X.clone()
+    copy_ms = event_time_ms(lambda: X.clone(), args.steps)
     bf16_fns = (lambda: X @ W.t(), lambda: dY @ W, lambda: dY.t() @ X)
     for f in bf16_fns:
         f()
         f()
     bf16_ms = sum(event_time_ms(f, args.steps) for f in bf16_fns)
+
+    # HBM-side bytes per GEMM launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled on the device
+    # copy above (profiles/bench_config2_block_channel_hbm_counters.md); measured for this scheme only
+    traffic = 393106918 if args.scheme == "block_channel" else None
 
     out = {
         "metric": METRIC, "value": round(tops, 2), "unit": "TOPS", "n_gpus": 1, "steps": args.steps,
@@ -160,7 +168,7 @@ def main():
                    "scheme": args.scheme, "M": M, "K": K, "N": N},
         "pct_int8_peak": round(100.0 * tops / INT8_PEAK_TOPS, 2),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": INT8_PEAK_TOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / INT8_PEAK_TOPS, 4), "traffic": None, "kernel": kernel,
+                     "frac": round(achieved / INT8_PEAK_TOPS, 4), "traffic": traffic, "kernel": kernel,
                      "ops_per_launch": 2 * M * N * K, "launch_ms": [round(t, 4) for t in gemm_ms],
                      "note": "int8 multiply-adds counted as 2*M*N*K operations per launch; peak is the dense int8 MFMA rate"},
         "quant_roofline": {"bound": "hbm", "kernel": "quant_block_kernel<1,true,true>",
@@ -168,6 +176,7 @@ def main():
                            "frac": round(q_bytes / (q_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "launch_ms": round(q_ms, 4),
                            "bytes_per_launch": int(q_bytes),
                            "single_output_GBs": round(3.0 * M * K / (q1_ms * 1e-3) / 1e9, 1)},
+        "copy_GBs": round(2.0 * X.numel() * 2 / (copy_ms * 1e-3) / 1e9, 1),
         "bf16_matmul_ms_per_step": round(bf16_ms, 4),
         "bf16_matmul_tflops": round(6.0 * M * N * K / (bf16_ms * 1e-3) / 1e12, 1),
     }

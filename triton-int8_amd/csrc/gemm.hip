@@ -14,7 +14,6 @@
 // for both operands, which is all an NT dot product needs); result register r of lane
 // l is C[8*(r/4) + 4*(l/32) + r%4][l % 32] with rows from A and columns from B.
 #include "ti8_common.h"
-#include <stdlib.h>
 
 namespace ti8 {
 
@@ -118,7 +117,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
     const int ntiles = g.tiles_m * g.tiles_n;
     int pid = blockIdx.x;
     if ((ntiles & 7) == 0) pid = (pid & 7) * (ntiles >> 3) + (pid >> 3);  // one contiguous range per XCD
-    constexpr int GROUP = 8;
+    // tile rows per group: the 32 workgroups one XCD runs at a time then cover GROUP x 32/GROUP
+    // tiles, chosen so that the A and B panels they share are about the same size
+    constexpr int GROUP = (BM > BN) ? 4 : 8;
     const int per_group = GROUP * g.tiles_n;
     const int group_id = pid / per_group;
     const int first_m = group_id * GROUP;
@@ -503,11 +504,6 @@ extern "C" int ti8_gemm_i8_nt(const int8_t* A, int64_t bsa, int64_t lda, const i
     const bool a_loop_per_row = (modeA == TI8_SCALE_ROW_K128);
     if (a.strict || a_loop_per_row || K > 256 * 128) return launch<128, 128, 2, 2, EPI_STRICT>(a, batch, st);
     if (modeB == TI8_SCALE_ROW_K128) return launch<256, 128, 4, 2, EPI_PROMOTE_LANE>(a, batch, st);
-    static const int cfg = getenv("TI8_PROMOTE_CFG") ? atoi(getenv("TI8_PROMOTE_CFG")) : 0;
-    if (cfg == 1) return launch<256, 128, 2, 2, EPI_PROMOTE>(a, batch, st);
-    if (cfg == 2) return launch<128, 256, 2, 4, EPI_PROMOTE>(a, batch, st);
-    if (cfg == 3) return launch<256, 256, 4, 4, EPI_PROMOTE>(a, batch, st);
-    if (cfg == 4) return launch<128, 128, 2, 2, EPI_PROMOTE>(a, batch, st);
     return launch<256, 128, 4, 2, EPI_PROMOTE>(a, batch, st);
 }
 
