@@ -95,14 +95,28 @@ def double_channel_nt(a, b, hadamard=None, rcp_mul=False):
     return C
 
 
+def _pad_rows(x, multiple=128):
+    """Zero-pad rows to the 128-row tile: zeros change no absmax, an all-padding block gets
+    the epsilon scale and zero codes, and padded tokens add nothing to dW."""
+    T = x.shape[0]
+    Tp = -(-T // multiple) * multiple
+    if Tp == T:
+        return x
+    out = x.new_zeros((Tp, x.shape[1]))
+    out[:T] = x
+    return out
+
+
 def linear_fwd_bwd(X, W, dY, scheme="block_channel", hadamard=None):
-    """Returns (Y, dX, dW) for X [B,M,K] (or [M,K]), W [N,K], dY like Y."""
+    """Returns (Y, dX, dW) for X [B,M,K] (or [M,K]), W [N,K], dY like Y.  Token counts that
+    are not multiples of 128 are zero-padded (skinny / ragged M) and the outputs cut back."""
     squeeze = X.dim() == 2
     if squeeze:
         X, dY = X[None], dY[None]
     B, M, K = X.shape
     N = W.shape[0]
-    Xf, dYf = X.reshape(B * M, K), dY.reshape(B * M, N)
+    T = B * M
+    Xf, dYf = _pad_rows(X.reshape(T, K)), _pad_rows(dY.reshape(T, N))
     if scheme == "double_channel":
         Y = double_channel_nt(Xf, W, hadamard)
         dX = double_channel_nt(dYf, W.t().contiguous(), hadamard)
@@ -115,7 +129,7 @@ def linear_fwd_bwd(X, W, dY, scheme="block_channel", hadamard=None):
         Y = nt_gemm(Xf, W, ma, mb, hadamard)
         dX = nt_gemm(dYf, W.t().contiguous(), ma, mb, hadamard)
         dW = nt_gemm(dYf.t().contiguous(), Xf.t().contiguous(), mabwd, mbwd, hadamard)
-    Y, dX = Y.reshape(B, M, N), dX.reshape(B, M, K)
+    Y, dX = Y[:T].reshape(B, M, N), dX[:T].reshape(B, M, K)
     if squeeze:
         Y, dX = Y[0], dX[0]
     return Y, dX, dW

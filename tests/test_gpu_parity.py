@@ -214,6 +214,47 @@ def test_autograd_module(T, dev):
     assert rel_err(lin.bias.grad, dy.float().sum((0, 1)).cpu()) <= REL_TOL
 
 
+@pytest.mark.parametrize("tokens", [16, 100, 128, 300])
+def test_skinny_and_ragged_token_counts(T, dev, tokens):
+    """Zero-pad semantics for M that is not a multiple of the 128-row tile (config 5's M = 16)."""
+    g = make_gen(12 + tokens)
+    X, W, dY = randn_bf16(g, tokens, 512), randn_bf16(g, 256, 512, std=0.02), randn_bf16(g, tokens, 256, std=1e-3)
+    for scheme in ("block_channel", "row_block", "double_channel"):
+        got = T.linear_fwd_bwd(X.to(dev), W.to(dev), dY.to(dev), scheme)
+        want = olin.linear_fwd_bwd(X, W, dY, scheme)
+        for a, b in zip(got, want):
+            assert a.shape == b.shape and rel_err(a, b) <= REL_TOL
+            if scheme == "double_channel":
+                assert bits_equal(a, b)
+
+
+def test_decoder_layer_step_matches_bf16_twin(T, dev):
+    """One training step of a (reduced-width) Llama-style layer with every linear in INT8 against its
+    bf16 twin: same loss and gradients up to int8 noise (cosine similarity)."""
+    torch.manual_seed(0)
+    ref = T.decoder.DecoderLayer(512, 4, 1024, int8=False, device=dev)
+    lay = T.decoder.DecoderLayer(512, 4, 1024, int8=True, device=dev)
+    lay.copy_weights_from(ref)
+    x = torch.randn(2, 256, 512, device=dev, dtype=torch.bfloat16)
+    tgt = torch.randn(2, 256, 512, device=dev, dtype=torch.bfloat16)
+    outs = []
+    for m in (ref, lay):
+        xi = x.clone().requires_grad_(True)
+        y = m(xi)
+        loss = (y.float() - tgt.float()).pow(2).mean()
+        loss.backward()
+        outs.append((y.detach(), loss.item(), xi.grad, m.down_proj.weight.grad, m.q_proj.weight.grad))
+    cos = lambda a, b: float(torch.nn.functional.cosine_similarity(a.float().flatten(), b.float().flatten(), dim=0))
+    assert cos(outs[0][0], outs[1][0]) > 0.999
+    assert abs(outs[0][1] - outs[1][1]) / outs[0][1] < 2e-2
+    assert cos(outs[0][2], outs[1][2]) > 0.99          # dL/dx
+    assert cos(outs[0][3], outs[1][3]) > 0.99          # dL/dW of the MLP down projection
+    # the gradient that reaches q_proj through the softmax spans orders of magnitude inside one
+    # 128x128 block, so most of it quantises to zero: int8 noise of the scheme, not of the kernels
+    # (the same layers match the CPU oracle in test_linear_fwd_bwd)
+    assert cos(outs[0][4], outs[1][4]) > 0.3
+
+
 def test_golden_vectors_on_gpu(T, dev):
     z = load("quant_256x256.npz")
     x = bf16(z["x"]).to(dev)

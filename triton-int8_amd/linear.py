@@ -30,7 +30,7 @@ import torch
 from . import ops
 from ._lib import (COMBINE_MUL_MUL, INV_AMAX_DIV_127, INV_RCP_OF_SCALE, SCALE_BLOCK128, SCALE_ROW)
 
-__all__ = ["linear_forward", "linear_backward", "linear_fwd_bwd", "Int8LinearFunction", "Int8Linear", "SCHEMES"]
+__all__ = ["linear_forward", "linear_backward", "linear_fwd_bwd", "pad_tokens", "Int8LinearFunction", "Int8Linear", "SCHEMES"]
 
 SCHEMES = ("block_channel", "row_block", "double_channel")
 
@@ -159,14 +159,32 @@ def linear_backward(dY2, X2, W, scheme="block_channel", hadamard=None, saved=Non
     return dX, dW
 
 
+def pad_tokens(x2, multiple=128):
+    """Zero-pad the token (row) dim of a [T, C] tensor up to a multiple of the 128-row tile.
+    Padding rows are zeros, so no absmax (block, row or column) changes, a block made only of
+    padding quantises to zeros with the epsilon scale, and padded rows add nothing to dW: this
+    is the "zero-pad to the tile, absmax over valid rows only" semantics for skinny / ragged M."""
+    T = x2.shape[0]
+    Tp = -(-T // multiple) * multiple
+    if Tp == T:
+        return x2
+    out = x2.new_zeros((Tp, x2.shape[1]))
+    out[:T] = x2
+    return out
+
+
 def linear_fwd_bwd(X, W, dY, scheme="block_channel", hadamard=None):
-    """One forward + backward of the layer: returns (Y, dX, dW) for X [B,M,K] or [M,K]."""
+    """One forward + backward of the layer: returns (Y, dX, dW) for X [B,M,K] or [M,K].
+    Any number of tokens is accepted (zero-padded to a multiple of 128, see :func:`pad_tokens`);
+    K and N must be multiples of 128."""
     lead = X.shape[:-1]
     K, N = X.shape[-1], W.shape[0]
     X2, dY2 = X.reshape(-1, K), dY.reshape(-1, N)
+    T = X2.shape[0]
+    X2, dY2 = pad_tokens(X2), pad_tokens(dY2)
     Y, saved = linear_forward(X2, W, scheme, hadamard)
     dX, dW = linear_backward(dY2, X2, W, scheme, hadamard, saved)
-    return Y.reshape(*lead, N), dX.reshape(*lead, K), dW
+    return Y[:T].reshape(*lead, N), dX[:T].reshape(*lead, K), dW
 
 
 class Int8LinearFunction(torch.autograd.Function):
@@ -176,10 +194,13 @@ class Int8LinearFunction(torch.autograd.Function):
     def forward(ctx, x, weight, bias, scheme, hadamard):
         K, N = x.shape[-1], weight.shape[0]
         x2 = x.reshape(-1, K)
+        ctx.tokens = x2.shape[0]
+        x2 = pad_tokens(x2)
         y, saved = linear_forward(x2, weight, scheme, hadamard)
         ctx.scheme, ctx.hadamard, ctx.saved_q = scheme, hadamard, saved
         ctx.has_bias = bias is not None
         ctx.save_for_backward(x2, weight)
+        y = y[:ctx.tokens]
         if bias is not None:
             y = y + bias
         return y.reshape(*x.shape[:-1], N)
@@ -188,15 +209,16 @@ class Int8LinearFunction(torch.autograd.Function):
     def backward(ctx, dy):
         x2, weight = ctx.saved_tensors
         N = weight.shape[0]
-        dy2 = dy.reshape(-1, N).contiguous()
+        dy2 = pad_tokens(dy.reshape(-1, N).contiguous())
         dx, dw = linear_backward(dy2, x2, weight, ctx.scheme, ctx.hadamard, ctx.saved_q)
         db = dy2.sum(dim=0).to(dy.dtype) if ctx.has_bias else None
-        return dx.reshape(*dy.shape[:-1], x2.shape[1]), dw, db, None, None
+        return dx[:ctx.tokens].reshape(*dy.shape[:-1], x2.shape[1]), dw, db, None, None
 
 
 class Int8Linear(torch.nn.Module):
     """``torch.nn.Linear`` whose three GEMMs (Y, dX, dW) run through the INT8 path.
-    in_features, out_features and the number of tokens must be multiples of 128."""
+    in_features and out_features must be multiples of 128; any number of tokens works
+    (zero-padded to the 128-row tile)."""
 
     def __init__(self, in_features, out_features, bias=False, scheme="block_channel", hadamard=None,
                  device=None, dtype=torch.bfloat16):
