@@ -40,7 +40,9 @@ enum ti8_status {
 enum ti8_qflags {
     TI8_Q_CLAMP = 1,        /* clamp floor(x*scale+0.5) to [-128,127] before the int8 cast */
     TI8_Q_EPS_ADD = 2,      /* amax + 1e-5 (fused kernels) instead of max(amax, 1e-4) */
-    TI8_Q_SCALE_BF16 = 4    /* round the stored scale through bf16 (TileLang copy) */
+    TI8_Q_SCALE_BF16 = 4,   /* round the stored scale through bf16 (TileLang copy) */
+    TI8_Q_HAD128 = 8        /* ti8_quant_row only: rotate every 128-column group by H_128 (fp32
+                               butterflies, one bf16 rounding) before the absmax */
 };
 
 /* which number is written to the scale tensor */
@@ -98,6 +100,23 @@ int ti8_quant_block(const void* x, int64_t bsx, int64_t ldx,
                     float* s, int64_t ssb, int64_t ssr, int64_t ssc,
                     int64_t B, int64_t R, int64_t C, int group_c,
                     int qflags, int inv_mode, ti8_stream_t stream);
+
+/* ---------------------------------------------------------------------------------
+ * Block quantiser with the block-diagonal 128-point Walsh-Hadamard rotation fused in: what
+ * BASELINE config 4 calls the "fused Hadamard + quantize path".  The reference has no such
+ * kernel (its Hadamard is the external full-length transform called before the quantiser,
+ * triton/double-channle_fwd32.py:299-300); the arithmetic is x' = bf16(FWHT_128(f32(x))) per
+ * group of 128 (butterfly strides 1,2,...,64) followed by per_block_quant_kernel
+ * (triton/block_channel_fwd32.py:160-192) on x'.
+ *   along_rows = 0: groups run along the columns of x, q int8 [B][R][C] (ldq, bsq)
+ *   along_rows = 1: groups run along the rows of x,    q int8 [B][C][R] (TRANSPOSED output:
+ *                   the K-contiguous operand of a GEMM that contracts over the rows)
+ *   s: scale of tile (b, rb, cb) of x at s[b*ssb + rb*ssr + cb*ssc].   R, C multiples of 128. */
+int ti8_quant_block_had128(const void* x, int64_t bsx, int64_t ldx,
+                           int8_t* q, int64_t bsq, int64_t ldq,
+                           float* s, int64_t ssb, int64_t ssr, int64_t ssc,
+                           int64_t B, int64_t R, int64_t C, int along_rows,
+                           int qflags, int inv_mode, ti8_stream_t stream);
 
 /* ---------------------------------------------------------------------------------
  * Per-row absmax quantiser in ONE pass over x: replaces triton_per_token_quant +

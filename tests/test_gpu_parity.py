@@ -116,6 +116,25 @@ def test_fwht(T, dev, n, cols):
         assert bits_equal(T.double_channel_fwd32.hadamard_transform(x.to(dev)), ohad.hadamard_transform(x))
 
 
+def test_fused_hadamard_quantisers(T, dev):
+    """H_128 fused into the quantisers equals the un-fused oracle (rotate, round to bf16, quantise)."""
+    x = planted(20, 2, 256, 384)
+    q, s = T.ops.quant_block_had128(x.to(dev), clamp=True)
+    qo, so = obf.block_quant(ohad.hadamard128(x), True)
+    assert bits_equal(q, qo) and bits_equal(s, so)
+    q, s = T.ops.quant_block_had128(x.to(dev), along_rows=True, clamp=True)
+    qo, so = obf.block_quant(ohad.hadamard128(x, dim=1), True)
+    assert q.shape == (2, 384, 256) and bits_equal(q, qo.transpose(1, 2).contiguous()) and bits_equal(s, so)
+    xr = randn_bf16(make_gen(21), 37, 1024)
+    q, s = T.ops.quant_row(xr.to(dev), clamp=True, hadamard128=True)
+    qo, so = obf.token_quant(ohad.hadamard128(xr), True)
+    assert bits_equal(q, qo) and bits_equal(s, so.flatten())
+    xw = randn_bf16(make_gen(22), 5, 14336)
+    q, s = T.ops.quant_row(xw.to(dev), clamp=True, hadamard128=True)
+    qo, so = obf.token_quant(ohad.hadamard128(xw), True)
+    assert bits_equal(q, qo) and bits_equal(s, so.flatten())
+
+
 def test_int32_accumulators_bit_exact(T, dev):
     g = make_gen(6)
     A = torch.randint(-127, 128, (2, 384, 1024), generator=g, dtype=torch.int8)

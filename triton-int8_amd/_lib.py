@@ -15,6 +15,7 @@ _i64, _int, _f32, _vp = ctypes.c_int64, ctypes.c_int, ctypes.c_float, ctypes.c_v
 PROTOTYPES = {
     "ti8_quant_block": [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _i64,
                         _i64, _i64, _i64, _int, _int, _int, _vp],
+    "ti8_quant_block_had128": [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _int, _vp],
     "ti8_quant_row": [_vp, _i64, _vp, _i64, _vp, _i64, _i64, _int, _int, _int, _vp],
     "ti8_quant_col_t": [_vp, _i64, _vp, _i64, _vp, _vp, _i64, _i64, _int, _int, _vp],
     "ti8_fwht": [_vp, _i64, _vp, _i64, _i64, _i64, _i64, _f32, _vp],
@@ -26,7 +27,7 @@ PROTOTYPES = {
 EXPORTS = ["ti8_version", "ti8_last_error", "ti8_arch"] + list(PROTOTYPES)
 
 # enums of include/ti8.h
-Q_CLAMP, Q_EPS_ADD, Q_SCALE_BF16 = 1, 2, 4
+Q_CLAMP, Q_EPS_ADD, Q_SCALE_BF16, Q_HAD128 = 1, 2, 4, 8
 INV_RCP_OF_SCALE, INV_AMAX_DIV_127, INV_AMAX_MUL_RCP127, INV_MULTIPLIER = 0, 1, 2, 3
 SCALE_ROW, SCALE_BLOCK128, SCALE_ROW_K128, SCALE_BLOCK_K256 = 0, 1, 2, 3
 COMBINE_MUL_MUL, COMBINE_MUL_PROD, COMBINE_DIV_PROD = 0, 1, 2

@@ -61,6 +61,38 @@ __device__ __forceinline__ float absmax8(const uint4& v, float m) {
     return m;
 }
 
+
+// 128-point Walsh-Hadamard transform of a row segment held as 8 consecutive bf16 per lane by 16
+// consecutive lanes (lane%16 = chunk index): butterflies in the fixed order stride 1, 2, 4 (in
+// registers), 8, 16, 32, 64 (lane xor 1, 2, 4, 8), fp32, un-normalised; one rounding to bf16.
+__device__ __forceinline__ uint4 fwht128_bf16(const uint4& v, int lane) {
+    float a[8] = {bf16_lo(v.x), bf16_hi(v.x), bf16_lo(v.y), bf16_hi(v.y), bf16_lo(v.z), bf16_hi(v.z), bf16_lo(v.w), bf16_hi(v.w)};
+#pragma unroll
+    for (int h = 1; h < 8; h <<= 1)
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            if ((e & h) == 0) {
+                const float u = a[e], w = a[e + h];
+                a[e] = u + w;
+                a[e + h] = u - w;
+            }
+#pragma unroll
+    for (int m = 1; m < 16; m <<= 1) {
+        const bool upper = (lane & m) != 0;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float p = __shfl_xor(a[e], m, 64);
+            a[e] = upper ? (p - a[e]) : (a[e] + p);   // (a, b) -> (a + b, a - b), a = the lane with the bit clear
+        }
+    }
+    uint4 o;
+    o.x = f32_to_bf16_bits(a[0]) | (f32_to_bf16_bits(a[1]) << 16);
+    o.y = f32_to_bf16_bits(a[2]) | (f32_to_bf16_bits(a[3]) << 16);
+    o.z = f32_to_bf16_bits(a[4]) | (f32_to_bf16_bits(a[5]) << 16);
+    o.w = f32_to_bf16_bits(a[6]) | (f32_to_bf16_bits(a[7]) << 16);
+    return o;
+}
+
 // max over the 256 threads of a workgroup (4 waves), result in every thread
 __device__ __forceinline__ float block_max_256(float v, float* red4) {
     v = wave_max(v);
@@ -168,12 +200,93 @@ __global__ __launch_bounds__(256) void quant_block_kernel(
     }
 }
 
+
+// ---------------------------------------------------------------------------------
+// Block quantiser with the 128-point Hadamard rotation fused in (one read of x, no bf16
+// intermediate in HBM).  ALONG_ROWS = false: rotate every 128-column row segment of the tile
+// and write q in the orientation of x.  ALONG_ROWS = true: rotate every 128-row column segment;
+// the tile goes through LDS once (16-byte chunks swizzled by row group) so that each thread
+// picks up 8 consecutive ROWS of one column, after which the same code runs on the transposed
+// tile and q comes out transposed, [C][R] -- the K-contiguous operand of a GEMM that contracts
+// over the rows (tokens).
+template <bool ALONG_ROWS>
+__global__ __launch_bounds__(256) void quant_block_had_kernel(
+    const uint16_t* __restrict__ x, int64_t bsx, int64_t ldx, int8_t* __restrict__ q, int64_t bsq, int64_t ldq,
+    float* __restrict__ s, int64_t ssb, int64_t ssr, int64_t ssc, int nrb, int ncb, QMode mode) {
+    __shared__ float red4[4];
+    __shared__ __attribute__((aligned(16))) uint16_t tile[ALONG_ROWS ? 128 * 128 : 8];
+
+    int t = blockIdx.x;
+    const int cb = t % ncb;
+    t /= ncb;
+    const int rb = t % nrb;
+    const int b = t / nrb;
+    const int tid = threadIdx.x;
+    const int cc = tid & 15, rg = tid >> 4;
+
+    const uint16_t* xt = x + b * bsx + (int64_t)rb * 128 * ldx + (int64_t)cb * 128;
+    uint4 v[2][4];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            v[h][j] = *reinterpret_cast<const uint4*>(xt + (int64_t)(h * 64 + rg * 4 + j) * ldx + cc * 8);
+
+    if (ALONG_ROWS) {
+        // tile[row][chunk ^ (row >> 3)]: the 16 lanes that later read one column from 16 different
+        // row groups hit 16 different chunks
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int row = h * 64 + rg * 4 + j;
+                *reinterpret_cast<uint4*>(tile + row * 128 + ((cc ^ (row >> 3)) & 15) * 8) = v[h][j];
+            }
+        __syncthreads();
+        // now this thread is (transposed row = original column h*64 + rg*4 + j, transposed columns = original rows 8cc..8cc+7)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int col = h * 64 + rg * 4 + j;
+                uint32_t e[8];
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    const int row = cc * 8 + k;   // row >> 3 == cc
+                    e[k] = tile[row * 128 + (((col >> 3) ^ cc) & 15) * 8 + (col & 7)];
+                }
+                v[h][j] = make_uint4(e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16));
+            }
+    }
+    const int lane = tid & 63;
+    float amax = 0.0f;
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            v[h][j] = fwht128_bf16(v[h][j], lane);
+            amax = absmax8(v[h][j], amax);
+        }
+    amax = block_max_256(amax, red4);
+    amax = amax_floor(amax, mode.eps_add);
+    const float scale = 127.0f / amax;
+    if (tid == 0) s[b * ssb + rb * ssr + cb * ssc] = stored_scale(amax, scale, mode);
+    // output tile origin: same orientation as x, or transposed
+    int8_t* qt = ALONG_ROWS ? q + b * bsq + (int64_t)cb * 128 * ldq + (int64_t)rb * 128
+                            : q + b * bsq + (int64_t)rb * 128 * ldq + (int64_t)cb * 128;
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            *reinterpret_cast<uint2*>(qt + (int64_t)(h * 64 + rg * 4 + j) * ldq + cc * 8) = quant8(v[h][j], scale, mode.clamp);
+}
+
 // ---------------------------------------------------------------------------------
 // Per-row quantiser, one pass.  WG_ROW = false: one wavefront per row (4 rows per
 // workgroup); WG_ROW = true: one 256-thread workgroup per row.  Each thread keeps
 // NLOAD 16-byte chunks of its row in registers.  GROUP16: one scale per 16 chunks
 // (128 columns) instead of per row.
-template <int NLOAD, bool WG_ROW, bool GROUP16>
+template <int NLOAD, bool WG_ROW, bool GROUP16, bool HAD>
 __global__ __launch_bounds__(256) void quant_row_kernel(const uint16_t* __restrict__ x, int64_t ldx,
                                                         int8_t* __restrict__ q, int64_t ldq,
                                                         float* __restrict__ s, int64_t rows, int cols,
@@ -191,6 +304,8 @@ __global__ __launch_bounds__(256) void quant_row_kernel(const uint16_t* __restri
     for (int i = 0; i < NLOAD; ++i) {
         const int c = t + i * T;
         v[i] = (c < nchunk) ? *reinterpret_cast<const uint4*>(xr + c * 8) : make_uint4(0, 0, 0, 0);
+        // chunks c, c^1, ... c^15 of a 128-column group sit in 16 consecutive lanes (T % 16 == 0)
+        if (HAD) v[i] = fwht128_bf16(v[i], threadIdx.x & 63);
     }
     int8_t* qr = q + row * ldq;
     if (GROUP16) {
@@ -334,7 +449,7 @@ __global__ __launch_bounds__(256) void quant_col_t_kernel(const uint16_t* __rest
 }
 
 static int parse_mode(int qflags, int inv_mode, QMode* m) {
-    if (qflags & ~(TI8_Q_CLAMP | TI8_Q_EPS_ADD | TI8_Q_SCALE_BF16)) return fail(TI8_ERR_MODE, "unknown quantiser flag 0x%x", qflags);
+    if (qflags & ~(TI8_Q_CLAMP | TI8_Q_EPS_ADD | TI8_Q_SCALE_BF16 | TI8_Q_HAD128)) return fail(TI8_ERR_MODE, "unknown quantiser flag 0x%x", qflags);
     if (inv_mode < 0 || inv_mode > 3) return fail(TI8_ERR_MODE, "unknown inv_mode %d", inv_mode);
     m->clamp = (qflags & TI8_Q_CLAMP) ? 1 : 0;
     m->eps_add = (qflags & TI8_Q_EPS_ADD) ? 1 : 0;
@@ -353,6 +468,7 @@ extern "C" int ti8_quant_block(const void* x, int64_t bsx, int64_t ldx, int8_t* 
                                int inv_mode, ti8_stream_t stream) {
     QMode mode;
     if (int e = parse_mode(qflags, inv_mode, &mode)) return e;
+    if (qflags & TI8_Q_HAD128) return fail(TI8_ERR_MODE, "ti8_quant_block: use ti8_quant_block_had128 for the Hadamard rotation");
     if (!x || !s || (!q && !qT)) return fail(TI8_ERR_NULL, "ti8_quant_block: x, s and one of q/qT are required");
     if (group_c != 128 && group_c != 256) return fail(TI8_ERR_MODE, "ti8_quant_block: group_c must be 128 or 256, got %d", group_c);
     if (qT && group_c != 128) return fail(TI8_ERR_MODE, "ti8_quant_block: the transposed output needs group_c = 128");
@@ -396,8 +512,10 @@ extern "C" int ti8_quant_row(const void* x, int64_t ldx, int8_t* q, int64_t ldq,
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     const int nchunk = (int)(cols / 8);
     const int c = (int)cols;
+    const bool had = (qflags & TI8_Q_HAD128) != 0;
 #define TI8_LAUNCH_QR(NL, WG, G16, GRID) \
-    hipLaunchKernelGGL((quant_row_kernel<NL, WG, G16>), dim3((unsigned)(GRID)), dim3(256), 0, st, xp, ldx, q, ldq, s, rows, c, mode)
+    do { if (had) hipLaunchKernelGGL((quant_row_kernel<NL, WG, G16, true>), dim3((unsigned)(GRID)), dim3(256), 0, st, xp, ldx, q, ldq, s, rows, c, mode); \
+         else hipLaunchKernelGGL((quant_row_kernel<NL, WG, G16, false>), dim3((unsigned)(GRID)), dim3(256), 0, st, xp, ldx, q, ldq, s, rows, c, mode); } while (0)
     const int64_t g4 = (rows + 3) / 4;
     if (group == 128) {
         if (nchunk <= 64 * 8) TI8_LAUNCH_QR(8, false, true, g4);
@@ -417,6 +535,7 @@ extern "C" int ti8_quant_col_t(const void* x, int64_t ldx, int8_t* qT, int64_t l
                                int64_t R, int64_t C, int qflags, int inv_mode, ti8_stream_t stream) {
     QMode mode;
     if (int e = parse_mode(qflags, inv_mode, &mode)) return e;
+    if (qflags & TI8_Q_HAD128) return fail(TI8_ERR_MODE, "ti8_quant_col_t: the Hadamard rotation is not offered here");
     if (!x || !qT || !s || !ws) return fail(TI8_ERR_NULL, "ti8_quant_col_t: x, qT, s and ws are required");
     if (R <= 0 || C <= 0 || R % 128 || C % 128 || C > 0x7fffffffLL)
         return fail(TI8_ERR_SHAPE, "ti8_quant_col_t: need R%%128==0 and C%%128==0; got R=%lld C=%lld", (long long)R, (long long)C);
@@ -434,4 +553,26 @@ extern "C" int ti8_quant_col_t(const void* x, int64_t ldx, int8_t* qT, int64_t l
     hipLaunchKernelGGL(quant_col_t_kernel, dim3((unsigned)ntiles), dim3(256), 0, st, xp, ldx, qT, ldqt, s, ws,
                        (int)(C / 128), mode);
     return check_launch("ti8_quant_col_t");
+}
+
+extern "C" int ti8_quant_block_had128(const void* x, int64_t bsx, int64_t ldx, int8_t* q, int64_t bsq, int64_t ldq,
+                                      float* s, int64_t ssb, int64_t ssr, int64_t ssc, int64_t B, int64_t R, int64_t C,
+                                      int along_rows, int qflags, int inv_mode, ti8_stream_t stream) {
+    QMode mode;
+    if (int e = parse_mode(qflags & ~TI8_Q_HAD128, inv_mode, &mode)) return e;
+    if (!x || !q || !s) return fail(TI8_ERR_NULL, "ti8_quant_block_had128: x, q and s are required");
+    if (B <= 0 || R <= 0 || C <= 0 || R % 128 || C % 128)
+        return fail(TI8_ERR_SHAPE, "ti8_quant_block_had128: need B>0, R%%128==0, C%%128==0; got B=%lld R=%lld C=%lld", (long long)B, (long long)R, (long long)C);
+    if (ldx < C || ldq < (along_rows ? R : C)) return fail(TI8_ERR_SHAPE, "ti8_quant_block_had128: leading dimension smaller than the row length");
+    if (!aligned16(x) || !aligned16(q) || (ldx % 8) || (bsx % 8) || (ldq % 16) || (bsq % 16))
+        return fail(TI8_ERR_ALIGN, "ti8_quant_block_had128: pointers must be 16-byte aligned and strides multiples of 16 bytes");
+    const int64_t ntiles = B * (R / 128) * (C / 128);
+    if (ntiles > 0x7fffffffLL) return fail(TI8_ERR_SHAPE, "ti8_quant_block_had128: too many tiles");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uint16_t* xp = static_cast<const uint16_t*>(x);
+    if (along_rows)
+        hipLaunchKernelGGL(quant_block_had_kernel<true>, dim3((unsigned)ntiles), dim3(256), 0, st, xp, bsx, ldx, q, bsq, ldq, s, ssb, ssr, ssc, (int)(R / 128), (int)(C / 128), mode);
+    else
+        hipLaunchKernelGGL(quant_block_had_kernel<false>, dim3((unsigned)ntiles), dim3(256), 0, st, xp, bsx, ldx, q, bsq, ldq, s, ssb, ssr, ssc, (int)(R / 128), (int)(C / 128), mode);
+    return check_launch("ti8_quant_block_had128");
 }

@@ -67,20 +67,19 @@ def linear_forward(X2, W, scheme="block_channel", hadamard=None):
     saved = {}
     if scheme == "block_channel":
         if hadamard == 128:
-            q, s = ops.quant_block(_h128(X2)[None], clamp=True)
-            wq, ws = ops.quant_row(_h128(W), clamp=True)
+            q, s = ops.quant_block_had128(X2[None], clamp=True)
+            wq, ws = ops.quant_row(W, clamp=True, hadamard128=True)
             return _gemm_bc(q[0], s[0], SCALE_BLOCK128, wq, ws, SCALE_ROW, 2.0 ** -7), saved
         q, qT, s = ops.quant_block(X2[None], clamp=True, with_transpose=True)
         saved["XqT"], saved["Xs"] = qT[0], s[0]
         wq, ws = ops.quant_row(W, clamp=True)
         return _gemm_bc(q[0], s[0], SCALE_BLOCK128, wq, ws, SCALE_ROW), saved
     if scheme == "row_block":
-        xs_in, w_in = (_h128(X2), _h128(W)) if hadamard == 128 else (X2, W)
-        q, s = ops.quant_row(xs_in, clamp=True)
+        q, s = ops.quant_row(X2, clamp=True, hadamard128=(hadamard == 128))
         if hadamard == 128:
-            wq, ws = ops.quant_block(w_in[None], clamp=True)
+            wq, ws = ops.quant_block_had128(W[None], clamp=True)
             return _gemm_bc(q, s, SCALE_ROW, wq[0], ws[0], SCALE_BLOCK128, 2.0 ** -7), saved
-        wq, wqT, ws = ops.quant_block(w_in[None], clamp=True, with_transpose=True)
+        wq, wqT, ws = ops.quant_block(W[None], clamp=True, with_transpose=True)
         saved["WqT"], saved["Ws"] = wqT[0], ws[0]
         return _gemm_bc(q, s, SCALE_ROW, wq[0], ws[0], SCALE_BLOCK128), saved
     # double_channel
@@ -103,12 +102,14 @@ def linear_backward(dY2, X2, W, scheme="block_channel", hadamard=None, saved=Non
     if scheme == "block_channel":
         if hadamard == 128:
             # H_128 along N for dX, along the tokens for dW: two differently rotated copies
-            dq, ds = ops.quant_block(_h128(dY2)[None], clamp=True)
-            wtq, wts = ops.quant_row(_h128(W.t().contiguous()), clamp=True)
+            dq, ds = ops.quant_block_had128(dY2[None], clamp=True)
+            wtq, wts = ops.quant_row(W.t().contiguous(), clamp=True, hadamard128=True)   # weights: small
             dX = _gemm_bc(dq[0], ds[0], SCALE_BLOCK128, wtq, wts, SCALE_ROW, 2.0 ** -7)
-            dyt, dyts = ops.quant_block(_h128(dY2.t().contiguous())[None], clamp=False)
-            xt, xts = ops.quant_block(_h128(X2.t().contiguous())[None], clamp=False)
-            dW = ops.gemm_i8_nt(dyt, xt, dyts, SCALE_BLOCK128, xts, SCALE_BLOCK128, out_scale=2.0 ** -7)[0]
+            # the token-dim rotation is fused too: one read of dY / X, transposed int8 out
+            dyt, dyts = ops.quant_block_had128(dY2[None], along_rows=True, clamp=False)
+            xt, xts = ops.quant_block_had128(X2[None], along_rows=True, clamp=False)
+            dW = ops.gemm_i8_nt(dyt, xt, dyts.transpose(1, 2), SCALE_BLOCK128, xts.transpose(1, 2), SCALE_BLOCK128,
+                                out_scale=2.0 ** -7)[0]
             return dX, dW
         dq, dqT, ds = ops.quant_block(dY2[None], clamp=True, with_transpose=True)
         wtq, wts = ops.quant_col_t(W, clamp=True)                    # W^T [K,N] per row
@@ -123,12 +124,12 @@ def linear_backward(dY2, X2, W, scheme="block_channel", hadamard=None, saved=Non
         return dX, dW
     if scheme == "row_block":
         if hadamard == 128:
-            dq, ds = ops.quant_row(_h128(dY2), clamp=True)
-            wtq, wts = ops.quant_block(_h128(W.t().contiguous())[None], clamp=True)
-            dX = _gemm_bc(dq, ds, SCALE_ROW, wtq[0], wts[0], SCALE_BLOCK128, 2.0 ** -7)
-            dytq, dyts = ops.quant_row(_h128(dY2.t().contiguous()), clamp=True)
-            xtq, xts = ops.quant_block(_h128(X2.t().contiguous())[None], clamp=True)
-            dW = _gemm_bc(dytq, dyts, SCALE_ROW, xtq[0], xts[0], SCALE_BLOCK128, 2.0 ** -7)
+            dq, ds = ops.quant_row(dY2, clamp=True, hadamard128=True)
+            wtq, wts = ops.quant_block_had128(W[None], along_rows=True, clamp=True)      # W^T [K,N], groups along N
+            dX = _gemm_bc(dq, ds, SCALE_ROW, wtq[0], wts[0].t(), SCALE_BLOCK128, 2.0 ** -7)
+            dytq, dyts = ops.quant_row(dY2.t().contiguous(), clamp=True, hadamard128=True)
+            xtq, xts = ops.quant_block_had128(X2[None], along_rows=True, clamp=True)
+            dW = _gemm_bc(dytq, dyts, SCALE_ROW, xtq[0], xts[0].t(), SCALE_BLOCK128, 2.0 ** -7)
             return dX, dW
         dq, ds = ops.quant_row(dY2, clamp=True)
         if "WqT" in saved:

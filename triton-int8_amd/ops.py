@@ -9,10 +9,10 @@ import torch
 
 from . import _lib
 from ._lib import (COMBINE_DIV_PROD, COMBINE_MUL_MUL, COMBINE_MUL_PROD, GEMM_STRICT, INV_AMAX_DIV_127,
-                   INV_AMAX_MUL_RCP127, INV_MULTIPLIER, INV_RCP_OF_SCALE, Q_CLAMP, Q_EPS_ADD, Q_SCALE_BF16,
+                   INV_AMAX_MUL_RCP127, INV_MULTIPLIER, INV_RCP_OF_SCALE, Q_CLAMP, Q_EPS_ADD, Q_HAD128, Q_SCALE_BF16,
                    SCALE_BLOCK128, SCALE_BLOCK_K256, SCALE_ROW, SCALE_ROW_K128)
 
-__all__ = ["quant_block", "quant_row", "quant_col_t", "fwht", "gemm_i8_nt", "gemm_i8_nt_i32"]
+__all__ = ["quant_block", "quant_block_had128", "quant_row", "quant_col_t", "fwht", "gemm_i8_nt", "gemm_i8_nt_i32"]
 
 
 def _stream():
@@ -90,9 +90,29 @@ def quant_block(x, *, clamp=True, group_c=128, eps_add=False, scale_bf16=False, 
     return (q, qT, s) if with_transpose else (q, s)
 
 
-def quant_row(x, *, clamp=True, group=0, eps_add=False, scale_bf16=False, inv_mode=INV_RCP_OF_SCALE):
+def quant_block_had128(x, *, along_rows=False, clamp=True, inv_mode=INV_RCP_OF_SCALE):
+    """Block-diagonal H_128 rotation fused with the 128x128 block quantiser, one read of ``x``
+    [B, R, C] (bf16, row-major).  ``along_rows=False``: groups of 128 along the columns,
+    returns ``q`` [B, R, C].  ``along_rows=True``: groups along the rows, returns ``q``
+    TRANSPOSED, [B, C, R].  ``s`` is fp32 [B, R/128, C/128] (tile grid of ``x``) in both cases."""
+    _check_bf16(x, "x")
+    _need(x.dim() == 3, "x must be [B, R, C]")
+    B, R, C = x.shape
+    _need(B > 0 and R % 128 == 0 and C % 128 == 0 and R > 0 and C > 0, f"need R % 128 == 0 and C % 128 == 0, got {R}x{C}")
+    if x.stride(2) != 1 or (B > 1 and x.stride(0) % 8) or x.stride(1) % 8 or x.data_ptr() % 16:
+        x = x.contiguous()
+    q = torch.empty((B, C, R) if along_rows else (B, R, C), dtype=torch.int8, device=x.device)
+    s = torch.empty((B, R // 128, C // 128), dtype=torch.float32, device=x.device)
+    _lib.call("ti8_quant_block_had128", x.data_ptr(), x.stride(0), x.stride(1), q.data_ptr(), R * C, q.shape[2],
+              s.data_ptr(), s.stride(0), s.stride(1), s.stride(2), B, R, C, 1 if along_rows else 0,
+              _qflags(clamp, False, False), inv_mode, _stream())
+    return q, s
+
+
+def quant_row(x, *, clamp=True, group=0, eps_add=False, scale_bf16=False, inv_mode=INV_RCP_OF_SCALE, hadamard128=False):
     """Per-row (``group=0``) or per-(row, 128 columns) absmax quantisation of the last dim.
-    ``x``: bf16 [..., cols].  Returns ``(q, s)`` with ``s`` fp32 [...] or [..., cols/128]."""
+    ``x``: bf16 [..., cols].  Returns ``(q, s)`` with ``s`` fp32 [...] or [..., cols/128].
+    ``hadamard128`` rotates every group of 128 columns by H_128 first (fused, one read)."""
     _check_bf16(x, "x")
     _need(x.dim() >= 1 and x.numel() > 0, "x must be a non-empty tensor")
     cols = x.shape[-1]
@@ -104,7 +124,7 @@ def quant_row(x, *, clamp=True, group=0, eps_add=False, scale_bf16=False, inv_mo
     q = torch.empty((rows, cols), dtype=torch.int8, device=x.device)
     s = torch.empty((rows, cols // 128) if group else (rows,), dtype=torch.float32, device=x.device)
     _lib.call("ti8_quant_row", x2.data_ptr(), x2.stride(0), q.data_ptr(), cols, s.data_ptr(), rows, cols, group,
-              _qflags(clamp, eps_add, scale_bf16), inv_mode, _stream())
+              _qflags(clamp, eps_add, scale_bf16) | (Q_HAD128 if hadamard128 else 0), inv_mode, _stream())
     lead = x.shape[:-1]
     return q.reshape(*lead, cols), s.reshape(*lead, cols // 128) if group else s.reshape(*lead)
 
