@@ -106,8 +106,8 @@ def test_col_quant_transposed(T, dev):
     assert bits_equal(qT, qo) and bits_equal(s, so)
 
 
-@pytest.mark.parametrize("n,cols", [(128, 384), (128, 4096), (1024, 2048), (2048, 2048), (4096, 4096),
-                                    (8192, 8192), (32768, 32768)])
+@pytest.mark.parametrize("n,cols", [(128, 384), (128, 4096), (256, 256), (512, 1536), (1024, 2048), (2048, 2048),
+                                    (4096, 4096), (8192, 8192), (16384, 16384), (32768, 32768)])
 def test_fwht(T, dev, n, cols):
     x = randn_bf16(make_gen(n + cols), 9, cols)
     y = T.ops.fwht(x.to(dev), n)

@@ -2,42 +2,72 @@
 // fp32 butterflies in the fixed order stride 1, 2, 4, ..., n/2.  The order is part of
 // the contract: fp32 sums are order dependent and the CPU checker uses the same one.
 //
-// A workgroup of 256 threads owns L consecutive elements of one row: L = n when
-// n >= 2048, else gcd(cols, 2048) (several length-n groups), staged in LDS as fp32.  The log2(n) stages
-// run in passes of up to 4 stages: in a pass over index bits [p, p+r) a thread gathers
-// the 2^r elements that differ only in those bits, does the butterflies in registers
-// and writes them back.  Compile with -ffp-contract=off (the optional scale multiply
-// must not fuse with a butterfly).
+// A workgroup owns L consecutive elements of one row: L = n when
+// n >= 2048, else gcd(cols, 2048) (several length-n groups).  The log2(n) stages run in
+// passes: in a pass over index bits [p, p+r) a thread gathers the 2^r elements that
+// differ only in those bits, does the butterflies in registers and hands them on through
+// LDS (fp32).  The first pass (bits 0..3) takes its 16 consecutive elements straight from
+// global memory; the passes are bits 0..3, 4..7 and then the remaining bits in one pass
+// (up to 5 bits) or two.
+//
+// LDS index i lives at word i + i/16.  With that padding a wave's 64 accesses of one
+// instruction fall into 64 different banks in every pass: stride 17 in the first pass,
+// four runs of 16 words at offsets 0, 16, 32, 48 (mod 64) in the second, consecutive
+// words afterwards.  Without it the first two passes serialise 16- and 4-fold.
+// Compile with -ffp-contract=off (the optional scale multiply must not fuse with a
+// butterfly).
 #include "ti8_common.h"
 
 namespace ti8 {
 
+__device__ __forceinline__ int padded(int i) { return i + (i >> 4); }
+
 template <int RB>
+__device__ __forceinline__ void butterflies(float (&a)[1 << RB]) {
+    constexpr int RAD = 1 << RB;
+#pragma unroll
+    for (int h = 1; h < RAD; h <<= 1)
+#pragma unroll
+        for (int e = 0; e < RAD; ++e)
+            if ((e & h) == 0) {
+                const float u = a[e], w = a[e + h];
+                a[e] = u + w;
+                a[e + h] = u - w;
+            }
+}
+
+template <int RB, int NT>
 __device__ __forceinline__ void pass_in_lds(float* lds, int L, int p, int tid) {
     constexpr int RAD = 1 << RB;
     const int ngroups = L >> RB;
-    for (int vt = tid; vt < ngroups; vt += 256) {
+    for (int vt = tid; vt < ngroups; vt += NT) {
         const int lo = vt & ((1 << p) - 1);
         const int hi = vt >> p;
         const int base = (hi << (p + RB)) | lo;
         float a[RAD];
 #pragma unroll
-        for (int e = 0; e < RAD; ++e) a[e] = lds[base + (e << p)];
+        for (int e = 0; e < RAD; ++e) a[e] = lds[padded(base + (e << p))];
+        butterflies<RB>(a);
 #pragma unroll
-        for (int h = 1; h < RAD; h <<= 1)
-#pragma unroll
-            for (int e = 0; e < RAD; ++e)
-                if ((e & h) == 0) {
-                    const float u = a[e], w = a[e + h];
-                    a[e] = u + w;
-                    a[e + h] = u - w;
-                }
-#pragma unroll
-        for (int e = 0; e < RAD; ++e) lds[base + (e << p)] = a[e];
+        for (int e = 0; e < RAD; ++e) lds[padded(base + (e << p))] = a[e];
     }
 }
 
-__global__ __launch_bounds__(256) void fwht_kernel(const uint16_t* __restrict__ x, int64_t ldx,
+template <int NT>
+__device__ __forceinline__ void pass_dispatch(float* lds, int L, int p, int rb, int tid) {
+    switch (rb) {
+        case 5: pass_in_lds<5, NT>(lds, L, p, tid); break;
+        case 4: pass_in_lds<4, NT>(lds, L, p, tid); break;
+        case 3: pass_in_lds<3, NT>(lds, L, p, tid); break;
+        case 2: pass_in_lds<2, NT>(lds, L, p, tid); break;
+        default: pass_in_lds<1, NT>(lds, L, p, tid); break;
+    }
+}
+
+// NT threads per workgroup: 256, or 1024 for segments of 16384 elements and more (their LDS
+// footprint allows only one or two workgroups per CU, which 256 threads would leave idle)
+template <int NT>
+__global__ __launch_bounds__(NT) void fwht_kernel(const uint16_t* __restrict__ x, int64_t ldx,
                                                    uint16_t* __restrict__ y, int64_t ldy, int cols, int logn,
                                                    int L, float scale) {
     extern __shared__ float lds[];
@@ -48,41 +78,47 @@ __global__ __launch_bounds__(256) void fwht_kernel(const uint16_t* __restrict__ 
     const uint16_t* xr = x + row * ldx + (int64_t)seg * L;
     uint16_t* yr = y + row * ldy + (int64_t)seg * L;
 
-    for (int c = tid; c < (L >> 3); c += 256) {
-        const uint4 v = *reinterpret_cast<const uint4*>(xr + c * 8);
-        float4 a = make_float4(bf16_lo(v.x), bf16_hi(v.x), bf16_lo(v.y), bf16_hi(v.y));
-        float4 b = make_float4(bf16_lo(v.z), bf16_hi(v.z), bf16_lo(v.w), bf16_hi(v.w));
-        *reinterpret_cast<float4*>(lds + c * 8) = a;
-        *reinterpret_cast<float4*>(lds + c * 8 + 4) = b;
+    // pass over bits 0..3 (n >= 128, so all four stages belong to every group)
+    for (int vt = tid; vt < (L >> 4); vt += NT) {
+        const uint4 v0 = *reinterpret_cast<const uint4*>(xr + vt * 16);
+        const uint4 v1 = *reinterpret_cast<const uint4*>(xr + vt * 16 + 8);
+        float a[16] = {bf16_lo(v0.x), bf16_hi(v0.x), bf16_lo(v0.y), bf16_hi(v0.y), bf16_lo(v0.z), bf16_hi(v0.z),
+                       bf16_lo(v0.w), bf16_hi(v0.w), bf16_lo(v1.x), bf16_hi(v1.x), bf16_lo(v1.y), bf16_hi(v1.y),
+                       bf16_lo(v1.z), bf16_hi(v1.z), bf16_lo(v1.w), bf16_hi(v1.w)};
+        butterflies<4>(a);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) lds[vt * 17 + e] = a[e];   // = padded(16 vt + e)
     }
     __syncthreads();
-    int p = 0;
-    while (p < logn) {
-        const int rb = (logn - p) >= 4 ? 4 : (logn - p);
-        switch (rb) {
-            case 4: pass_in_lds<4>(lds, L, p, tid); break;
-            case 3: pass_in_lds<3>(lds, L, p, tid); break;
-            case 2: pass_in_lds<2>(lds, L, p, tid); break;
-            default: pass_in_lds<1>(lds, L, p, tid); break;
-        }
-        p += rb;
+    // bits 4..7 (4..6 when n = 128)
+    const int rb1 = min(4, logn - 4);
+    pass_dispatch<NT>(lds, L, 4, rb1, tid);
+    __syncthreads();
+    int rem = logn - 8;
+    if (rem > 0) {
+        const int rb2 = rem <= 5 ? rem : (rem + 1) / 2;
+        pass_dispatch<NT>(lds, L, 8, rb2, tid);
         __syncthreads();
-    }
-    for (int c = tid; c < (L >> 3); c += 256) {
-        const float4 a = *reinterpret_cast<const float4*>(lds + c * 8);
-        const float4 b = *reinterpret_cast<const float4*>(lds + c * 8 + 4);
-        uint4 o;
-        if (scale != 1.0f) {
-            o.x = f32_to_bf16_bits(a.x * scale) | (f32_to_bf16_bits(a.y * scale) << 16);
-            o.y = f32_to_bf16_bits(a.z * scale) | (f32_to_bf16_bits(a.w * scale) << 16);
-            o.z = f32_to_bf16_bits(b.x * scale) | (f32_to_bf16_bits(b.y * scale) << 16);
-            o.w = f32_to_bf16_bits(b.z * scale) | (f32_to_bf16_bits(b.w * scale) << 16);
-        } else {
-            o.x = f32_to_bf16_bits(a.x) | (f32_to_bf16_bits(a.y) << 16);
-            o.y = f32_to_bf16_bits(a.z) | (f32_to_bf16_bits(a.w) << 16);
-            o.z = f32_to_bf16_bits(b.x) | (f32_to_bf16_bits(b.y) << 16);
-            o.w = f32_to_bf16_bits(b.z) | (f32_to_bf16_bits(b.w) << 16);
+        rem -= rb2;
+        if (rem > 0) {
+            pass_dispatch<NT>(lds, L, 8 + rb2, rem, tid);
+            __syncthreads();
         }
+    }
+    for (int c = tid; c < (L >> 3); c += NT) {
+        const float* src = lds + padded(c * 8);   // 8 words of one 16-word run: contiguous
+        float f[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) f[e] = src[e];
+        if (scale != 1.0f) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) f[e] = f[e] * scale;
+        }
+        uint4 o;
+        o.x = f32_to_bf16_bits(f[0]) | (f32_to_bf16_bits(f[1]) << 16);
+        o.y = f32_to_bf16_bits(f[2]) | (f32_to_bf16_bits(f[3]) << 16);
+        o.z = f32_to_bf16_bits(f[4]) | (f32_to_bf16_bits(f[5]) << 16);
+        o.w = f32_to_bf16_bits(f[6]) | (f32_to_bf16_bits(f[7]) << 16);
         *reinterpret_cast<uint4*>(yr + c * 8) = o;
     }
 }
@@ -110,16 +146,20 @@ extern "C" int ti8_fwht(const void* x, int64_t ldx, void* y, int64_t ldy, int64_
     if (nblocks > 0x7fffffffLL) return fail(TI8_ERR_SHAPE, "ti8_fwht: too many segments");
     int logn = 0;
     while ((1LL << logn) < n) ++logn;
-    const size_t shmem = (size_t)L * sizeof(float);
+    const size_t shmem = (size_t)(L + L / 16) * sizeof(float);
     static thread_local int attr_set_for = -1;
     int dev = 0;
     (void)hipGetDevice(&dev);
-    if (shmem > 64 * 1024 && attr_set_for != dev) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fwht_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+    if (attr_set_for != dev) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fwht_kernel<1024>), hipFuncAttributeMaxDynamicSharedMemorySize, 136 * 1024);
         if (e != hipSuccess) return fail(TI8_ERR_HIP, "ti8_fwht: cannot raise the LDS limit: %s", hipGetErrorString(e));
         attr_set_for = dev;
     }
-    hipLaunchKernelGGL(fwht_kernel, dim3((unsigned)nblocks), dim3(256), shmem, static_cast<hipStream_t>(stream),
-                       static_cast<const uint16_t*>(x), ldx, static_cast<uint16_t*>(y), ldy, (int)cols, logn, (int)L, scale);
+    if (L >= 16384)
+        hipLaunchKernelGGL(fwht_kernel<1024>, dim3((unsigned)nblocks), dim3(1024), shmem, static_cast<hipStream_t>(stream),
+                           static_cast<const uint16_t*>(x), ldx, static_cast<uint16_t*>(y), ldy, (int)cols, logn, (int)L, scale);
+    else
+        hipLaunchKernelGGL(fwht_kernel<256>, dim3((unsigned)nblocks), dim3(256), shmem, static_cast<hipStream_t>(stream),
+                           static_cast<const uint16_t*>(x), ldx, static_cast<uint16_t*>(y), ldy, (int)cols, logn, (int)L, scale);
     return check_launch("ti8_fwht");
 }
