@@ -12,8 +12,8 @@ config 2: X 8192x4096 bf16 ~N(0,1) with 1% of the input channels x20, W 4096x409
 Prints ONE JSON line.  `value` = 6*M*N*K int8 operations (three GEMMs) divided by the
 mean wall-clock time of a step, in TOPS.  `roofline` describes the dominant kernel (the
 i8 MFMA GEMM): 2*M*N*K operations per launch over its mean launch duration, measured with
-HIP events on the launch stream in a second pass of K steps (so the events do not sit in
-the region `value` is timed on).  `cpu_baseline` is the torch-CPU oracle of the same path
+HIP events on the launch stream around each of its launches while whole steps run, in a second
+pass of K steps (so the events do not sit in the region `value` is timed on).  `cpu_baseline` is the torch-CPU oracle of the same path
 timed once on the host cores on a bounded sample; it is a reported baseline, not a target.
 """
 import argparse
@@ -85,7 +85,6 @@ def main():
 
     import triton_int8_amd as T
     from triton_int8_amd import ops
-    from triton_int8_amd._lib import SCALE_BLOCK128, SCALE_ROW
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
@@ -104,39 +103,19 @@ def main():
     dt = (time.perf_counter() - t0) / args.steps
     tops = 6.0 * M * N * K / dt / 1e12
 
-    # ---- dominant kernel: the three GEMM launches of a step, timed alone with HIP events
-    if args.scheme == "double_channel":
-        xq, xs = ops.quant_row(X, clamp=True, inv_mode=1)
-        wq, ws = ops.quant_row(W, clamp=True, inv_mode=1)
-        dq, ds = ops.quant_row(dY, clamp=True, inv_mode=1)
-        wtq, wts = ops.quant_col_t(W, clamp=True, inv_mode=1)
-        dtq, dts = ops.quant_col_t(dY, clamp=True, inv_mode=1)
-        xtq, xts = ops.quant_col_t(X, clamp=True, inv_mode=1)
-        gemms = [lambda: ops.gemm_i8_nt(xq[None], wq, xs[None], SCALE_ROW, ws, SCALE_ROW, acc_i32_full=True),
-                 lambda: ops.gemm_i8_nt(dq[None], wtq, ds[None], SCALE_ROW, wts, SCALE_ROW, acc_i32_full=True),
-                 lambda: ops.gemm_i8_nt(dtq[None], xtq, dts[None], SCALE_ROW, xts, SCALE_ROW, acc_i32_full=True)]
-        kernel = "gemm_i8_kernel<256,256,2,4,EPI_ROWS>"
-    else:
-        xq, xqT, xs = ops.quant_block(X[None], clamp=True, with_transpose=True)
-        dq, dqT, ds = ops.quant_block(dY[None], clamp=True, with_transpose=True)
-        if args.scheme == "block_channel":
-            wq, ws = ops.quant_row(W, clamp=True)
-            wtq, wts = ops.quant_col_t(W, clamp=True)
-            gemms = [lambda: ops.gemm_i8_nt(xq, wq, xs, SCALE_BLOCK128, ws, SCALE_ROW),
-                     lambda: ops.gemm_i8_nt(dq, wtq, ds, SCALE_BLOCK128, wts, SCALE_ROW),
-                     lambda: ops.gemm_i8_nt(dqT, xqT, ds.transpose(1, 2), SCALE_BLOCK128, xs.transpose(1, 2), SCALE_BLOCK128)]
-        else:
-            xrq, xrs = ops.quant_row(X, clamp=True)
-            drq, drs = ops.quant_row(dY, clamp=True)
-            wq, wqT, ws = ops.quant_block(W[None], clamp=True, with_transpose=True)
-            dtq, dts = ops.quant_col_t(dY, clamp=True)
-            gemms = [lambda: ops.gemm_i8_nt(xrq[None], wq[0], xrs[None], SCALE_ROW, ws[0], SCALE_BLOCK128),
-                     lambda: ops.gemm_i8_nt(drq[None], wqT[0], drs[None], SCALE_ROW, ws[0].t(), SCALE_BLOCK128),
-                     lambda: ops.gemm_i8_nt(dtq[None], xqT[0], dts[None], SCALE_ROW, xs[0].t(), SCALE_BLOCK128)]
-        kernel = "gemm_i8_kernel<256,128,4,2,EPI_PROMOTE>"
-    for f in gemms:
-        f()
-    gemm_ms = [event_time_ms(f, args.steps) for f in gemms]
+    # ---- dominant kernel: the three GEMM launches of a step (Y, dX, dW), each bracketed by HIP
+    # events on the launch stream while whole steps run, in a second pass of K steps (so the events
+    # do not sit in the region `value` is timed on)
+    from triton_int8_amd import _lib
+    with _lib.timed_launches() as rec:
+        for _ in range(args.steps):
+            step()
+    torch.cuda.synchronize()
+    per_entry_ms = {name: sum(a.elapsed_time(b) for a, b in ev) / args.steps for name, ev in rec.items()}
+    g = [a.elapsed_time(b) for a, b in rec["ti8_gemm_i8_nt"]]
+    assert len(g) == 3 * args.steps
+    gemm_ms = [sum(g[i::3]) / args.steps for i in range(3)]
+    kernel = "gemm_i8_kernel<256,256,2,4,EPI_ROWS>" if args.scheme == "double_channel" else "gemm_i8_kernel<256,128,4,2,EPI_PROMOTE>"
     avg_ms = sum(gemm_ms) / len(gemm_ms)
     achieved = 2.0 * M * N * K / (avg_ms * 1e-3) / 1e12
 
@@ -157,7 +136,7 @@ def main():
 
     # HBM-side bytes per GEMM launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled on the device
     # copy above (profiles/bench_config2_block_channel_hbm_counters.md); measured for this scheme only
-    traffic = 393106918 if args.scheme == "block_channel" else None
+    traffic = 324650225 if args.scheme == "block_channel" else None
 
     out = {
         "metric": METRIC, "value": round(tops, 2), "unit": "TOPS", "n_gpus": 1, "steps": args.steps,
@@ -179,6 +158,7 @@ def main():
         "copy_GBs": round(2.0 * X.numel() * 2 / (copy_ms * 1e-3) / 1e9, 1),
         "bf16_matmul_ms_per_step": round(bf16_ms, 4),
         "bf16_matmul_tflops": round(6.0 * M * N * K / (bf16_ms * 1e-3) / 1e12, 1),
+        "entry_point_ms_per_step": {k: round(v, 4) for k, v in sorted(per_entry_ms.items())},
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.scheme)

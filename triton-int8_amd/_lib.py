@@ -3,6 +3,7 @@
 The library is the product: there is no fallback.  If it has not been built
 (``python triton-int8_amd/build.py``) importing any operator raises.
 """
+import contextlib
 import ctypes
 import os
 
@@ -64,9 +65,39 @@ def lib():
     return _lib
 
 
+_timing = None  # {entry point: [(start event, end event), ...]} while `timed_launches` is active
+
+
+@contextlib.contextmanager
+def timed_launches():
+    """Bracket every entry-point call with a pair of HIP events on the launch stream.
+
+    Yields the dict the pairs are appended to (``{name: [(start, end), ...]}``); read
+    ``start.elapsed_time(end)`` after a device synchronise.  Used by the benchmark to time the
+    kernels of a whole step where they run, between the other launches of that step.
+    """
+    global _timing
+    import torch
+    rec = {}
+    _timing = (rec, torch.cuda.Event)
+    try:
+        yield rec
+    finally:
+        _timing = None
+
+
 def call(name, *args):
     """Call an entry point; raise :class:`Ti8Error` with the library's message on failure."""
     l = lib()
-    rc = getattr(l, name)(*args)
+    t = _timing
+    if t is None:
+        rc = getattr(l, name)(*args)
+    else:
+        rec, Event = t
+        a, b = Event(enable_timing=True), Event(enable_timing=True)
+        a.record()
+        rc = getattr(l, name)(*args)
+        b.record()
+        rec.setdefault(name, []).append((a, b))
     if rc != 0:
         raise Ti8Error(name, rc, l.ti8_last_error().decode())
