@@ -69,9 +69,14 @@ enum ti8_combine {
 };
 
 enum ti8_gemm_flags {
-    TI8_GEMM_STRICT = 1   /* evaluate the combine formula literally (separate roundings, true
+    TI8_GEMM_STRICT = 1,  /* evaluate the combine formula literally (separate roundings, true
                              division); without it the kernel may use fma / reciprocal, which
                              moves results by a few fp32 ulps before the bf16 rounding */
+    TI8_GEMM_TILED = 2,   /* always take the LDS-tiled kernel */
+    TI8_GEMM_SKINNY = 4   /* take the few-rows kernel (no LDS staging, K split over waves) whenever
+                             it supports the scale modes; by default it is used for M <= 256.  Both
+                             kernels give bit-identical results with acc_i32_full; otherwise their
+                             fp32 sums associate differently (few ulps before the bf16 rounding) */
 };
 
 /* Library version (major*10000 + minor*100 + patch). */

@@ -29,6 +29,16 @@ def T():
     return triton_int8_amd
 
 
+@pytest.fixture(params=["tiled", "skinny"])
+def gemm_path(request, T):
+    """Run the case through the LDS-tiled GEMM kernel and through the few-rows kernel (the default
+    picks by M, and most cases here are small enough to land on the few-rows one only)."""
+    old = T.ops.GEMM_PATH
+    T.ops.GEMM_PATH = request.param
+    yield request.param
+    T.ops.GEMM_PATH = old
+
+
 def planted(seed, B=2, M=256, N=384):
     x = randn_bf16(make_gen(seed), B, M, N)
     x[0, :128, :128] = 0
@@ -162,7 +172,7 @@ PIPELINES = [("block_channel_fwd32", "fwd_32", obf.fwd_32, False),
 
 
 @pytest.mark.parametrize("module,fn,oracle_fn,three_d", PIPELINES)
-def test_entry_points_match_oracle(T, dev, module, fn, oracle_fn, three_d):
+def test_entry_points_match_oracle(T, dev, module, fn, oracle_fn, three_d, gemm_path):
     g = make_gen(7)
     a = randn_bf16(g, 2, 256, 2048)
     b = randn_bf16(g, 2, 384, 2048) if three_d else randn_bf16(g, 384, 2048)
@@ -174,6 +184,46 @@ def test_entry_points_match_oracle(T, dev, module, fn, oracle_fn, three_d):
         assert bits_equal(C, Co)          # integer accumulation + literal epilogue: exact
     ref = torch.matmul(a.float(), b.float().transpose(-1, -2))
     assert float(T.calc_diff(C.cpu(), ref)) < 1e-3
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 128, 128), (128, 256, 384), (256, 128, 640), (128, 384, 896), (384, 256, 4096)])
+def test_few_rows_kernel(T, dev, M, N, K):
+    """The kernel for few rows (K split over waves, partials added in LDS) against the oracle and
+    against the tiled kernel, for every number of K tiles modulo 4 and every scale layout it takes."""
+    from triton_int8_amd._lib import SCALE_BLOCK128, SCALE_ROW
+    g = make_gen(M + N + K)
+    A = torch.randint(-127, 128, (2, M, K), generator=g, dtype=torch.int8)
+    B = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+    B3 = torch.randint(-127, 128, (2, N, K), generator=g, dtype=torch.int8)
+    pos = lambda *shape: torch.rand(*shape, generator=g) * 1e-2 + 1e-4
+    sa_row, sb_row, sb3_row = pos(2, M), pos(N), pos(2, N)
+    sa_blk, sb_blk, sb3_blk = pos(2, M // 128, K // 128), pos(N // 128, K // 128), pos(2, N // 128, K // 128)
+    Ad, Bd, B3d = A.to(dev), B.to(dev), B3.to(dev)
+
+    def run(path, *args, **kw):
+        T.ops.GEMM_PATH = path
+        try:
+            return T.ops.gemm_i8_nt(*args, **kw)
+        finally:
+            T.ops.GEMM_PATH = "auto"
+
+    # int32 over the whole K, per-row scales: bit-exact, and identical in both kernels
+    want = odf.dequant_epilogue(odf.gemm_i32(A, B), sa_row, sb_row)
+    args = (Ad, Bd, sa_row.to(dev), SCALE_ROW, sb_row.to(dev), SCALE_ROW)
+    got = run("skinny", *args, acc_i32_full=True)
+    assert bits_equal(got, want) and torch.equal(got, run("tiled", *args, acc_i32_full=True))
+    # promotion per 128-deep K block: every mix of row / block scales, shared and batched B
+    for sA, mA, oA in ((sa_blk, SCALE_BLOCK128, olin.BLOCK), (sa_row, SCALE_ROW, olin.ROW)):
+        for Bq, sB, mB, oB in ((B, sb_row, SCALE_ROW, olin.ROW), (B, sb_blk, SCALE_BLOCK128, olin.BLOCK),
+                               (B3, sb3_row, SCALE_ROW, olin.ROW), (B3, sb3_blk, SCALE_BLOCK128, olin.BLOCK)):
+            if mA == SCALE_ROW and mB == SCALE_ROW:
+                continue
+            want = torch.stack([olin.gemm_scaled(A[b], sA[b], oA, Bq[b] if Bq.dim() == 3 else Bq,
+                                                 sB[b] if Bq.dim() == 3 else sB, oB) for b in range(2)])
+            args = (Ad, Bq.to(dev), sA.to(dev), mA, sB.to(dev), mB)
+            got = run("skinny", *args)
+            assert rel_err(got, want) <= 1e-4          # fp32 association only; the bar is REL_TOL
+            assert rel_err(run("tiled", *args), want) <= 1e-4
 
 
 def test_strict_mode_is_bit_exact(T, dev):
@@ -190,7 +240,7 @@ def test_strict_mode_is_bit_exact(T, dev):
     assert bits_equal(T.fused_bwd33.fused_int8_gemm(a.to(dev), b3.to(dev), strict=True), ofb.bwd_33(a, b3))
 
 
-def test_bwd33_on_transposed_views(T, dev):
+def test_bwd33_on_transposed_views(T, dev, gemm_path):
     g = make_gen(9)
     at = randn_bf16(g, 1, 1024, 256).transpose(1, 2)
     bt = randn_bf16(g, 1, 1024, 384).transpose(1, 2)
@@ -200,7 +250,7 @@ def test_bwd33_on_transposed_views(T, dev):
 
 @pytest.mark.parametrize("scheme,h", [("block_channel", None), ("row_block", None), ("double_channel", None),
                                       ("block_channel", 128), ("row_block", 128), ("double_channel", "full")])
-def test_linear_fwd_bwd(T, dev, scheme, h):
+def test_linear_fwd_bwd(T, dev, scheme, h, gemm_path):
     g = make_gen(10)
     N = 512 if h == "full" else 384          # the full-length rotation needs power-of-two dims
     X = randn_bf16(g, 2, 256, 1024)
@@ -219,7 +269,7 @@ def test_linear_fwd_bwd(T, dev, scheme, h):
         assert float(T.calc_diff(got.cpu(), ref)) < 1e-2
 
 
-def test_autograd_module(T, dev):
+def test_autograd_module(T, dev, gemm_path):
     g = make_gen(11)
     lin = T.Int8Linear(512, 256, bias=True, device=dev)
     x = randn_bf16(g, 2, 128, 512).to(dev).requires_grad_(True)
@@ -234,7 +284,7 @@ def test_autograd_module(T, dev):
 
 
 @pytest.mark.parametrize("tokens", [16, 100, 128, 300])
-def test_skinny_and_ragged_token_counts(T, dev, tokens):
+def test_skinny_and_ragged_token_counts(T, dev, tokens, gemm_path):
     """Zero-pad semantics for M that is not a multiple of the 128-row tile (config 5's M = 16)."""
     g = make_gen(12 + tokens)
     X, W, dY = randn_bf16(g, tokens, 512), randn_bf16(g, 256, 512, std=0.02), randn_bf16(g, tokens, 256, std=1e-3)
@@ -274,7 +324,7 @@ def test_decoder_layer_step_matches_bf16_twin(T, dev):
     assert cos(outs[0][4], outs[1][4]) > 0.3
 
 
-def test_golden_vectors_on_gpu(T, dev):
+def test_golden_vectors_on_gpu(T, dev, gemm_path):
     z = load("quant_256x256.npz")
     x = bf16(z["x"]).to(dev)
     q, s = T.block_channel_fwd32.triton_per_block_quant(x)

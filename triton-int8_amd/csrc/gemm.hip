@@ -13,58 +13,9 @@
 // operand and the 16 bytes k = 16*(l / 32) .. +15 of the 32-deep slice (the same map
 // for both operands, which is all an NT dot product needs); result register r of lane
 // l is C[8*(r/4) + 4*(l/32) + r%4][l % 32] with rows from A and columns from B.
-#include "ti8_common.h"
+#include "gemm_args.h"
 
 namespace ti8 {
-
-struct ScaleDesc {
-    const float* p;
-    int mode;         // ti8_scale_mode
-    int64_t bs, rs, ks;
-};
-
-struct GemmArgs {
-    const int8_t* A;
-    const int8_t* B;
-    void* C;
-    int64_t bsa, lda, bsb, ldb, bsc, ldc;
-    ScaleDesc sa, sb;
-    int M, N, K;
-    int tiles_m, tiles_n;
-    int combine;
-    int strict;
-    float out_scale, post_scale;
-};
-
-// EPI_PROMOTE: the per-K-tile factor is uniform over a wave's 128 x 64 tile (block or per-row scales
-// on both operands); EPI_PROMOTE_LANE: operand B carries one scale per (column, K tile).
-enum { EPI_I32 = 0, EPI_ROWS = 1, EPI_PROMOTE = 2, EPI_STRICT = 3, EPI_PROMOTE_LANE = 4 };
-
-
-// scale of operand row `row` at K block kb
-__device__ __forceinline__ float scale_at(const ScaleDesc& d, int64_t batch, int row, int kb) {
-    switch (d.mode) {
-        case TI8_SCALE_ROW: return d.p[batch * d.bs + (int64_t)row * d.rs];
-        case TI8_SCALE_BLOCK128: return d.p[batch * d.bs + (int64_t)(row >> 7) * d.rs + (int64_t)kb * d.ks];
-        case TI8_SCALE_ROW_K128: return d.p[batch * d.bs + (int64_t)row * d.rs + (int64_t)kb * d.ks];
-        default: return d.p[batch * d.bs + (int64_t)(row >> 7) * d.rs + (int64_t)(kb >> 1) * d.ks];
-    }
-}
-
-// One wave's share of a K tile: NI global->LDS instructions of 64 x 16 bytes; instruction i
-// fills the 1 KiB slab at lds + i*1024 (lane l lands at byte 16*l of the slab) from
-// base + i*stride8 (wave-uniform: 8 rows further per instruction) + voff[(t0 + i) & 1] (per lane).
-template <int NI>
-__device__ __forceinline__ void issue_tile_loads(const int8_t* base, int64_t stride8, const uint32_t (&voff)[2], int t0,
-                                                 int8_t* lds) {
-#if defined(__HIP_DEVICE_COMPILE__)  // the builtin only exists in the device pass
-#pragma unroll
-    for (int i = 0; i < NI; ++i)
-        __builtin_amdgcn_global_load_lds(base + i * stride8 + voff[(t0 + i) & 1], lds + i * 1024, 16, 0, 0);
-#else
-    (void)base; (void)stride8; (void)voff; (void)t0; (void)lds;
-#endif
-}
 
 // Interleaving hint for one k-step: TM*TN MFMAs, with up to NDS LDS reads, NVM global->LDS
 // loads and NVA*TM*TN VALU ops slotted one group per MFMA so that the matrix pipe never waits
@@ -196,6 +147,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
     const bool a_in = FAST && g.sa.mode != TI8_SCALE_ROW, b_in = FAST && g.sb.mode != TI8_SCALE_ROW;
     const int sha = g.sa.mode == TI8_SCALE_BLOCK_K256 ? 1 : 0, shb = g.sb.mode == TI8_SCALE_BLOCK_K256 ? 1 : 0;
     float fvec[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+    float fraw_a[4] = {1.0f, 1.0f, 1.0f, 1.0f}, fraw_b[4] = {1.0f, 1.0f, 1.0f, 1.0f};
     const float* pfb[TN];  // LANEB: this lane's column of B's scale grid
     if (FAST) {
         static_assert(!FAST || (128 % (TM * 32) == 0 && 128 % (TN * 32) == 0), "a wave tile must lie inside one 128 x 128 scale block");
@@ -204,19 +156,35 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
         const int colblk = min(n0 + wn * TN * 32, g.N - 1) >> 7;
         const float* pb = g.sb.p + batch * g.sb.bs + (int64_t)colblk * g.sb.rs;
         const int nkt = g.K >> 7;
+        // unconditional loads (an operand without in-loop factors is read with stride 0 and its
+        // value dropped): a load under a branch is waited for on the spot, one after the other
+        const int64_t ska = a_in ? g.sa.ks : 0, skb = (b_in && !LANEB) ? g.sb.ks : 0;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             const int kt = min(c * 64 + lane, nkt - 1);
-            float f = a_in ? pa[(int64_t)(kt >> sha) * g.sa.ks] : 1.0f;
-            if (!LANEB && b_in) f = f * pb[(int64_t)(kt >> shb) * g.sb.ks];
-            if (!LANEB && divide) f = 1.0f / f;
-            fvec[c] = f;
+            fraw_a[c] = pa[(int64_t)(kt >> sha) * ska];
+            fraw_b[c] = pb[(int64_t)(kt >> shb) * skb];
         }
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
             const int col = min(n0 + (wn * TN + j) * 32 + fr_row, g.N - 1);
             pfb[j] = g.sb.p + batch * g.sb.bs + (int64_t)col * g.sb.rs;
         }
+    }
+    // column scale vector of the epilogue (4 columns per lane there), fetched now for the same reason
+    constexpr int WCOLS = TN * 32;                       // columns of the wave tile
+    constexpr int LPR = WCOLS / 4;                       // lanes per row in the epilogue's read-back
+    constexpr int RPI = 64 / LPR;                        // rows per wave instruction there
+    const int rb_col = (lane % LPR) * 4;
+    const int rb_row = lane / LPR;
+    const int ncol0 = n0 + wn * WCOLS + rb_col;          // first of this lane's 4 columns
+    const bool col_part = EPI == EPI_ROWS || (FAST && g.sb.mode == TI8_SCALE_ROW);
+    const bool row_part = EPI == EPI_ROWS || (FAST && g.sa.mode == TI8_SCALE_ROW);
+    float coln[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+    if (EPI == EPI_ROWS || FAST) {
+        const int64_t cs = col_part ? g.sb.rs : 0;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) coln[c] = g.sb.p[batch * g.sb.bs + (int64_t)min(ncol0 + c, g.N - 1) * cs];
     }
     float f_cur = 1.0f;   // wave-uniform factor of the K tile being accumulated
     float fb[TN];         // LANEB only: per-lane factors of that tile
@@ -275,6 +243,19 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
     const int tA0 = wave * A_INSTR, tB0 = wave * B_INSTR;
     issue_tile_loads<A_INSTR>(baseA, strideA8, voffA, tA0, wA);
     issue_tile_loads<B_INSTR>(baseB, strideB8, voffB, tB0, wB);
+    if (FAST) {   // the scale loads have been in flight since before the tile loads
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            float f = a_in ? fraw_a[c] : 1.0f;
+            if (!LANEB && b_in) f = f * fraw_b[c];
+            if (!LANEB && divide) f = 1.0f / f;
+            fvec[c] = f;
+        }
+    }
+    if (divide) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) coln[c] = 1.0f / coln[c];
+    }
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     const int klast = (nk - 1) * 128;  // loads past the last K tile re-read it into a free buffer: no branches in the loop
@@ -346,28 +327,23 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
     __syncthreads();
 
     // ---- epilogue ---------------------------------------------------------------------
-    // Each wave moves its accumulators through a private 16 KiB LDS slab, 32 tile rows at
-    // a time, so that the global stores are whole row segments (4 columns per lane, two
-    // rows of WN-th of the tile per wave instruction) instead of one column per lane.
-    // The main loop ended with a workgroup barrier, so the operand buffers are free.
-    constexpr int WCOLS = TN * 32;                       // columns of the wave tile
-    constexpr int LPR = WCOLS / 4;                       // lanes per row in the read-back
-    constexpr int RPI = 64 / LPR;                        // rows per wave instruction
+    // Each wave moves its accumulators through a private LDS slab, 32 tile rows at a time, so
+    // that the global stores are whole row segments (4 columns per lane) instead of one column
+    // per lane.  The main loop ended with a workgroup barrier, so the operand buffers are free.
     static_assert(WCOLS * 32 * 4 * NW <= 2 * (A_BYTES + B_BYTES), "epilogue slab does not fit");
     uint32_t* slab = reinterpret_cast<uint32_t*>(smem) + wave * (32 * WCOLS);
-    const int rb_col = (lane % LPR) * 4;
-    const int rb_row = lane / LPR;
-    const int ncol0 = n0 + wn * WCOLS + rb_col;          // first of this lane's 4 columns
-    float coln[4] = {1.0f, 1.0f, 1.0f, 1.0f};
-    if (EPI == EPI_ROWS || (FAST && g.sb.mode == TI8_SCALE_ROW)) {
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            coln[c] = scale_at(g.sb, batch, min(ncol0 + c, g.N - 1), 0);
-            if (divide) coln[c] = 1.0f / coln[c];
-        }
-    }
+    constexpr int NRR = 32 / RPI;                        // rows of a 32-row block per lane
+    const float* prow = g.sa.p + batch * g.sa.bs;        // per-row scales of A (unused pointer otherwise)
+    const int64_t rstride = row_part ? g.sa.rs : 0;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
+        const int mbase = m0 + (wm * TM + i) * 32;
+        // the block's row scales: all loads go out before the slab traffic, nothing waits per row
+        float rowv[NRR];
+        if (EPI == EPI_ROWS || FAST) {
+#pragma unroll
+            for (int k = 0; k < NRR; ++k) rowv[k] = prow[(int64_t)min(mbase + rb_row + k * RPI, g.M - 1) * rstride];
+        }
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -380,8 +356,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
         // same wave reads what it wrote: an LDS counter wait is enough, no barrier
         __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
         __builtin_amdgcn_wave_barrier();
-        const int mbase = m0 + (wm * TM + i) * 32;
-        for (int rr = rb_row; rr < 32; rr += RPI) {
+#pragma unroll
+        for (int k = 0; k < NRR; ++k) {
+            const int rr = rb_row + k * RPI;
             const int m = mbase + rr;
             const uint4 w = *reinterpret_cast<const uint4*>(slab + rr * WCOLS + rb_col);
             if (m >= g.M || ncol0 >= g.N) continue;  // N is a multiple of 4: a lane's 4 columns are all in or all out
@@ -393,7 +370,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
             float t[4];
             const uint32_t wb[4] = {w.x, w.y, w.z, w.w};
             if (EPI == EPI_ROWS) {
-                const float rowm = scale_at(g.sa, batch, m, 0);
+                const float rowm = rowv[k];
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
                     float v = static_cast<float>(static_cast<int32_t>(wb[c])) * rowm;
@@ -403,16 +380,15 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
                 }
             } else {
                 float rowm = 1.0f;
-                const bool row_part = (FAST && g.sa.mode == TI8_SCALE_ROW);
-                if (row_part) {
-                    rowm = scale_at(g.sa, batch, m, 0);
+                if (FAST && row_part) {
+                    rowm = rowv[k];
                     if (divide) rowm = 1.0f / rowm;
                 }
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
                     float v = __uint_as_float(wb[c]);
-                    if (row_part) v = v * rowm;
-                    if (FAST && g.sb.mode == TI8_SCALE_ROW) v = v * coln[c];
+                    if (FAST && row_part) v = v * rowm;
+                    if (FAST && col_part) v = v * coln[c];
                     if (g.out_scale != 1.0f) v = v * g.out_scale;
                     t[c] = v;
                 }
@@ -481,7 +457,8 @@ extern "C" int ti8_gemm_i8_nt(const int8_t* A, int64_t bsa, int64_t lda, const i
     if (int e = check_scale(fn, "A", sA, modeA)) return e;
     if (int e = check_scale(fn, "B", sB, modeB)) return e;
     if (combine < 0 || combine > 2) return fail(TI8_ERR_MODE, "%s: unknown combine %d", fn, combine);
-    if (gemm_flags & ~TI8_GEMM_STRICT) return fail(TI8_ERR_MODE, "%s: unknown flag 0x%x", fn, gemm_flags);
+    if (gemm_flags & ~(TI8_GEMM_STRICT | TI8_GEMM_TILED | TI8_GEMM_SKINNY)) return fail(TI8_ERR_MODE, "%s: unknown flag 0x%x", fn, gemm_flags);
+    if ((gemm_flags & TI8_GEMM_TILED) && (gemm_flags & TI8_GEMM_SKINNY)) return fail(TI8_ERR_MODE, "%s: TI8_GEMM_TILED and TI8_GEMM_SKINNY exclude each other", fn);
     if (acc_i32_full && (modeA != TI8_SCALE_ROW || modeB != TI8_SCALE_ROW))
         return fail(TI8_ERR_MODE, "%s: int32 accumulation over the whole K needs per-row scales on both operands", fn);
     if ((modeA == TI8_SCALE_BLOCK_K256 || modeB == TI8_SCALE_BLOCK_K256) && (K % 256))
@@ -498,6 +475,9 @@ extern "C" int ti8_gemm_i8_nt(const int8_t* A, int64_t bsa, int64_t lda, const i
     a.strict = (gemm_flags & TI8_GEMM_STRICT) ? 1 : 0;
     a.out_scale = out_scale; a.post_scale = post_scale;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    // few rows: too few 256-row tiles to fill the machine, take the kernel that splits N and K finer
+    const bool want_skinny = (gemm_flags & TI8_GEMM_SKINNY) || (!(gemm_flags & TI8_GEMM_TILED) && M <= 256);
+    if (want_skinny && !a.strict && skinny_supported(a)) return launch_skinny(a, batch, acc_i32_full != 0, st);
     if (acc_i32_full) return launch<256, 256, 2, 4, EPI_ROWS>(a, batch, st);
     // the fast promotion keeps at most 256 per-K-tile factors in registers and cannot apply a
     // factor that varies per row of A inside the loop: those cases take the literal kernel

@@ -1,0 +1,61 @@
+// Argument block, scale descriptors and epilogue kinds shared by the INT8 GEMM kernels.
+#pragma once
+#include "ti8_common.h"
+
+namespace ti8 {
+
+struct ScaleDesc {
+    const float* p;
+    int mode;         // ti8_scale_mode
+    int64_t bs, rs, ks;
+};
+
+struct GemmArgs {
+    const int8_t* A;
+    const int8_t* B;
+    void* C;
+    int64_t bsa, lda, bsb, ldb, bsc, ldc;
+    ScaleDesc sa, sb;
+    int M, N, K;
+    int tiles_m, tiles_n;
+    int combine;
+    int strict;
+    float out_scale, post_scale;
+};
+
+// EPI_PROMOTE: the per-K-tile factor is uniform over a wave's 128 x 64 tile (block or per-row scales
+// on both operands); EPI_PROMOTE_LANE: operand B carries one scale per (column, K tile).
+enum { EPI_I32 = 0, EPI_ROWS = 1, EPI_PROMOTE = 2, EPI_STRICT = 3, EPI_PROMOTE_LANE = 4 };
+
+
+// scale of operand row `row` at K block kb
+__device__ __forceinline__ float scale_at(const ScaleDesc& d, int64_t batch, int row, int kb) {
+    switch (d.mode) {
+        case TI8_SCALE_ROW: return d.p[batch * d.bs + (int64_t)row * d.rs];
+        case TI8_SCALE_BLOCK128: return d.p[batch * d.bs + (int64_t)(row >> 7) * d.rs + (int64_t)kb * d.ks];
+        case TI8_SCALE_ROW_K128: return d.p[batch * d.bs + (int64_t)row * d.rs + (int64_t)kb * d.ks];
+        default: return d.p[batch * d.bs + (int64_t)(row >> 7) * d.rs + (int64_t)(kb >> 1) * d.ks];
+    }
+}
+
+// One wave's share of a K tile: NI global->LDS instructions of 64 x 16 bytes; instruction i
+// fills the 1 KiB slab at lds + i*1024 (lane l lands at byte 16*l of the slab) from
+// base + i*stride8 (wave-uniform: 8 rows further per instruction) + voff[(t0 + i) & 1] (per lane).
+template <int NI>
+__device__ __forceinline__ void issue_tile_loads(const int8_t* base, int64_t stride8, const uint32_t (&voff)[2], int t0,
+                                                 int8_t* lds) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the builtin only exists in the device pass
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+        __builtin_amdgcn_global_load_lds(base + i * stride8 + voff[(t0 + i) & 1], lds + i * 1024, 16, 0, 0);
+#else
+    (void)base; (void)stride8; (void)voff; (void)t0; (void)lds;
+#endif
+}
+
+// Kernel for few rows (gemm_skinny.hip): M a multiple of 128, operand A without per-(row, K tile)
+// scales.  i32_full: int32 accumulation over the whole K with per-row scales (bit-exact path).
+bool skinny_supported(const GemmArgs& a);
+int launch_skinny(const GemmArgs& a, int64_t batch, bool i32_full, hipStream_t st);
+
+}  // namespace ti8
