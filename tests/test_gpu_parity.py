@@ -297,6 +297,25 @@ def test_skinny_and_ragged_token_counts(T, dev, tokens, gemm_path):
                 assert bits_equal(a, b)
 
 
+@pytest.mark.parametrize("tokens,scheme", [(256, "block_channel"), (16, "block_channel"), (384, "double_channel"), (128, "row_block")])
+def test_graphed_step_replays_match_eager(T, dev, tokens, scheme):
+    """A whole fwd+bwd step captured into a HIP graph: every replay, with eager work and device
+    synchronisations in between and with new inputs, must equal the eager result bit for bit."""
+    g = make_gen(40 + tokens)
+    W = randn_bf16(g, 256, 512, std=0.02).to(dev)
+    mk = lambda: (randn_bf16(g, tokens, 512).to(dev), randn_bf16(g, tokens, 256, std=1e-3).to(dev))
+    X0, dY0 = mk()
+    step = T.GraphedStep(lambda x, w, dy: T.linear_fwd_bwd(x, w, dy, scheme), X0, W, dY0)
+    for it in range(4):
+        X, dY = (X0, dY0) if it == 0 else mk()
+        eager = T.linear_fwd_bwd(X, W, dY, scheme)          # eager launches between the replays
+        torch.cuda.synchronize()
+        got = step(X, W, dY)
+        torch.cuda.synchronize()
+        for a, b in zip(got, eager):
+            assert torch.equal(a, b), f"replay {it} differs from the eager result"
+
+
 def test_decoder_layer_step_matches_bf16_twin(T, dev):
     """One training step of a (reduced-width) Llama-style layer with every linear in INT8 against its
     bf16 twin: same loss and gradients up to int8 noise (cosine similarity)."""

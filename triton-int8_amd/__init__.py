@@ -11,10 +11,11 @@ top-level shim of that name loads this package).
 """
 from . import _lib  # noqa: F401
 from . import (block_channel_bwd33, block_channel_fwd32, decoder, double_channel_bwd33, double_channel_fwd32,
-               double_channel_triton_bwd, double_channel_triton_fwd, fused_bwd33, fused_fwd32, latency, linear, ops,
+               double_channel_triton_bwd, double_channel_triton_fwd, fused_bwd33, fused_fwd32, graph, latency, linear, ops,
                tilelang_block_channel_bwd, tilelang_block_channel_fwd)
 from ._common import calc_diff
 from .decoder import DecoderLayer
+from .graph import GraphedStep
 from .linear import Int8Linear, Int8LinearFunction, linear_fwd_bwd
 
 __version__ = "0.1.0"
