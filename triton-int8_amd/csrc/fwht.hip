@@ -115,10 +115,10 @@ __global__ __launch_bounds__(NT) void fwht_kernel(const uint16_t* __restrict__ x
             for (int e = 0; e < 8; ++e) f[e] = f[e] * scale;
         }
         uint4 o;
-        o.x = f32_to_bf16_bits(f[0]) | (f32_to_bf16_bits(f[1]) << 16);
-        o.y = f32_to_bf16_bits(f[2]) | (f32_to_bf16_bits(f[3]) << 16);
-        o.z = f32_to_bf16_bits(f[4]) | (f32_to_bf16_bits(f[5]) << 16);
-        o.w = f32_to_bf16_bits(f[6]) | (f32_to_bf16_bits(f[7]) << 16);
+        o.x = pack_bf16x2(f[0], f[1]);
+        o.y = pack_bf16x2(f[2], f[3]);
+        o.z = pack_bf16x2(f[4], f[5]);
+        o.w = pack_bf16x2(f[6], f[7]);
         *reinterpret_cast<uint4*>(yr + c * 8) = o;
     }
 }

@@ -394,8 +394,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
                 }
             }
             uint2 o;
-            o.x = f32_to_bf16_bits(t[0]) | (f32_to_bf16_bits(t[1]) << 16);
-            o.y = f32_to_bf16_bits(t[2]) | (f32_to_bf16_bits(t[3]) << 16);
+            o.x = pack_bf16x2(t[0], t[1]);
+            o.y = pack_bf16x2(t[2], t[3]);
             *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(g.C) + off) = o;
         }
         __builtin_amdgcn_s_waitcnt(0xc07f);

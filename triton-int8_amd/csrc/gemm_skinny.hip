@@ -222,7 +222,7 @@ __global__ __launch_bounds__(256) void gemm_i8_skinny_kernel(const GemmArgs g) {
             if (col_part) v = v * coln;
             if (g.out_scale != 1.0f) v = v * g.out_scale;
         }
-        crow[(int64_t)m * g.ldc] = static_cast<uint16_t>(f32_to_bf16_bits(v));
+        crow[(int64_t)m * g.ldc] = static_cast<uint16_t>(pack_bf16x2(v, 0.0f));
     }
 }
 

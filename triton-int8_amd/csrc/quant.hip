@@ -62,9 +62,20 @@ __device__ __forceinline__ float absmax8(const uint4& v, float m) {
 }
 
 
+// Value of `v` in another lane of the same row of 16 lanes (DPP: no LDS traffic, and the move
+// folds into the add that consumes it).  CTRL: 0xB1 / 0x4E = quad_perm lane^1 / lane^2,
+// 0x104 / 0x114 = row_shl:4 / row_shr:4 (lane+4 / lane-4), 0x128 = row_ror:8 (lane^8).
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+
 // 128-point Walsh-Hadamard transform of a row segment held as 8 consecutive bf16 per lane by 16
 // consecutive lanes (lane%16 = chunk index): butterflies in the fixed order stride 1, 2, 4 (in
 // registers), 8, 16, 32, 64 (lane xor 1, 2, 4, 8), fp32, un-normalised; one rounding to bf16.
+// A cross-lane stage is (a, b) -> (a + b, a - b) with a in the lane whose bit is clear: the lower
+// lane computes a + partner, the upper one partner - a = partner + (-a), so flipping the sign of
+// the own value in upper lanes (one xor) makes both a single add with a DPP operand.
 __device__ __forceinline__ uint4 fwht128_bf16(const uint4& v, int lane) {
     float a[8] = {bf16_lo(v.x), bf16_hi(v.x), bf16_lo(v.y), bf16_hi(v.y), bf16_lo(v.z), bf16_hi(v.z), bf16_lo(v.w), bf16_hi(v.w)};
 #pragma unroll
@@ -76,20 +87,25 @@ __device__ __forceinline__ uint4 fwht128_bf16(const uint4& v, int lane) {
                 a[e] = u + w;
                 a[e + h] = u - w;
             }
+    const uint32_t s1 = (lane & 1) ? 0x80000000u : 0u, s2 = (lane & 2) ? 0x80000000u : 0u;
+    const uint32_t s8 = (lane & 8) ? 0x80000000u : 0u;
+    const bool up4 = (lane & 4) != 0;
 #pragma unroll
-    for (int m = 1; m < 16; m <<= 1) {
-        const bool upper = (lane & m) != 0;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const float p = __shfl_xor(a[e], m, 64);
-            a[e] = upper ? (p - a[e]) : (a[e] + p);   // (a, b) -> (a + b, a - b), a = the lane with the bit clear
-        }
+    for (int e = 0; e < 8; ++e) {
+        float x = a[e];
+        x = dpp_f32<0xB1>(x) + __uint_as_float(__float_as_uint(x) ^ s1);
+        x = dpp_f32<0x4E>(x) + __uint_as_float(__float_as_uint(x) ^ s2);
+        const float lo = x + dpp_f32<0x104>(x);   // lanes with bit 2 clear: own + lane+4
+        const float hi = dpp_f32<0x114>(x) - x;   // lanes with bit 2 set: lane-4 - own
+        x = up4 ? hi : lo;
+        x = dpp_f32<0x128>(x) + __uint_as_float(__float_as_uint(x) ^ s8);
+        a[e] = x;
     }
     uint4 o;
-    o.x = f32_to_bf16_bits(a[0]) | (f32_to_bf16_bits(a[1]) << 16);
-    o.y = f32_to_bf16_bits(a[2]) | (f32_to_bf16_bits(a[3]) << 16);
-    o.z = f32_to_bf16_bits(a[4]) | (f32_to_bf16_bits(a[5]) << 16);
-    o.w = f32_to_bf16_bits(a[6]) | (f32_to_bf16_bits(a[7]) << 16);
+    o.x = pack_bf16x2(a[0], a[1]);
+    o.y = pack_bf16x2(a[2], a[3]);
+    o.z = pack_bf16x2(a[4], a[5]);
+    o.w = pack_bf16x2(a[6], a[7]);
     return o;
 }
 

@@ -45,6 +45,15 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
     return u >> 16;
 }
 
+// two fp32 -> two bf16 in one dword (`lo` in the low half), round to nearest even: gfx950's
+// v_cvt_pk_bf16_f32, same results as f32_to_bf16_bits for every finite value and infinity
+typedef __bf16 ti8_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float ti8_f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    const ti8_f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, ti8_bf16x2));
+}
+
 // max over the 64 lanes of a wavefront, result in every lane
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
