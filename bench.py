@@ -1,13 +1,17 @@
 #!/usr/bin/env python3
 """Benchmark of the INT8 linear layer (forward + backward) on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--scheme block_channel]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--scheme block_channel] [--config 2]
 
 One step = one pass of the hot path over one batch of synthetic input resident in HBM:
 Y = X W^T, dX = dY W, dW = dY^T X, every operand quantised to int8 on the way (all
 quantiser launches are inside the timed region).  The workload is BASELINE.json's
 config 2: X 8192x4096 bf16 ~N(0,1) with 1% of the input channels x20, W 4096x4096
 ~N(0,0.02), dY 8192x4096 ~N(0,1e-3), seed 1, block-channel scheme.
+
+``--config 3|4|5`` times the other benchmark configurations (Llama MLP shapes in the double-channel
+scheme; the fused Hadamard path at 8192^3; the decoder layer step and the M = 16 / 128 shapes) with the
+same protocol and prints a shorter line; the default, config 2, is the headline.
 
 Prints ONE JSON line.  `value` = 6*M*N*K int8 operations (three GEMMs) divided by the
 mean wall-clock time of a step, in TOPS.  `roofline` describes the dominant kernel (the
@@ -43,6 +47,90 @@ def make_inputs(m=M, k=K, n=N, seed=1):
     return X.to(torch.bfloat16), W.to(torch.bfloat16), dY.to(torch.bfloat16)
 
 
+def make_operand(rows, cols, gen, kind, std=1.0, outlier_frac=0.0, outlier_mul=1.0):
+    """bf16 operand of a benchmark configuration: N(0, std), optional outlier channels, or Student-t(3)."""
+    if kind == "student_t":
+        x = torch.randn(rows, cols, generator=gen) / torch.sqrt(torch.randn(3, rows, cols, generator=gen).pow(2).mean(0))
+    else:
+        x = torch.randn(rows, cols, generator=gen) * std
+    if outlier_frac:
+        idx = torch.randperm(cols, generator=gen)[: int(-(-cols * outlier_frac // 1))]
+        x[:, idx] *= outlier_mul
+    return x.to(torch.bfloat16)
+
+
+def other_config(args, T, dev):
+    """Configs 3-5: the same step protocol on their shapes; one short JSON line."""
+    from triton_int8_amd import _lib
+    cfg = args.config
+    g = torch.Generator().manual_seed(cfg - 1)
+    layers = []   # (X, W, dY, scheme, hadamard)
+    if cfg == 3:
+        for (k, n) in ((4096, 14336), (14336, 4096)):
+            layers.append((make_operand(16384, k, g, "normal", outlier_frac=0.005, outlier_mul=50.0),
+                           make_operand(n, k, g, "normal", std=0.02), make_operand(16384, n, g, "normal", std=1e-3),
+                           "double_channel", None))
+        name = "config 3: double_channel fwd+bwd, 16384 tokens, 4096->14336 and 14336->4096, 0.5% channels x50"
+    elif cfg == 4:
+        layers.append((make_operand(8192, 8192, g, "student_t"), make_operand(8192, 8192, g, "normal", std=0.02),
+                       make_operand(8192, 8192, g, "normal", std=1e-3), "block_channel", 128))
+        name = "config 4: block_channel + fused 128-point Hadamard fwd+bwd, 8192x8192x8192, X Student-t(3)"
+    else:
+        for m in (16, 128):
+            layers.append((make_operand(m, 4096, g, "normal"), make_operand(4096, 4096, g, "normal", std=0.02),
+                           make_operand(m, 4096, g, "normal", std=1e-3), "block_channel", None))
+        name = "config 5 (skinny part): block_channel fwd+bwd at M=16 and M=128, K=N=4096"
+    layers = [tuple(t.to(dev) if isinstance(t, torch.Tensor) else t for t in l) for l in layers]
+    ops = sum(6.0 * l[0].shape[0] * l[0].shape[1] * l[1].shape[0] for l in layers)
+
+    def step():
+        return [T.linear_fwd_bwd(*l) for l in layers]
+
+    def bf16_step():
+        return [(X @ W.t(), dY @ W, dY.t() @ X) for X, W, dY, _, _ in layers]
+
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / args.steps
+
+    dt = timed(step)
+    out = {"metric": METRIC, "value": round(ops / dt / 1e12, 2), "unit": "TOPS", "n_gpus": 1, "steps": args.steps,
+           "warmup": args.warmup, "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+           "vs_baseline": None, "dtype": "int8", "data": "synthetic", "config": {"workload": name},
+           "pct_int8_peak": round(100.0 * ops / dt / 1e12 / INT8_PEAK_TOPS, 2)}
+    if cfg == 5:   # launch-bound shapes: the same step replayed from a HIP graph
+        graphed = [T.GraphedStep(lambda x, w, dy, l=l: T.linear_fwd_bwd(x, w, dy, l[3], l[4]), *l[:3], copy_inputs=False) for l in layers]
+        out["graph_ms_per_step"] = round(timed(lambda: [gs() for gs in graphed]) * 1e3, 4)
+    with _lib.timed_launches() as rec:
+        for _ in range(args.steps):
+            step()
+    torch.cuda.synchronize()
+    out["entry_point_ms_per_step"] = {k: round(sum(a.elapsed_time(b) for a, b in ev) / args.steps, 4) for k, ev in sorted(rec.items())}
+    gemm_s = out["entry_point_ms_per_step"]["ti8_gemm_i8_nt"] * 1e-3
+    out["roofline"] = {"bound": "mfma", "achieved": round(ops / gemm_s / 1e12, 1), "peak": INT8_PEAK_TOPS, "unit": "TFLOP/s",
+                       "frac": round(ops / gemm_s / 1e12 / INT8_PEAK_TOPS, 4), "traffic": None,
+                       "note": "all GEMM launches of a step together: 6*M*N*K summed over the layers / their summed event time"}
+    out["bf16_matmul_ms_per_step"] = round(timed(bf16_step) * 1e3, 4)
+    if cfg == 5:   # the decoder layer training step of the same configuration
+        torch.manual_seed(4)
+        x = torch.randn(4, 4096, 4096, device=dev, dtype=torch.bfloat16)
+        for int8 in (True, False):
+            lay = T.decoder.DecoderLayer(4096, 32, 14336, int8=int8, device=dev)
+
+            def layer_step():
+                xi = x.clone().requires_grad_(True)
+                lay(xi).float().pow(2).mean().backward()
+            out["decoder_layer_step_ms_" + ("int8" if int8 else "bf16")] = round(timed(layer_step) * 1e3, 3)
+            del lay
+    print(json.dumps(out), flush=True)
+
+
 def event_time_ms(fn, reps):
     """Mean duration of fn() over `reps` launches, HIP events on the current stream."""
     evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
@@ -76,6 +164,7 @@ def main():
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--scheme", default="block_channel", choices=["block_channel", "row_block", "double_channel"])
+    ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5], help="benchmark configuration (2 = headline)")
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU baseline leg (profiling runs)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -88,6 +177,8 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.config != 2:
+        return other_config(args, T, dev)
     X, W, dY = (t.to(dev) for t in make_inputs())
 
     def step():
