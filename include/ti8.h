@@ -151,6 +151,22 @@ int ti8_quant_col_t(const void* x, int64_t ldx, int8_t* qT, int64_t ldqt, float*
                     int64_t R, int64_t C, int qflags, int inv_mode, ti8_stream_t stream);
 
 /* ---------------------------------------------------------------------------------
+ * Both of the above on one operand with one launch sequence: the per-row quantisation
+ * (as ti8_quant_row, group = 0) AND the per-column quantisation with transposed output
+ * (as ti8_quant_col_t), bit-identical to the two separate calls.  A training step needs
+ * both for W (triton/block_channel_fwd32.py:221-222 called with b = W for Y and with
+ * b = W^T for dX) and, in the double-channel scheme, for X and dY as well
+ * (triton/double-channle_fwd32.py:277-278 on X, W and on the transposed operands of
+ * triton/double_channel_bwd33.py:193-194); x is read twice instead of three times.
+ *
+ *   x bf16 [R][C] (ldx) -> q int8 [R][C] (ldq), s_row[R];  qT int8 [C][R] (ldqt), s_col[C]
+ *   ws: workspace of R + C floats, contents undefined afterwards.
+ * R % 128 == 0, C % 128 == 0. */
+int ti8_quant_row_col_t(const void* x, int64_t ldx, int8_t* q, int64_t ldq, float* s_row,
+                        int8_t* qT, int64_t ldqt, float* s_col, float* ws,
+                        int64_t R, int64_t C, int qflags, int inv_mode, ti8_stream_t stream);
+
+/* ---------------------------------------------------------------------------------
  * Un-normalised Walsh-Hadamard transform along the last dim (Sylvester order):
  * replaces fast_hadamard_transform.hadamard_transform at its call sites
  * (triton/double-channle_fwd32.py:273-274,299-300; triton/double_channel_bwd33.py:

@@ -116,6 +116,27 @@ def test_col_quant_transposed(T, dev):
     assert bits_equal(qT, qo) and bits_equal(s, so)
 
 
+@pytest.mark.parametrize("R,C", [(128, 128), (256, 384), (384, 4096), (1024, 14336)])
+def test_row_and_col_quant_in_one_go(T, dev, R, C):
+    """ti8_quant_row_col_t = ti8_quant_row + ti8_quant_col_t on the same operand, bit for bit (and
+    therefore equal to the oracle's per-token quantiser applied to x and to x^T)."""
+    x = randn_bf16(make_gen(R + C), R, C)
+    x[3] = 0                      # an all-zero row
+    x[:, 5] = 0                   # an all-zero column
+    x[7, 9] = 250.0               # an outlier that sets one row and one column scale
+    xd = x.to(dev)
+    for inv_mode in (0, 1):
+        q, s_row, qT, s_col = T.ops.quant_row_col_t(xd, inv_mode=inv_mode)
+        q0, s0 = T.ops.quant_row(xd, clamp=True, inv_mode=inv_mode)
+        qT0, sT0 = T.ops.quant_col_t(xd, clamp=True, inv_mode=inv_mode)
+        assert torch.equal(q, q0) and bits_equal(s_row, s0) and torch.equal(qT, qT0) and bits_equal(s_col, sT0)
+    if R * C <= 384 * 4096:
+        qo, so = obf.token_quant(x, True)
+        qTo, sTo = obf.token_quant(x.t().contiguous(), True)
+        q, s_row, qT, s_col = T.ops.quant_row_col_t(xd)
+        assert bits_equal(q, qo) and bits_equal(s_row, so.flatten()) and bits_equal(qT, qTo) and bits_equal(s_col, sTo.flatten())
+
+
 @pytest.mark.parametrize("n,cols", [(128, 384), (128, 4096), (256, 256), (512, 1536), (1024, 2048), (2048, 2048),
                                     (4096, 4096), (8192, 8192), (16384, 16384), (32768, 32768)])
 def test_fwht(T, dev, n, cols):

@@ -19,6 +19,7 @@ PROTOTYPES = {
     "ti8_quant_block_had128": [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _int, _vp],
     "ti8_quant_row": [_vp, _i64, _vp, _i64, _vp, _i64, _i64, _int, _int, _int, _vp],
     "ti8_quant_col_t": [_vp, _i64, _vp, _i64, _vp, _vp, _i64, _i64, _int, _int, _vp],
+    "ti8_quant_row_col_t": [_vp, _i64, _vp, _i64, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _int, _int, _vp],
     "ti8_fwht": [_vp, _i64, _vp, _i64, _i64, _i64, _i64, _f32, _vp],
     "ti8_gemm_i8_nt": [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64,
                        _vp, _int, _i64, _i64, _i64, _vp, _int, _i64, _i64, _i64,

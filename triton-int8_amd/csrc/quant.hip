@@ -464,6 +464,126 @@ __global__ __launch_bounds__(256) void quant_col_t_kernel(const uint16_t* __rest
     }
 }
 
+// ---------------------------------------------------------------------------------
+// Row AND column absmax of x in one read (both quantisations of an operand that a training
+// step needs: by rows for one GEMM, by columns -- transposed -- for another).  Same
+// 128 x 256 tile and thread map as col_absmax_kernel; a row of the tile is spread over the
+// 32 lanes of a half-wave, whose maxima meet through lane shuffles.
+__global__ __launch_bounds__(256) void rowcol_absmax_kernel(const uint16_t* __restrict__ x, int64_t ldx,
+                                                            unsigned int* __restrict__ ws_row,
+                                                            unsigned int* __restrict__ ws_col, int64_t R, int C) {
+    __shared__ float part[8][256];
+    const int tid = threadIdx.x;
+    const int cc = tid & 31, rg = tid >> 5;
+    const int c0 = blockIdx.x * 256 + cc * 8;
+    const int64_t r0 = (int64_t)blockIdx.y * 128;
+    float m[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    float rmax[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) rmax[i] = 0.0f;
+    if (c0 < C) {
+        uint4 v[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+            v[i] = *reinterpret_cast<const uint4*>(x + (r0 + rg + 8 * i) * ldx + c0);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const float e0 = fabsf(bf16_lo(v[i].x)), e1 = fabsf(bf16_hi(v[i].x)), e2 = fabsf(bf16_lo(v[i].y)),
+                        e3 = fabsf(bf16_hi(v[i].y)), e4 = fabsf(bf16_lo(v[i].z)), e5 = fabsf(bf16_hi(v[i].z)),
+                        e6 = fabsf(bf16_lo(v[i].w)), e7 = fabsf(bf16_hi(v[i].w));
+            m[0] = fmaxf(m[0], e0); m[1] = fmaxf(m[1], e1); m[2] = fmaxf(m[2], e2); m[3] = fmaxf(m[3], e3);
+            m[4] = fmaxf(m[4], e4); m[5] = fmaxf(m[5], e5); m[6] = fmaxf(m[6], e6); m[7] = fmaxf(m[7], e7);
+            rmax[i] = fmaxf(fmaxf(fmaxf(e0, e1), fmaxf(e2, e3)), fmaxf(fmaxf(e4, e5), fmaxf(e6, e7)));
+        }
+    }
+    // row maxima: over the 32 lanes (tid % 32) that hold the same rows
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        float a = rmax[i];
+#pragma unroll
+        for (int off = 16; off >= 1; off >>= 1) a = fmaxf(a, __shfl_xor(a, off, 64));
+        if (cc == 0) atomicMax(ws_row + r0 + rg + 8 * i, __float_as_uint(a));
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) part[rg][cc * 8 + e] = m[e];
+    __syncthreads();
+    float a = part[0][tid];
+#pragma unroll
+    for (int g = 1; g < 8; ++g) a = fmaxf(a, part[g][tid]);
+    const int c = blockIdx.x * 256 + tid;
+    if (c < C) atomicMax(ws_col + c, __float_as_uint(a));
+}
+
+// Quantise a 128x128 tile of x twice: with one scale per ROW into q (same orientation) and
+// with one scale per COLUMN into qT (transposed).  Thread <-> element map of quant_block_kernel.
+__global__ __launch_bounds__(256) void quant_rowcol_kernel(const uint16_t* __restrict__ x, int64_t ldx,
+                                                           int8_t* __restrict__ q, int64_t ldq,
+                                                           float* __restrict__ s_row, int8_t* __restrict__ qT,
+                                                           int64_t ldqt, float* __restrict__ s_col,
+                                                           const float* __restrict__ ws_row,
+                                                           const float* __restrict__ ws_col, int ncb, QMode mode) {
+    __shared__ uint32_t tileT[128 * 33];
+    const int cb = blockIdx.x % ncb;
+    const int rb = blockIdx.x / ncb;
+    const int tid = threadIdx.x;
+    const int cc = tid & 15, rg = tid >> 4;
+    const uint16_t* xt = x + (int64_t)rb * 128 * ldx + (int64_t)cb * 128;
+
+    uint4 v[2][4];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            v[h][j] = *reinterpret_cast<const uint4*>(xt + (int64_t)(h * 64 + rg * 4 + j) * ldx + cc * 8);
+
+    float cscale[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const float amax = amax_floor(ws_col[cb * 128 + cc * 8 + e], mode.eps_add);
+        cscale[e] = 127.0f / amax;
+        if (rb == 0 && rg == 0) s_col[cb * 128 + cc * 8 + e] = stored_scale(amax, cscale[e], mode);
+    }
+    int8_t* qt = q + (int64_t)rb * 128 * ldq + (int64_t)cb * 128 + cc * 8;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        uint32_t qq[4][8];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int row = h * 64 + rg * 4 + j;
+            const float amax = amax_floor(ws_row[(int64_t)rb * 128 + row], mode.eps_add);
+            const float rscale = 127.0f / amax;
+            if (cb == 0 && cc == 0) s_row[(int64_t)rb * 128 + row] = stored_scale(amax, rscale, mode);
+            const uint4& w = v[h][j];
+            *reinterpret_cast<uint2*>(qt + (int64_t)row * ldq) = quant8(w, rscale, mode.clamp);
+            qq[j][0] = q1(bf16_lo(w.x), cscale[0], mode.clamp);
+            qq[j][1] = q1(bf16_hi(w.x), cscale[1], mode.clamp);
+            qq[j][2] = q1(bf16_lo(w.y), cscale[2], mode.clamp);
+            qq[j][3] = q1(bf16_hi(w.y), cscale[3], mode.clamp);
+            qq[j][4] = q1(bf16_lo(w.z), cscale[4], mode.clamp);
+            qq[j][5] = q1(bf16_hi(w.z), cscale[5], mode.clamp);
+            qq[j][6] = q1(bf16_lo(w.w), cscale[6], mode.clamp);
+            qq[j][7] = q1(bf16_hi(w.w), cscale[7], mode.clamp);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            tileT[(cc * 8 + e) * 33 + h * 16 + rg] =
+                qq[0][e] | (qq[1][e] << 8) | (qq[2][e] << 16) | (qq[3][e] << 24);
+    }
+    __syncthreads();
+    int8_t* qtt = qT + (int64_t)cb * 128 * ldqt + (int64_t)rb * 128;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const int tr = p * 32 + (tid >> 3);
+        const int tc = tid & 7;
+        uint4 w;
+        w.x = tileT[tr * 33 + tc * 4 + 0];
+        w.y = tileT[tr * 33 + tc * 4 + 1];
+        w.z = tileT[tr * 33 + tc * 4 + 2];
+        w.w = tileT[tr * 33 + tc * 4 + 3];
+        *reinterpret_cast<uint4*>(qtt + (int64_t)tr * ldqt + tc * 16) = w;
+    }
+}
+
 static int parse_mode(int qflags, int inv_mode, QMode* m) {
     if (qflags & ~(TI8_Q_CLAMP | TI8_Q_EPS_ADD | TI8_Q_SCALE_BF16 | TI8_Q_HAD128)) return fail(TI8_ERR_MODE, "unknown quantiser flag 0x%x", qflags);
     if (inv_mode < 0 || inv_mode > 3) return fail(TI8_ERR_MODE, "unknown inv_mode %d", inv_mode);
@@ -569,6 +689,32 @@ extern "C" int ti8_quant_col_t(const void* x, int64_t ldx, int8_t* qT, int64_t l
     hipLaunchKernelGGL(quant_col_t_kernel, dim3((unsigned)ntiles), dim3(256), 0, st, xp, ldx, qT, ldqt, s, ws,
                        (int)(C / 128), mode);
     return check_launch("ti8_quant_col_t");
+}
+
+extern "C" int ti8_quant_row_col_t(const void* x, int64_t ldx, int8_t* q, int64_t ldq, float* s_row, int8_t* qT,
+                                   int64_t ldqt, float* s_col, float* ws, int64_t R, int64_t C, int qflags,
+                                   int inv_mode, ti8_stream_t stream) {
+    const char* fn = "ti8_quant_row_col_t";
+    QMode mode;
+    if (int e = parse_mode(qflags, inv_mode, &mode)) return e;
+    if (qflags & TI8_Q_HAD128) return fail(TI8_ERR_MODE, "%s: the Hadamard rotation is not offered here", fn);
+    if (!x || !q || !s_row || !qT || !s_col || !ws) return fail(TI8_ERR_NULL, "%s: x, q, s_row, qT, s_col and ws are required", fn);
+    if (R <= 0 || C <= 0 || R % 128 || C % 128 || C > 0x7fffffffLL)
+        return fail(TI8_ERR_SHAPE, "%s: need R%%128==0 and C%%128==0; got R=%lld C=%lld", fn, (long long)R, (long long)C);
+    if (ldx < C || ldq < C || ldqt < R) return fail(TI8_ERR_SHAPE, "%s: leading dimension smaller than the row length", fn);
+    if (!aligned16(x) || !aligned16(q) || !aligned16(qT) || (ldx % 8) || (ldq % 16) || (ldqt % 16))
+        return fail(TI8_ERR_ALIGN, "%s: pointers must be 16-byte aligned and strides multiples of 16 bytes", fn);
+    const int64_t ntiles = (R / 128) * (C / 128);
+    if (ntiles > 0x7fffffffLL || R / 128 > 65535 || R + C > 0x7fffffffLL) return fail(TI8_ERR_SHAPE, "%s: too many tiles", fn);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uint16_t* xp = static_cast<const uint16_t*>(x);
+    unsigned int* wsu = reinterpret_cast<unsigned int*>(ws);   // [R row maxima][C column maxima]
+    hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((R + C + 255) / 256)), dim3(256), 0, st, wsu, (int)(R + C), 0u);
+    hipLaunchKernelGGL(rowcol_absmax_kernel, dim3((unsigned)((C + 255) / 256), (unsigned)(R / 128)), dim3(256), 0, st, xp,
+                       ldx, wsu, wsu + R, R, (int)C);
+    hipLaunchKernelGGL(quant_rowcol_kernel, dim3((unsigned)ntiles), dim3(256), 0, st, xp, ldx, q, ldq, s_row, qT, ldqt,
+                       s_col, ws, ws + R, (int)(C / 128), mode);
+    return check_launch(fn);
 }
 
 extern "C" int ti8_quant_block_had128(const void* x, int64_t bsx, int64_t ldx, int8_t* q, int64_t bsq, int64_t ldq,

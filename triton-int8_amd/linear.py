@@ -60,9 +60,24 @@ def _gemm_dc(a_q, a_s, b_q, b_s, post_scale=0.0):
                           post_scale=post_scale)[0]
 
 
-def linear_forward(X2, W, scheme="block_channel", hadamard=None):
+# Quantise an operand by rows and by columns in one launch sequence (ops.quant_row_col_t) where a
+# step needs both; False falls back to separate quant_row / quant_col_t calls (same bits).
+FUSE_ROW_COL = True
+
+
+def _row_col(x, **kw):
+    if FUSE_ROW_COL:
+        return ops.quant_row_col_t(x, **kw)
+    q, s = ops.quant_row(x, **kw)
+    qT, sT = ops.quant_col_t(x, **kw)
+    return q, s, qT, sT
+
+
+def linear_forward(X2, W, scheme="block_channel", hadamard=None, need_backward=True):
     """X2 bf16 [T, K] (tokens flattened), W bf16 [N, K] -> (Y bf16 [T, N], saved) where
-    ``saved`` holds what the backward can reuse (quantised X^T and its scales)."""
+    ``saved`` holds what the backward can reuse: operands the forward quantises anyway are
+    quantised for the backward GEMMs in the same pass (transposed copies, column-wise scales)
+    unless ``need_backward`` is false."""
     _check(scheme, hadamard)
     saved = {}
     if scheme == "block_channel":
@@ -70,9 +85,13 @@ def linear_forward(X2, W, scheme="block_channel", hadamard=None):
             q, s = ops.quant_block_had128(X2[None], clamp=True)
             wq, ws = ops.quant_row(W, clamp=True, hadamard128=True)
             return _gemm_bc(q[0], s[0], SCALE_BLOCK128, wq, ws, SCALE_ROW, 2.0 ** -7), saved
+        if not need_backward:
+            q, s = ops.quant_block(X2[None], clamp=True)
+            wq, ws = ops.quant_row(W, clamp=True)
+            return _gemm_bc(q[0], s[0], SCALE_BLOCK128, wq, ws, SCALE_ROW), saved
         q, qT, s = ops.quant_block(X2[None], clamp=True, with_transpose=True)
         saved["XqT"], saved["Xs"] = qT[0], s[0]
-        wq, ws = ops.quant_row(W, clamp=True)
+        wq, ws, saved["WtQ"], saved["Wts"] = _row_col(W, clamp=True)   # rows for Y, columns for dX
         return _gemm_bc(q[0], s[0], SCALE_BLOCK128, wq, ws, SCALE_ROW), saved
     if scheme == "row_block":
         q, s = ops.quant_row(X2, clamp=True, hadamard128=(hadamard == 128))
@@ -88,8 +107,12 @@ def linear_forward(X2, W, scheme="block_channel", hadamard=None):
         q, s = ops.quant_row(ops.fwht(X2), clamp=True, inv_mode=INV_AMAX_DIV_127)
         wq, ws = ops.quant_row(ops.fwht(W), clamp=True, inv_mode=INV_AMAX_DIV_127)
         return _gemm_dc(q, s, wq, ws, 1.0 / K), saved
-    q, s = ops.quant_row(X2, clamp=True, inv_mode=INV_AMAX_DIV_127)
-    wq, ws = ops.quant_row(W, clamp=True, inv_mode=INV_AMAX_DIV_127)
+    if not need_backward:
+        q, s = ops.quant_row(X2, clamp=True, inv_mode=INV_AMAX_DIV_127)
+        wq, ws = ops.quant_row(W, clamp=True, inv_mode=INV_AMAX_DIV_127)
+        return _gemm_dc(q, s, wq, ws), saved
+    q, s, saved["XtQ"], saved["Xts"] = _row_col(X2, clamp=True, inv_mode=INV_AMAX_DIV_127)
+    wq, ws, saved["WtQ"], saved["Wts"] = _row_col(W, clamp=True, inv_mode=INV_AMAX_DIV_127)
     return _gemm_dc(q, s, wq, ws), saved
 
 
@@ -112,7 +135,10 @@ def linear_backward(dY2, X2, W, scheme="block_channel", hadamard=None, saved=Non
                                 out_scale=2.0 ** -7)[0]
             return dX, dW
         dq, dqT, ds = ops.quant_block(dY2[None], clamp=True, with_transpose=True)
-        wtq, wts = ops.quant_col_t(W, clamp=True)                    # W^T [K,N] per row
+        if "WtQ" in saved:
+            wtq, wts = saved["WtQ"], saved["Wts"]
+        else:
+            wtq, wts = ops.quant_col_t(W, clamp=True)                # W^T [K,N] per row
         dX = _gemm_bc(dq[0], ds[0], SCALE_BLOCK128, wtq, wts, SCALE_ROW)
         if "XqT" in saved:
             xqT, xs = saved["XqT"], saved["Xs"]
@@ -131,14 +157,13 @@ def linear_backward(dY2, X2, W, scheme="block_channel", hadamard=None, saved=Non
             xtq, xts = ops.quant_block_had128(X2[None], along_rows=True, clamp=True)
             dW = _gemm_bc(dytq, dyts, SCALE_ROW, xtq[0], xts[0].t(), SCALE_BLOCK128, 2.0 ** -7)
             return dX, dW
-        dq, ds = ops.quant_row(dY2, clamp=True)
+        dq, ds, dytq, dyts = _row_col(dY2, clamp=True)    # rows for dX, columns (dY^T [N,T] per row) for dW
         if "WqT" in saved:
             wqT, ws = saved["WqT"], saved["Ws"]
         else:
             _, wqT3, ws3 = ops.quant_block(W[None], clamp=True, with_transpose=True)
             wqT, ws = wqT3[0], ws3[0]
         dX = _gemm_bc(dq, ds, SCALE_ROW, wqT, ws.t(), SCALE_BLOCK128)
-        dytq, dyts = ops.quant_col_t(dY2, clamp=True)                # dY^T [N,T] per row
         _, xqT, xs = ops.quant_block(X2[None], clamp=True, with_transpose=True)
         dW = _gemm_bc(dytq, dyts, SCALE_ROW, xqT[0], xs[0].t(), SCALE_BLOCK128)
         return dX, dW
@@ -151,11 +176,16 @@ def linear_backward(dY2, X2, W, scheme="block_channel", hadamard=None, saved=Non
         xtq, xts = ops.quant_row(ops.fwht(X2.t().contiguous()), clamp=True, inv_mode=INV_AMAX_DIV_127)
         dW = _gemm_dc(dytq, dyts, xtq, xts, 1.0 / T)
         return dX, dW
-    dq, ds = ops.quant_row(dY2, clamp=True, inv_mode=INV_AMAX_DIV_127)
-    wtq, wts = ops.quant_col_t(W, clamp=True, inv_mode=INV_AMAX_DIV_127)
+    dq, ds, dytq, dyts = _row_col(dY2, clamp=True, inv_mode=INV_AMAX_DIV_127)
+    if "WtQ" in saved:
+        wtq, wts = saved["WtQ"], saved["Wts"]
+    else:
+        wtq, wts = ops.quant_col_t(W, clamp=True, inv_mode=INV_AMAX_DIV_127)
     dX = _gemm_dc(dq, ds, wtq, wts)
-    dytq, dyts = ops.quant_col_t(dY2, clamp=True, inv_mode=INV_AMAX_DIV_127)
-    xtq, xts = ops.quant_col_t(X2, clamp=True, inv_mode=INV_AMAX_DIV_127)
+    if "XtQ" in saved:
+        xtq, xts = saved["XtQ"], saved["Xts"]
+    else:
+        xtq, xts = ops.quant_col_t(X2, clamp=True, inv_mode=INV_AMAX_DIV_127)
     dW = _gemm_dc(dytq, dyts, xtq, xts)
     return dX, dW
 
@@ -197,7 +227,8 @@ class Int8LinearFunction(torch.autograd.Function):
         x2 = x.reshape(-1, K)
         ctx.tokens = x2.shape[0]
         x2 = pad_tokens(x2)
-        y, saved = linear_forward(x2, weight, scheme, hadamard)
+        need_bwd = any(ctx.needs_input_grad[:2])
+        y, saved = linear_forward(x2, weight, scheme, hadamard, need_backward=need_bwd)
         ctx.scheme, ctx.hadamard, ctx.saved_q = scheme, hadamard, saved
         ctx.has_bias = bias is not None
         ctx.save_for_backward(x2, weight)

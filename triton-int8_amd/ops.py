@@ -12,7 +12,7 @@ from ._lib import (COMBINE_DIV_PROD, COMBINE_MUL_MUL, COMBINE_MUL_PROD, GEMM_SKI
                    INV_AMAX_MUL_RCP127, INV_MULTIPLIER, INV_RCP_OF_SCALE, Q_CLAMP, Q_EPS_ADD, Q_HAD128, Q_SCALE_BF16,
                    SCALE_BLOCK128, SCALE_BLOCK_K256, SCALE_ROW, SCALE_ROW_K128)
 
-__all__ = ["quant_block", "quant_block_had128", "quant_row", "quant_col_t", "fwht", "gemm_i8_nt", "gemm_i8_nt_i32"]
+__all__ = ["quant_block", "quant_block_had128", "quant_row", "quant_col_t", "quant_row_col_t", "fwht", "gemm_i8_nt", "gemm_i8_nt_i32"]
 
 
 # Which GEMM kernel `gemm_i8_nt` asks for: "auto" (the few-rows kernel for M <= 256, else the
@@ -150,6 +150,26 @@ def quant_col_t(x, *, clamp=True, inv_mode=INV_RCP_OF_SCALE):
     _lib.call("ti8_quant_col_t", x.data_ptr(), x.stride(0), qT.data_ptr(), R, s.data_ptr(), ws.data_ptr(), R, C,
               _qflags(clamp, False, False), inv_mode, _stream())
     return qT, s
+
+
+def quant_row_col_t(x, *, clamp=True, inv_mode=INV_RCP_OF_SCALE):
+    """Per-row AND per-column (transposed) quantisation of x [R, C] in one go:
+    returns (q [R, C], s_row [R], qT [C, R], s_col [C]), the same bits as
+    ``quant_row(x)`` and ``quant_col_t(x)``."""
+    _check_bf16(x, "x")
+    _need(x.dim() == 2, "x must be [R, C]")
+    R, C = x.shape
+    _need(R % 128 == 0 and C % 128 == 0, f"R and C must be multiples of 128, got {R} x {C}")
+    if x.stride(1) != 1 or x.stride(0) % 8 or x.data_ptr() % 16:
+        x = x.contiguous()
+    q = torch.empty((R, C), dtype=torch.int8, device=x.device)
+    qT = torch.empty((C, R), dtype=torch.int8, device=x.device)
+    s_row = torch.empty((R,), dtype=torch.float32, device=x.device)
+    s_col = torch.empty((C,), dtype=torch.float32, device=x.device)
+    ws = torch.empty((R + C,), dtype=torch.float32, device=x.device)
+    _lib.call("ti8_quant_row_col_t", x.data_ptr(), x.stride(0), q.data_ptr(), C, s_row.data_ptr(), qT.data_ptr(), R,
+              s_col.data_ptr(), ws.data_ptr(), R, C, _qflags(clamp, False, False), inv_mode, _stream())
+    return q, s_row, qT, s_col
 
 
 def fwht(x, n=None, scale=1.0):
