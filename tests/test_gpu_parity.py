@@ -304,6 +304,26 @@ def test_autograd_module(T, dev, gemm_path):
     assert rel_err(lin.bias.grad, dy.float().sum((0, 1)).cpu()) <= REL_TOL
 
 
+@pytest.mark.parametrize("scheme,h", [("block_channel", None), ("block_channel", 128), ("row_block", None),
+                                      ("row_block", 128), ("double_channel", None), ("double_channel", "full")])
+def test_forward_only_path_caches_the_quantised_weight(T, dev, scheme, h):
+    """Without autograd the module quantises its weight once and reuses it: same bits as the
+    training forward, and the cache follows in-place weight updates."""
+    g = make_gen(77)
+    lin = T.Int8Linear(512, 256, bias=True, scheme=scheme, hadamard=h, device=dev)
+    x = randn_bf16(g, 3, 50, 512).to(dev)
+    y_train = lin(x.clone().requires_grad_(True)).detach()
+    with torch.no_grad():
+        y1 = lin(x)
+        key = lin._wq_key
+        y2 = lin(x)
+        assert lin._wq_key == key and torch.equal(y1, y2) and torch.equal(y1, y_train)
+        lin.weight.mul_(0.5)                                  # an optimiser step in miniature
+        y3 = lin(x)
+        assert lin._wq_key != key
+    assert torch.equal(y3, lin(x.clone().requires_grad_(True)).detach())
+
+
 @pytest.mark.parametrize("tokens", [16, 100, 128, 300])
 def test_skinny_and_ragged_token_counts(T, dev, tokens, gemm_path):
     """Zero-pad semantics for M that is not a multiple of the 128-row tile (config 5's M = 16)."""

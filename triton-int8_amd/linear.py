@@ -30,7 +30,7 @@ import torch
 from . import ops
 from ._lib import (COMBINE_MUL_MUL, INV_AMAX_DIV_127, INV_RCP_OF_SCALE, SCALE_BLOCK128, SCALE_ROW)
 
-__all__ = ["linear_forward", "linear_backward", "linear_fwd_bwd", "pad_tokens", "Int8LinearFunction", "Int8Linear", "SCHEMES"]
+__all__ = ["quantize_weight", "linear_forward", "linear_backward", "linear_fwd_bwd", "pad_tokens", "Int8LinearFunction", "Int8Linear", "SCHEMES"]
 
 SCHEMES = ("block_channel", "row_block", "double_channel")
 
@@ -73,21 +73,38 @@ def _row_col(x, **kw):
     return q, s, qT, sT
 
 
-def linear_forward(X2, W, scheme="block_channel", hadamard=None, need_backward=True):
+def quantize_weight(W, scheme="block_channel", hadamard=None):
+    """The forward GEMM's view of W [N, K]: ``(Wq int8 [N, K], scales)`` in the scheme's layout (per
+    output channel, or 128x128 blocks for "row_block"; rotated first when ``hadamard`` asks).
+    A forward-only caller (inference) computes it once per weight update and hands it to
+    :func:`linear_forward` as ``wq``."""
+    _check(scheme, hadamard)
+    if scheme == "block_channel":
+        return ops.quant_row(W, clamp=True, hadamard128=(hadamard == 128))
+    if scheme == "row_block":
+        wq, ws = ops.quant_block_had128(W[None], clamp=True) if hadamard == 128 else ops.quant_block(W[None], clamp=True)
+        return wq[0], ws[0]
+    return ops.quant_row(ops.fwht(W) if hadamard == "full" else W, clamp=True, inv_mode=INV_AMAX_DIV_127)
+
+
+def linear_forward(X2, W, scheme="block_channel", hadamard=None, need_backward=True, wq=None):
     """X2 bf16 [T, K] (tokens flattened), W bf16 [N, K] -> (Y bf16 [T, N], saved) where
     ``saved`` holds what the backward can reuse: operands the forward quantises anyway are
     quantised for the backward GEMMs in the same pass (transposed copies, column-wise scales)
-    unless ``need_backward`` is false."""
+    unless ``need_backward`` is false.  ``wq`` = :func:`quantize_weight` of W computed earlier
+    (forward-only use; W itself is then not read)."""
     _check(scheme, hadamard)
     saved = {}
+    if wq is not None and need_backward:
+        raise ValueError("a pre-quantised weight serves the forward only")
     if scheme == "block_channel":
         if hadamard == 128:
             q, s = ops.quant_block_had128(X2[None], clamp=True)
-            wq, ws = ops.quant_row(W, clamp=True, hadamard128=True)
+            wq, ws = wq if wq is not None else quantize_weight(W, scheme, hadamard)
             return _gemm_bc(q[0], s[0], SCALE_BLOCK128, wq, ws, SCALE_ROW, 2.0 ** -7), saved
         if not need_backward:
             q, s = ops.quant_block(X2[None], clamp=True)
-            wq, ws = ops.quant_row(W, clamp=True)
+            wq, ws = wq if wq is not None else quantize_weight(W, scheme, hadamard)
             return _gemm_bc(q[0], s[0], SCALE_BLOCK128, wq, ws, SCALE_ROW), saved
         q, qT, s = ops.quant_block(X2[None], clamp=True, with_transpose=True)
         saved["XqT"], saved["Xs"] = qT[0], s[0]
@@ -95,22 +112,18 @@ def linear_forward(X2, W, scheme="block_channel", hadamard=None, need_backward=T
         return _gemm_bc(q[0], s[0], SCALE_BLOCK128, wq, ws, SCALE_ROW), saved
     if scheme == "row_block":
         q, s = ops.quant_row(X2, clamp=True, hadamard128=(hadamard == 128))
-        if hadamard == 128:
-            wq, ws = ops.quant_block_had128(W[None], clamp=True)
-            return _gemm_bc(q, s, SCALE_ROW, wq[0], ws[0], SCALE_BLOCK128, 2.0 ** -7), saved
+        if hadamard == 128 or not need_backward:
+            wq, ws = wq if wq is not None else quantize_weight(W, scheme, hadamard)
+            return _gemm_bc(q, s, SCALE_ROW, wq, ws, SCALE_BLOCK128, 2.0 ** -7 if hadamard == 128 else 1.0), saved
         wq, wqT, ws = ops.quant_block(W[None], clamp=True, with_transpose=True)
         saved["WqT"], saved["Ws"] = wqT[0], ws[0]
         return _gemm_bc(q, s, SCALE_ROW, wq[0], ws[0], SCALE_BLOCK128), saved
     # double_channel
     K = X2.shape[1]
-    if hadamard == "full":
-        q, s = ops.quant_row(ops.fwht(X2), clamp=True, inv_mode=INV_AMAX_DIV_127)
-        wq, ws = ops.quant_row(ops.fwht(W), clamp=True, inv_mode=INV_AMAX_DIV_127)
-        return _gemm_dc(q, s, wq, ws, 1.0 / K), saved
-    if not need_backward:
-        q, s = ops.quant_row(X2, clamp=True, inv_mode=INV_AMAX_DIV_127)
-        wq, ws = ops.quant_row(W, clamp=True, inv_mode=INV_AMAX_DIV_127)
-        return _gemm_dc(q, s, wq, ws), saved
+    if hadamard == "full" or not need_backward:
+        q, s = ops.quant_row(ops.fwht(X2) if hadamard == "full" else X2, clamp=True, inv_mode=INV_AMAX_DIV_127)
+        wq, ws = wq if wq is not None else quantize_weight(W, scheme, hadamard)
+        return _gemm_dc(q, s, wq, ws, 1.0 / K if hadamard == "full" else 0.0), saved
     q, s, saved["XtQ"], saved["Xts"] = _row_col(X2, clamp=True, inv_mode=INV_AMAX_DIV_127)
     wq, ws, saved["WtQ"], saved["Wts"] = _row_col(W, clamp=True, inv_mode=INV_AMAX_DIV_127)
     return _gemm_dc(q, s, wq, ws), saved
@@ -263,9 +276,23 @@ class Int8Linear(torch.nn.Module):
         self.weight = torch.nn.Parameter(torch.empty(out_features, in_features, device=device, dtype=dtype))
         self.bias = torch.nn.Parameter(torch.zeros(out_features, device=device, dtype=dtype)) if bias else None
         torch.nn.init.normal_(self.weight, std=0.02)
+        self._wq, self._wq_key = None, None   # quantised weight of the forward-only path and what it was made from
 
     def forward(self, x):
-        return Int8LinearFunction.apply(x, self.weight, self.bias, self.scheme, self.hadamard)
+        if torch.is_grad_enabled() and (x.requires_grad or self.weight.requires_grad):
+            return Int8LinearFunction.apply(x, self.weight, self.bias, self.scheme, self.hadamard)
+        # forward only (inference): the weight is quantised once per weight update, not per call
+        key = (self.weight._version, self.weight.data_ptr(), self.scheme, self.hadamard)
+        if self._wq_key != key:
+            self._wq, self._wq_key = quantize_weight(self.weight.detach(), self.scheme, self.hadamard), key
+        K = x.shape[-1]
+        x2 = x.reshape(-1, K)
+        tokens = x2.shape[0]
+        y, _ = linear_forward(pad_tokens(x2), None, self.scheme, self.hadamard, need_backward=False, wq=self._wq)
+        y = y[:tokens]
+        if self.bias is not None:
+            y = y + self.bias
+        return y.reshape(*x.shape[:-1], self.out_features)
 
     def extra_repr(self):
         return f"in_features={self.in_features}, out_features={self.out_features}, scheme={self.scheme}, hadamard={self.hadamard}"
