@@ -227,7 +227,7 @@ def main():
 
     # HBM-side bytes per GEMM launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled on the device
     # copy above (profiles/bench_config2_block_channel_hbm_counters.md); measured for this scheme only
-    traffic = 324650225 if args.scheme == "block_channel" else None
+    traffic = 324716454 if args.scheme == "block_channel" else None
 
     out = {
         "metric": METRIC, "value": round(tops, 2), "unit": "TOPS", "n_gpus": 1, "steps": args.steps,
