@@ -432,6 +432,8 @@ static int check_operands(const char* fn, const void* A, int64_t bsa, int64_t ld
     if (M > 0x3fffffff || N > 0x3fffffff || K > 0x3fffffff || batch > 65535)
         return fail(TI8_ERR_SHAPE, "%s: dimension too large", fn);
     if (lda < K || ldb < K || ldc < N) return fail(TI8_ERR_SHAPE, "%s: leading dimension smaller than the row length", fn);
+    // the kernels keep 8 * ld in 32-bit lane offsets
+    if (lda > 0x0fffffff || ldb > 0x0fffffff) return fail(TI8_ERR_SHAPE, "%s: leading dimension of A or B too large", fn);
     if (!aligned16(A) || !aligned16(B) || (lda % 16) || (ldb % 16) || (bsa % 16) || (bsb % 16))
         return fail(TI8_ERR_ALIGN, "%s: A and B must be 16-byte aligned with strides multiples of 16", fn);
     return TI8_OK;
