@@ -480,12 +480,27 @@ extern "C" int ti8_gemm_i8_nt(const int8_t* A, int64_t bsa, int64_t lda, const i
     // few rows: too few 256-row tiles to fill the machine, take the kernel that splits N and K finer
     const bool want_skinny = (gemm_flags & TI8_GEMM_SKINNY) || (!(gemm_flags & TI8_GEMM_TILED) && M <= 256);
     if (want_skinny && !a.strict && skinny_supported(a)) return launch_skinny(a, batch, acc_i32_full != 0, st);
-    if (acc_i32_full) return launch<256, 256, 2, 4, EPI_ROWS>(a, batch, st);
+    // Medium sizes: when the large tiles would leave CUs without a workgroup, use 128 x 128 tiles
+    // (4 waves of 64 x 64, two workgroups per CU): four (two) times as many workgroups.
+    static int num_cu = 0;
+    if (num_cu == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        (void)hipGetDevice(&dev);
+        num_cu = (hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
+    }
+    const int64_t tiles_256x256 = ((M + 255) / 256) * ((N + 255) / 256) * batch;
+    const int64_t tiles_256x128 = ((M + 255) / 256) * (N / 128) * batch;
+    if (acc_i32_full) {
+        if (tiles_256x256 < num_cu) return launch<128, 128, 2, 2, EPI_ROWS>(a, batch, st);
+        return launch<256, 256, 2, 4, EPI_ROWS>(a, batch, st);
+    }
     // the fast promotion keeps at most 256 per-K-tile factors in registers and cannot apply a
     // factor that varies per row of A inside the loop: those cases take the literal kernel
     const bool a_loop_per_row = (modeA == TI8_SCALE_ROW_K128);
     if (a.strict || a_loop_per_row || K > 256 * 128) return launch<128, 128, 2, 2, EPI_STRICT>(a, batch, st);
     if (modeB == TI8_SCALE_ROW_K128) return launch<256, 128, 4, 2, EPI_PROMOTE_LANE>(a, batch, st);
+    if (tiles_256x128 < num_cu) return launch<128, 128, 2, 2, EPI_PROMOTE>(a, batch, st);
     return launch<256, 128, 4, 2, EPI_PROMOTE>(a, batch, st);
 }
 
