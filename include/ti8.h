@@ -193,7 +193,10 @@ int ti8_fwht(const void* x, int64_t ldx, void* y, int64_t ldy,
  *       C = bf16(f32(C) * post_scale) follows (the reference's `C * inv_K`).
  *   acc_i32_full = 0: per 128-deep K block, exact int32 dot d, then `combine`;
  *       C = bf16(acc * out_scale) (out_scale = 1 for none).
- * M, N, K multiples of 128. */
+ * N, K multiples of 128.  M a multiple of 128, or any multiple of 32 up to 256 (decode
+ * shapes: only the first M rows of a quantised, zero-padded operand are multiplied; block
+ * scales are indexed by row / 128 as usual).  Those M are served by the few-rows kernel
+ * only, i.e. not with TI8_GEMM_STRICT / TI8_GEMM_TILED, TI8_SCALE_ROW_K128 or K > 32768. */
 int ti8_gemm_i8_nt(const int8_t* A, int64_t bsa, int64_t lda,
                    const int8_t* B, int64_t bsb, int64_t ldb,
                    void* C, int64_t bsc, int64_t ldc,

@@ -38,7 +38,7 @@ def _expand(s, mode, rows, kb):
     """Scale of every row of a 2-D operand at K block ``kb`` as an fp32 vector."""
     if mode == ROW:
         return s.reshape(rows).to(F32)
-    return s[:, kb].to(F32).repeat_interleave(128)
+    return s[:, kb].to(F32).repeat_interleave(128)[:rows]   # row r uses block r // 128 (rows need not fill the last block)
 
 
 def gemm_scaled(Aq, sA, modeA, Bq, sB, modeB, out_scale=None, out_dtype=torch.bfloat16):

@@ -424,10 +424,10 @@ static int launch(const GemmArgs& a0, int64_t batch, hipStream_t st) {
 }
 
 static int check_operands(const char* fn, const void* A, int64_t bsa, int64_t lda, const void* B, int64_t bsb, int64_t ldb,
-                          const void* C, int64_t ldc, int64_t batch, int64_t M, int64_t N, int64_t K) {
+                          const void* C, int64_t ldc, int64_t batch, int64_t M, int64_t N, int64_t K, int m_step = 128) {
     if (!A || !B || !C) return fail(TI8_ERR_NULL, "%s: A, B and C are required", fn);
-    if (batch <= 0 || M <= 0 || N <= 0 || K <= 0 || K % 128 || M % 128 || N % 128)
-        return fail(TI8_ERR_SHAPE, "%s: need batch>0 and M, N, K positive multiples of 128; got batch=%lld M=%lld N=%lld K=%lld",
+    if (batch <= 0 || M <= 0 || N <= 0 || K <= 0 || K % 128 || M % m_step || N % 128)
+        return fail(TI8_ERR_SHAPE, "%s: need batch>0 and M, N, K positive multiples of 128 (M: of 32 up to 256 rows); got batch=%lld M=%lld N=%lld K=%lld",
                     fn, (long long)batch, (long long)M, (long long)N, (long long)K);
     if (M > 0x3fffffff || N > 0x3fffffff || K > 0x3fffffff || batch > 65535)
         return fail(TI8_ERR_SHAPE, "%s: dimension too large", fn);
@@ -455,7 +455,8 @@ extern "C" int ti8_gemm_i8_nt(const int8_t* A, int64_t bsa, int64_t lda, const i
                               int64_t sb_ks, int64_t batch, int64_t M, int64_t N, int64_t K, int acc_i32_full,
                               int combine, float out_scale, float post_scale, int gemm_flags, ti8_stream_t stream) {
     const char* fn = "ti8_gemm_i8_nt";
-    if (int e = check_operands(fn, A, bsa, lda, B, bsb, ldb, C, ldc, batch, M, N, K)) return e;
+    // up to 256 rows M may be any multiple of 32 (decode shapes): only the few-rows kernel takes those
+    if (int e = check_operands(fn, A, bsa, lda, B, bsb, ldb, C, ldc, batch, M, N, K, M <= 256 ? 32 : 128)) return e;
     if (int e = check_scale(fn, "A", sA, modeA)) return e;
     if (int e = check_scale(fn, "B", sB, modeB)) return e;
     if (combine < 0 || combine > 2) return fail(TI8_ERR_MODE, "%s: unknown combine %d", fn, combine);
@@ -480,6 +481,9 @@ extern "C" int ti8_gemm_i8_nt(const int8_t* A, int64_t bsa, int64_t lda, const i
     // few rows: too few 256-row tiles to fill the machine, take the kernel that splits N and K finer
     const bool want_skinny = (gemm_flags & TI8_GEMM_SKINNY) || (!(gemm_flags & TI8_GEMM_TILED) && M <= 256);
     if (want_skinny && !a.strict && skinny_supported(a)) return launch_skinny(a, batch, acc_i32_full != 0, st);
+    if (M % 128)
+        return fail(TI8_ERR_SHAPE, "%s: M = %lld is not a multiple of 128, which only the few-rows kernel accepts "
+                    "(not with TI8_GEMM_STRICT / TI8_GEMM_TILED, per-(row, K tile) scales or K > 32768)", fn, (long long)M);
     // Medium sizes: when the large tiles would leave CUs without a workgroup, use 128 x 128 tiles
     // (4 waves of 64 x 64, two workgroups per CU): four (two) times as many workgroups.
     static int num_cu = 0;

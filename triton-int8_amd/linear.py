@@ -48,15 +48,28 @@ def _h128(x2d):
     return ops.fwht(x2d, 128)
 
 
-def _gemm_bc(a_q, a_s, a_mode, b_q, b_s, b_mode, out_scale=1.0):
+def _live_rows(a_q, tokens):
+    """Rows of the (zero-padded, 128-row-quantised) token operand that the GEMM has to multiply:
+    with few tokens the GEMM takes any multiple of 32 rows, and the padding rows are zeros whose
+    products nobody reads."""
+    rows = a_q.shape[0]
+    if tokens is None or rows > 256 or ops.GEMM_PATH == "tiled" or a_q.shape[1] > 32768:
+        return rows
+    return min(rows, -(-tokens // 32) * 32)
+
+
+def _gemm_bc(a_q, a_s, a_mode, b_q, b_s, b_mode, out_scale=1.0, tokens=None):
     """2-D operands through the batched block-channel GEMM (batch of one)."""
-    a_s3 = a_s.reshape(1, -1) if a_mode == SCALE_ROW else a_s[None]
+    rows = _live_rows(a_q, tokens)
+    a_q = a_q[:rows]
+    a_s3 = a_s[:rows].reshape(1, -1) if a_mode == SCALE_ROW else a_s[None]
     return ops.gemm_i8_nt(a_q[None], b_q, a_s3, a_mode, b_s, b_mode, combine=COMBINE_MUL_MUL,
                           out_scale=out_scale)[0]
 
 
-def _gemm_dc(a_q, a_s, b_q, b_s, post_scale=0.0):
-    return ops.gemm_i8_nt(a_q[None], b_q, a_s.reshape(1, -1), SCALE_ROW, b_s, SCALE_ROW, acc_i32_full=True,
+def _gemm_dc(a_q, a_s, b_q, b_s, post_scale=0.0, tokens=None):
+    rows = _live_rows(a_q, tokens)
+    return ops.gemm_i8_nt(a_q[:rows][None], b_q, a_s[:rows].reshape(1, -1), SCALE_ROW, b_s, SCALE_ROW, acc_i32_full=True,
                           post_scale=post_scale)[0]
 
 
@@ -87,12 +100,13 @@ def quantize_weight(W, scheme="block_channel", hadamard=None):
     return ops.quant_row(ops.fwht(W) if hadamard == "full" else W, clamp=True, inv_mode=INV_AMAX_DIV_127)
 
 
-def linear_forward(X2, W, scheme="block_channel", hadamard=None, need_backward=True, wq=None):
+def linear_forward(X2, W, scheme="block_channel", hadamard=None, need_backward=True, wq=None, tokens=None):
     """X2 bf16 [T, K] (tokens flattened), W bf16 [N, K] -> (Y bf16 [T, N], saved) where
     ``saved`` holds what the backward can reuse: operands the forward quantises anyway are
     quantised for the backward GEMMs in the same pass (transposed copies, column-wise scales)
     unless ``need_backward`` is false.  ``wq`` = :func:`quantize_weight` of W computed earlier
-    (forward-only use; W itself is then not read)."""
+    (forward-only use; W itself is then not read).  ``tokens`` = number of real rows of X2 when the
+    caller has zero-padded it: with few tokens the GEMM skips the padding rows."""
     _check(scheme, hadamard)
     saved = {}
     if wq is not None and need_backward:
@@ -101,35 +115,35 @@ def linear_forward(X2, W, scheme="block_channel", hadamard=None, need_backward=T
         if hadamard == 128:
             q, s = ops.quant_block_had128(X2[None], clamp=True)
             wq, ws = wq if wq is not None else quantize_weight(W, scheme, hadamard)
-            return _gemm_bc(q[0], s[0], SCALE_BLOCK128, wq, ws, SCALE_ROW, 2.0 ** -7), saved
+            return _gemm_bc(q[0], s[0], SCALE_BLOCK128, wq, ws, SCALE_ROW, 2.0 ** -7, tokens=tokens), saved
         if not need_backward:
             q, s = ops.quant_block(X2[None], clamp=True)
             wq, ws = wq if wq is not None else quantize_weight(W, scheme, hadamard)
-            return _gemm_bc(q[0], s[0], SCALE_BLOCK128, wq, ws, SCALE_ROW), saved
+            return _gemm_bc(q[0], s[0], SCALE_BLOCK128, wq, ws, SCALE_ROW, tokens=tokens), saved
         q, qT, s = ops.quant_block(X2[None], clamp=True, with_transpose=True)
         saved["XqT"], saved["Xs"] = qT[0], s[0]
         wq, ws, saved["WtQ"], saved["Wts"] = _row_col(W, clamp=True)   # rows for Y, columns for dX
-        return _gemm_bc(q[0], s[0], SCALE_BLOCK128, wq, ws, SCALE_ROW), saved
+        return _gemm_bc(q[0], s[0], SCALE_BLOCK128, wq, ws, SCALE_ROW, tokens=tokens), saved
     if scheme == "row_block":
         q, s = ops.quant_row(X2, clamp=True, hadamard128=(hadamard == 128))
         if hadamard == 128 or not need_backward:
             wq, ws = wq if wq is not None else quantize_weight(W, scheme, hadamard)
-            return _gemm_bc(q, s, SCALE_ROW, wq, ws, SCALE_BLOCK128, 2.0 ** -7 if hadamard == 128 else 1.0), saved
+            return _gemm_bc(q, s, SCALE_ROW, wq, ws, SCALE_BLOCK128, 2.0 ** -7 if hadamard == 128 else 1.0, tokens=tokens), saved
         wq, wqT, ws = ops.quant_block(W[None], clamp=True, with_transpose=True)
         saved["WqT"], saved["Ws"] = wqT[0], ws[0]
-        return _gemm_bc(q, s, SCALE_ROW, wq[0], ws[0], SCALE_BLOCK128), saved
+        return _gemm_bc(q, s, SCALE_ROW, wq[0], ws[0], SCALE_BLOCK128, tokens=tokens), saved
     # double_channel
     K = X2.shape[1]
     if hadamard == "full" or not need_backward:
         q, s = ops.quant_row(ops.fwht(X2) if hadamard == "full" else X2, clamp=True, inv_mode=INV_AMAX_DIV_127)
         wq, ws = wq if wq is not None else quantize_weight(W, scheme, hadamard)
-        return _gemm_dc(q, s, wq, ws, 1.0 / K if hadamard == "full" else 0.0), saved
+        return _gemm_dc(q, s, wq, ws, 1.0 / K if hadamard == "full" else 0.0, tokens=tokens), saved
     q, s, saved["XtQ"], saved["Xts"] = _row_col(X2, clamp=True, inv_mode=INV_AMAX_DIV_127)
     wq, ws, saved["WtQ"], saved["Wts"] = _row_col(W, clamp=True, inv_mode=INV_AMAX_DIV_127)
-    return _gemm_dc(q, s, wq, ws), saved
+    return _gemm_dc(q, s, wq, ws, tokens=tokens), saved
 
 
-def linear_backward(dY2, X2, W, scheme="block_channel", hadamard=None, saved=None):
+def linear_backward(dY2, X2, W, scheme="block_channel", hadamard=None, saved=None, tokens=None):
     """dY2 bf16 [T, N], X2 bf16 [T, K], W bf16 [N, K] -> (dX bf16 [T, K], dW bf16 [N, K])."""
     _check(scheme, hadamard)
     saved = saved or {}
@@ -140,7 +154,7 @@ def linear_backward(dY2, X2, W, scheme="block_channel", hadamard=None, saved=Non
             # H_128 along N for dX, along the tokens for dW: two differently rotated copies
             dq, ds = ops.quant_block_had128(dY2[None], clamp=True)
             wtq, wts = ops.quant_row(W.t().contiguous(), clamp=True, hadamard128=True)   # weights: small
-            dX = _gemm_bc(dq[0], ds[0], SCALE_BLOCK128, wtq, wts, SCALE_ROW, 2.0 ** -7)
+            dX = _gemm_bc(dq[0], ds[0], SCALE_BLOCK128, wtq, wts, SCALE_ROW, 2.0 ** -7, tokens=tokens)
             # the token-dim rotation is fused too: one read of dY / X, transposed int8 out
             dyt, dyts = ops.quant_block_had128(dY2[None], along_rows=True, clamp=False)
             xt, xts = ops.quant_block_had128(X2[None], along_rows=True, clamp=False)
@@ -152,7 +166,7 @@ def linear_backward(dY2, X2, W, scheme="block_channel", hadamard=None, saved=Non
             wtq, wts = saved["WtQ"], saved["Wts"]
         else:
             wtq, wts = ops.quant_col_t(W, clamp=True)                # W^T [K,N] per row
-        dX = _gemm_bc(dq[0], ds[0], SCALE_BLOCK128, wtq, wts, SCALE_ROW)
+        dX = _gemm_bc(dq[0], ds[0], SCALE_BLOCK128, wtq, wts, SCALE_ROW, tokens=tokens)
         if "XqT" in saved:
             xqT, xs = saved["XqT"], saved["Xs"]
         else:
@@ -165,7 +179,7 @@ def linear_backward(dY2, X2, W, scheme="block_channel", hadamard=None, saved=Non
         if hadamard == 128:
             dq, ds = ops.quant_row(dY2, clamp=True, hadamard128=True)
             wtq, wts = ops.quant_block_had128(W[None], along_rows=True, clamp=True)      # W^T [K,N], groups along N
-            dX = _gemm_bc(dq, ds, SCALE_ROW, wtq[0], wts[0].t(), SCALE_BLOCK128, 2.0 ** -7)
+            dX = _gemm_bc(dq, ds, SCALE_ROW, wtq[0], wts[0].t(), SCALE_BLOCK128, 2.0 ** -7, tokens=tokens)
             dytq, dyts = ops.quant_row(dY2.t().contiguous(), clamp=True, hadamard128=True)
             xtq, xts = ops.quant_block_had128(X2[None], along_rows=True, clamp=True)
             dW = _gemm_bc(dytq, dyts, SCALE_ROW, xtq[0], xts[0].t(), SCALE_BLOCK128, 2.0 ** -7)
@@ -176,7 +190,7 @@ def linear_backward(dY2, X2, W, scheme="block_channel", hadamard=None, saved=Non
         else:
             _, wqT3, ws3 = ops.quant_block(W[None], clamp=True, with_transpose=True)
             wqT, ws = wqT3[0], ws3[0]
-        dX = _gemm_bc(dq, ds, SCALE_ROW, wqT, ws.t(), SCALE_BLOCK128)
+        dX = _gemm_bc(dq, ds, SCALE_ROW, wqT, ws.t(), SCALE_BLOCK128, tokens=tokens)
         _, xqT, xs = ops.quant_block(X2[None], clamp=True, with_transpose=True)
         dW = _gemm_bc(dytq, dyts, SCALE_ROW, xqT[0], xs[0].t(), SCALE_BLOCK128)
         return dX, dW
@@ -184,7 +198,7 @@ def linear_backward(dY2, X2, W, scheme="block_channel", hadamard=None, saved=Non
     if hadamard == "full":
         dq, ds = ops.quant_row(ops.fwht(dY2), clamp=True, inv_mode=INV_AMAX_DIV_127)
         wtq, wts = ops.quant_row(ops.fwht(W.t().contiguous()), clamp=True, inv_mode=INV_AMAX_DIV_127)
-        dX = _gemm_dc(dq, ds, wtq, wts, 1.0 / N)
+        dX = _gemm_dc(dq, ds, wtq, wts, 1.0 / N, tokens=tokens)
         dytq, dyts = ops.quant_row(ops.fwht(dY2.t().contiguous()), clamp=True, inv_mode=INV_AMAX_DIV_127)
         xtq, xts = ops.quant_row(ops.fwht(X2.t().contiguous()), clamp=True, inv_mode=INV_AMAX_DIV_127)
         dW = _gemm_dc(dytq, dyts, xtq, xts, 1.0 / T)
@@ -194,7 +208,7 @@ def linear_backward(dY2, X2, W, scheme="block_channel", hadamard=None, saved=Non
         wtq, wts = saved["WtQ"], saved["Wts"]
     else:
         wtq, wts = ops.quant_col_t(W, clamp=True, inv_mode=INV_AMAX_DIV_127)
-    dX = _gemm_dc(dq, ds, wtq, wts)
+    dX = _gemm_dc(dq, ds, wtq, wts, tokens=tokens)
     if "XtQ" in saved:
         xtq, xts = saved["XtQ"], saved["Xts"]
     else:
@@ -226,8 +240,8 @@ def linear_fwd_bwd(X, W, dY, scheme="block_channel", hadamard=None):
     X2, dY2 = X.reshape(-1, K), dY.reshape(-1, N)
     T = X2.shape[0]
     X2, dY2 = pad_tokens(X2), pad_tokens(dY2)
-    Y, saved = linear_forward(X2, W, scheme, hadamard)
-    dX, dW = linear_backward(dY2, X2, W, scheme, hadamard, saved)
+    Y, saved = linear_forward(X2, W, scheme, hadamard, tokens=T)
+    dX, dW = linear_backward(dY2, X2, W, scheme, hadamard, saved, tokens=T)
     return Y[:T].reshape(*lead, N), dX[:T].reshape(*lead, K), dW
 
 
@@ -241,7 +255,7 @@ class Int8LinearFunction(torch.autograd.Function):
         ctx.tokens = x2.shape[0]
         x2 = pad_tokens(x2)
         need_bwd = any(ctx.needs_input_grad[:2])
-        y, saved = linear_forward(x2, weight, scheme, hadamard, need_backward=need_bwd)
+        y, saved = linear_forward(x2, weight, scheme, hadamard, need_backward=need_bwd, tokens=ctx.tokens)
         ctx.scheme, ctx.hadamard, ctx.saved_q = scheme, hadamard, saved
         ctx.has_bias = bias is not None
         ctx.save_for_backward(x2, weight)
@@ -255,7 +269,7 @@ class Int8LinearFunction(torch.autograd.Function):
         x2, weight = ctx.saved_tensors
         N = weight.shape[0]
         dy2 = pad_tokens(dy.reshape(-1, N).contiguous())
-        dx, dw = linear_backward(dy2, x2, weight, ctx.scheme, ctx.hadamard, ctx.saved_q)
+        dx, dw = linear_backward(dy2, x2, weight, ctx.scheme, ctx.hadamard, ctx.saved_q, tokens=ctx.tokens)
         db = dy2.sum(dim=0).to(dy.dtype) if ctx.has_bias else None
         return dx[:ctx.tokens].reshape(*dy.shape[:-1], x2.shape[1]), dw, db, None, None
 
@@ -288,7 +302,7 @@ class Int8Linear(torch.nn.Module):
         K = x.shape[-1]
         x2 = x.reshape(-1, K)
         tokens = x2.shape[0]
-        y, _ = linear_forward(pad_tokens(x2), None, self.scheme, self.hadamard, need_backward=False, wq=self._wq)
+        y, _ = linear_forward(pad_tokens(x2), None, self.scheme, self.hadamard, need_backward=False, wq=self._wq, tokens=tokens)
         y = y[:tokens]
         if self.bias is not None:
             y = y + self.bias

@@ -203,11 +203,11 @@ def _scale_desc(s, mode, rows, nkb, batch, batched, who):
         v = s.reshape(shape)
         return v, (v.stride(0) if batched else 0), v.stride(-1), 0
     if mode == SCALE_BLOCK128:
-        shape = (rows // 128, nkb)
+        shape = (-(-rows // 128), nkb)
     elif mode == SCALE_ROW_K128:
         shape = (rows, nkb)
     else:
-        shape = (rows // 128, nkb // 2)
+        shape = (-(-rows // 128), nkb // 2)
     full = ((batch,) + shape) if batched else shape
     _need(tuple(s.shape) == full or (not batched and tuple(s.shape) == (1,) + shape),
           f"{who} scale must have shape {full}, got {tuple(s.shape)}")
@@ -224,8 +224,8 @@ def gemm_i8_nt(A, B, sA, modeA, sB, modeB, *, acc_i32_full=False, combine=COMBIN
     N = B.shape[-2]
     _need(B.shape[-1] == K, f"K mismatch: A has {K}, B has {B.shape[-1]}")
     _need(B.dim() == 2 or B.shape[0] == batch, "batch mismatch between A and B")
-    _need(M % 128 == 0 and N % 128 == 0 and K % 128 == 0 and batch > 0,
-          f"M, N, K must be positive multiples of 128, got M={M} N={N} K={K}")
+    _need((M % 128 == 0 or (M % 32 == 0 and M <= 256)) and N % 128 == 0 and K % 128 == 0 and batch > 0,
+          f"N, K must be positive multiples of 128 and M one of 128 (of 32 up to 256 rows), got M={M} N={N} K={K}")
     A, B = _k_contig(A), _k_contig(B)
     nkb = K // 128
     sAv, sa_bs, sa_rs, sa_ks = _scale_desc(sA, modeA, M, nkb, batch, True, "A")
