@@ -146,7 +146,10 @@ int ti8_quant_row(const void* x, int64_t ldx, int8_t* q, int64_t ldq, float* s,
  *
  *   x bf16 [R][C] (ldx) -> qT int8 [C][R] (ldqt), s[C]
  *   ws: workspace of C floats (column absmax), contents undefined afterwards.
- * R % 128 == 0, C % 128 == 0. */
+ * R % 128 == 0, C % 128 == 0.
+ * With TI8_Q_HAD128 every 128-row segment of every column is rotated by H_128 first (x^T rotated
+ * along its contraction dim, the rule of ti8_quant_row's flag applied to x^T): the
+ * hadamard = 128 mode of dX = dY W, whose second operand is W^T per row. */
 int ti8_quant_col_t(const void* x, int64_t ldx, int8_t* qT, int64_t ldqt, float* s, float* ws,
                     int64_t R, int64_t C, int qflags, int inv_mode, ti8_stream_t stream);
 

@@ -166,6 +166,20 @@ def test_fused_hadamard_quantisers(T, dev):
     assert bits_equal(q, qo) and bits_equal(s, so.flatten())
 
 
+@pytest.mark.parametrize("R,C", [(128, 128), (384, 256), (1024, 512)])
+def test_col_quant_transposed_with_rotation(T, dev, R, C):
+    """quant_col_t(hadamard128) = the rotated per-row quantiser applied to x^T, without the transpose."""
+    x = randn_bf16(make_gen(R * 3 + C), R, C)
+    x[:, 3] = 0
+    x[5, 9] = 100.0
+    xd = x.to(dev)
+    qT, s = T.ops.quant_col_t(xd, hadamard128=True)
+    q0, s0 = T.ops.quant_row(xd.t().contiguous(), clamp=True, hadamard128=True)
+    assert torch.equal(qT, q0) and bits_equal(s, s0)
+    qo, so = obf.token_quant(ohad.hadamard128(x.t().contiguous(), -1), True)
+    assert bits_equal(qT, qo) and bits_equal(s, so.flatten())
+
+
 def test_int32_accumulators_bit_exact(T, dev):
     g = make_gen(6)
     A = torch.randint(-127, 128, (2, 384, 1024), generator=g, dtype=torch.int8)

@@ -225,10 +225,19 @@ __global__ __launch_bounds__(256) void quant_block_kernel(
 // picks up 8 consecutive ROWS of one column, after which the same code runs on the transposed
 // tile and q comes out transposed, [C][R] -- the K-contiguous operand of a GEMM that contracts
 // over the rows (tokens).
-template <bool ALONG_ROWS>
+// SCALE selects the quantisation group: HAD_BLOCK = the 128 x 128 tile (one scale per tile);
+// HAD_COLMAX / HAD_COL (ALONG_ROWS only) = a whole column of the rotated operand, i.e. a whole row
+// of the transposed output, in two launches: HAD_COLMAX only merges the tile's column maxima
+// into ws[C] (atomic max on the float bits), HAD_COL quantises with the scales that ws then
+// holds and writes them to s[C].
+enum { HAD_BLOCK = 0, HAD_COLMAX = 1, HAD_COL = 2 };
+
+template <bool ALONG_ROWS, int SCALE = HAD_BLOCK>
 __global__ __launch_bounds__(256) void quant_block_had_kernel(
     const uint16_t* __restrict__ x, int64_t bsx, int64_t ldx, int8_t* __restrict__ q, int64_t bsq, int64_t ldq,
-    float* __restrict__ s, int64_t ssb, int64_t ssr, int64_t ssc, int nrb, int ncb, QMode mode) {
+    float* __restrict__ s, int64_t ssb, int64_t ssr, int64_t ssc, int nrb, int ncb, QMode mode,
+    unsigned int* __restrict__ ws = nullptr) {
+    static_assert(SCALE == HAD_BLOCK || ALONG_ROWS, "column-wise scales go with the rotation along rows");
     __shared__ float red4[4];
     __shared__ __attribute__((aligned(16))) uint16_t tile[ALONG_ROWS ? 128 * 128 : 8];
 
@@ -275,6 +284,30 @@ __global__ __launch_bounds__(256) void quant_block_had_kernel(
             }
     }
     const int lane = tid & 63;
+    if (SCALE != HAD_BLOCK) {
+        // this thread holds, per (h, j), 8 consecutive rows of column h*64 + rg*4 + j of the tile;
+        // the 16 lanes with the same rg hold the other rows of that column
+        int8_t* qcol = q + (int64_t)cb * 128 * ldq + (int64_t)rb * 128 + cc * 8;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int col = cb * 128 + h * 64 + rg * 4 + j;
+                const uint4 r = fwht128_bf16(v[h][j], lane);
+                if (SCALE == HAD_COLMAX) {
+                    float m = absmax8(r, 0.0f);
+#pragma unroll
+                    for (int off = 8; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+                    if (cc == 0) atomicMax(ws + col, __float_as_uint(m));
+                } else {
+                    const float amax = amax_floor(__uint_as_float(ws[col]), mode.eps_add);
+                    const float scale = 127.0f / amax;
+                    if (rb == 0 && cc == 0) s[col] = stored_scale(amax, scale, mode);
+                    *reinterpret_cast<uint2*>(qcol + (int64_t)(h * 64 + rg * 4 + j) * ldq) = quant8(r, scale, mode.clamp);
+                }
+            }
+        return;
+    }
     float amax = 0.0f;
 #pragma unroll
     for (int h = 0; h < 2; ++h)
@@ -671,7 +704,6 @@ extern "C" int ti8_quant_col_t(const void* x, int64_t ldx, int8_t* qT, int64_t l
                                int64_t R, int64_t C, int qflags, int inv_mode, ti8_stream_t stream) {
     QMode mode;
     if (int e = parse_mode(qflags, inv_mode, &mode)) return e;
-    if (qflags & TI8_Q_HAD128) return fail(TI8_ERR_MODE, "ti8_quant_col_t: the Hadamard rotation is not offered here");
     if (!x || !qT || !s || !ws) return fail(TI8_ERR_NULL, "ti8_quant_col_t: x, qT, s and ws are required");
     if (R <= 0 || C <= 0 || R % 128 || C % 128 || C > 0x7fffffffLL)
         return fail(TI8_ERR_SHAPE, "ti8_quant_col_t: need R%%128==0 and C%%128==0; got R=%lld C=%lld", (long long)R, (long long)C);
@@ -684,6 +716,16 @@ extern "C" int ti8_quant_col_t(const void* x, int64_t ldx, int8_t* qT, int64_t l
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     unsigned int* wsu = reinterpret_cast<unsigned int*>(ws);
     hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((C + 255) / 256)), dim3(256), 0, st, wsu, (int)C, 0u);
+    if (qflags & TI8_Q_HAD128) {
+        // rotate every 128-row segment of every column first (x^T rotated along its contraction
+        // dim): both passes redo the rotation on the tile they read instead of storing it
+        const int nrb = (int)(R / 128), ncb = (int)(C / 128);
+        hipLaunchKernelGGL((quant_block_had_kernel<true, HAD_COLMAX>), dim3((unsigned)ntiles), dim3(256), 0, st, xp, (int64_t)0, ldx,
+                           qT, (int64_t)0, ldqt, s, (int64_t)0, (int64_t)0, (int64_t)0, nrb, ncb, mode, wsu);
+        hipLaunchKernelGGL((quant_block_had_kernel<true, HAD_COL>), dim3((unsigned)ntiles), dim3(256), 0, st, xp, (int64_t)0, ldx,
+                           qT, (int64_t)0, ldqt, s, (int64_t)0, (int64_t)0, (int64_t)0, nrb, ncb, mode, wsu);
+        return check_launch("ti8_quant_col_t");
+    }
     hipLaunchKernelGGL(col_absmax_kernel, dim3((unsigned)((C + 255) / 256), (unsigned)(R / 128)), dim3(256), 0, st, xp,
                        ldx, wsu, R, (int)C);
     hipLaunchKernelGGL(quant_col_t_kernel, dim3((unsigned)ntiles), dim3(256), 0, st, xp, ldx, qT, ldqt, s, ws,

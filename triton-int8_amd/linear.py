@@ -153,7 +153,7 @@ def linear_backward(dY2, X2, W, scheme="block_channel", hadamard=None, saved=Non
         if hadamard == 128:
             # H_128 along N for dX, along the tokens for dW: two differently rotated copies
             dq, ds = ops.quant_block_had128(dY2[None], clamp=True)
-            wtq, wts = ops.quant_row(W.t().contiguous(), clamp=True, hadamard128=True)   # weights: small
+            wtq, wts = ops.quant_col_t(W, clamp=True, hadamard128=True)   # W^T [K,N] per row, rotated along N
             dX = _gemm_bc(dq[0], ds[0], SCALE_BLOCK128, wtq, wts, SCALE_ROW, 2.0 ** -7, tokens=tokens)
             # the token-dim rotation is fused too: one read of dY / X, transposed int8 out
             dyt, dyts = ops.quant_block_had128(dY2[None], along_rows=True, clamp=False)

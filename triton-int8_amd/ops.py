@@ -135,9 +135,11 @@ def quant_row(x, *, clamp=True, group=0, eps_add=False, scale_bf16=False, inv_mo
     return q.reshape(*lead, cols), s.reshape(*lead, cols // 128) if group else s.reshape(*lead)
 
 
-def quant_col_t(x, *, clamp=True, inv_mode=INV_RCP_OF_SCALE):
+def quant_col_t(x, *, clamp=True, inv_mode=INV_RCP_OF_SCALE, hadamard128=False):
     """Per-column absmax quantisation of ``x`` [R, C] with transposed output: the per-row
-    quantiser applied to ``x.T``.  Returns ``(qT int8 [C, R], s fp32 [C])``."""
+    quantiser applied to ``x.T``.  Returns ``(qT int8 [C, R], s fp32 [C])``.
+    ``hadamard128`` rotates every group of 128 rows by H_128 first (= ``quant_row(x.T, hadamard128=True)``
+    without the bf16 transpose)."""
     _check_bf16(x, "x")
     _need(x.dim() == 2, "x must be [R, C]")
     R, C = x.shape
@@ -148,7 +150,7 @@ def quant_col_t(x, *, clamp=True, inv_mode=INV_RCP_OF_SCALE):
     s = torch.empty((C,), dtype=torch.float32, device=x.device)
     ws = torch.empty((C,), dtype=torch.float32, device=x.device)
     _lib.call("ti8_quant_col_t", x.data_ptr(), x.stride(0), qT.data_ptr(), R, s.data_ptr(), ws.data_ptr(), R, C,
-              _qflags(clamp, False, False), inv_mode, _stream())
+              _qflags(clamp, False, False) | (Q_HAD128 if hadamard128 else 0), inv_mode, _stream())
     return qT, s
 
 
