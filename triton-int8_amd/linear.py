@@ -180,7 +180,7 @@ def linear_backward(dY2, X2, W, scheme="block_channel", hadamard=None, saved=Non
             dq, ds = ops.quant_row(dY2, clamp=True, hadamard128=True)
             wtq, wts = ops.quant_block_had128(W[None], along_rows=True, clamp=True)      # W^T [K,N], groups along N
             dX = _gemm_bc(dq, ds, SCALE_ROW, wtq[0], wts[0].t(), SCALE_BLOCK128, 2.0 ** -7, tokens=tokens)
-            dytq, dyts = ops.quant_row(dY2.t().contiguous(), clamp=True, hadamard128=True)
+            dytq, dyts = ops.quant_col_t(dY2, clamp=True, hadamard128=True)   # dY^T [N,T] per row, rotated along the tokens
             xtq, xts = ops.quant_block_had128(X2[None], along_rows=True, clamp=True)
             dW = _gemm_bc(dytq, dyts, SCALE_ROW, xtq[0], xts[0].t(), SCALE_BLOCK128, 2.0 ** -7)
             return dX, dW
