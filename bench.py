@@ -226,8 +226,8 @@ def main():
     bf16_ms = sum(event_time_ms(f, args.steps) for f in bf16_fns)
 
     # HBM-side bytes per GEMM launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled on the device
-    # copy above (profiles/bench_config2_block_channel_hbm_counters.md); measured for this scheme only
-    traffic = 324716454 if args.scheme == "block_channel" else None
+    # copy above (profiles/bench_config2_*_hbm_counters.md); measured for these two schemes
+    traffic = {"block_channel": 324716454, "double_channel": 257920121}.get(args.scheme)
 
     out = {
         "metric": METRIC, "value": round(tops, 2), "unit": "TOPS", "n_gpus": 1, "steps": args.steps,
