@@ -29,10 +29,11 @@ def T():
     return triton_int8_amd
 
 
-@pytest.fixture(params=["tiled", "skinny"])
+@pytest.fixture(params=["tiled", "large", "skinny"])
 def gemm_path(request, T):
-    """Run the case through the LDS-tiled GEMM kernel and through the few-rows kernel (the default
-    picks by M, and most cases here are small enough to land on the few-rows one only)."""
+    """Run the case through the LDS-tiled GEMM kernels (tiles sized to the shape, and the 256 x 256
+    tiles that large shapes get) and through the few-rows kernel: the default picks by shape, and
+    most cases here are small enough to land on the few-rows kernel only."""
     old = T.ops.GEMM_PATH
     T.ops.GEMM_PATH = request.param
     yield request.param
@@ -249,6 +250,7 @@ def test_few_rows_kernel(T, dev, M, N, K):
     args = (Ad, Bd, sa_row.to(dev), SCALE_ROW, sb_row.to(dev), SCALE_ROW)
     got = run("skinny", *args, acc_i32_full=True)
     assert bits_equal(got, want) and (not tiled_ok or torch.equal(got, run("tiled", *args, acc_i32_full=True)))
+    assert not tiled_ok or torch.equal(got, run("large", *args, acc_i32_full=True))
     # promotion per 128-deep K block: every mix of row / block scales, shared and batched B
     for sA, mA, oA in ((sa_blk, SCALE_BLOCK128, olin.BLOCK), (sa_row, SCALE_ROW, olin.ROW)):
         for Bq, sB, mB, oB in ((B, sb_row, SCALE_ROW, olin.ROW), (B, sb_blk, SCALE_BLOCK128, olin.BLOCK),
@@ -261,6 +263,7 @@ def test_few_rows_kernel(T, dev, M, N, K):
             got = run("skinny", *args)
             assert rel_err(got, want) <= 1e-4          # fp32 association only; the bar is REL_TOL
             assert not tiled_ok or rel_err(run("tiled", *args), want) <= 1e-4
+            assert not tiled_ok or rel_err(run("large", *args), want) <= 1e-4
     if not tiled_ok:
         with pytest.raises(T._lib.Ti8Error, match="few-rows"):
             run("tiled", Ad, Bd, sa_row.to(dev), SCALE_ROW, sb_row.to(dev), SCALE_ROW, acc_i32_full=True)

@@ -50,7 +50,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
     constexpr int A_INSTR = BM / 8 / NW;  // global->LDS wave instructions per K tile per wave
     constexpr int B_INSTR = BN / 8 / NW;
     constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128;
-    constexpr bool FAST = (EPI == EPI_PROMOTE || EPI == EPI_PROMOTE_LANE);
+    constexpr bool CHAIN = (EPI == EPI_PROMOTE_CHAIN);
+    constexpr bool FAST = (EPI == EPI_PROMOTE || EPI == EPI_PROMOTE_LANE || CHAIN);
     constexpr bool LANEB = (EPI == EPI_PROMOTE_LANE);
     constexpr bool PROMOTE = (FAST || EPI == EPI_STRICT);
     static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "tile/wave mismatch");
@@ -260,6 +261,85 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
     __syncthreads();
     const int klast = (nk - 1) * 128;  // loads past the last K tile re-read it into a free buffer: no branches in the loop
     issue_tile_loads<A_INSTR>(baseA + min(128, klast), strideA8, voffA, tA0, wA + A_BYTES);
+    if constexpr (CHAIN) {
+        // Promotion without int32 accumulators that outlive a K tile: a 32 x 32 block's four MFMAs of
+        // a K tile chain into a temporary (two blocks of one block row interleaved, so that
+        // dependent MFMAs are two issues apart), which is folded into the float accumulators
+        // right away.  Only the float accumulators persist, which is what lets a wave own
+        // 128 x 64 (8 blocks = 128 VGPRs) instead of 64 x 64: a third fewer LDS reads and L2->LDS
+        // bytes per MFMA.  Registers: A fragments of one block row (4 k-steps) + the next row's
+        // being read, B fragments of both block columns for the whole K tile, two temporaries.
+        v4i fa[2][4], fbv[TN][4];
+        static_assert(!CHAIN || TN == 2, "two block columns per wave");
+        auto read_a = [&](int buf, const int8_t* stage_a, int i) {
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) fa[buf][ks] = *reinterpret_cast<const v4i*>(stage_a + a_row_off + i * 4096 + choff[ks]);
+        };
+        auto read_b = [&](const int8_t* stage_b, int ks) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j) fbv[j][ks] = *reinterpret_cast<const v4i*>(stage_b + b_row_off + j * 4096 + choff[ks]);
+        };
+        auto fold = [&](int i, const v16i& d0, const v16i& d1) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) accf[PROMOTE ? i : 0][0][r] = __builtin_fmaf(static_cast<float>(d0[r]), f_cur, accf[PROMOTE ? i : 0][0][r]);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) accf[PROMOTE ? i : 0][PROMOTE ? 1 : 0][r] = __builtin_fmaf(static_cast<float>(d1[r]), f_cur, accf[PROMOTE ? i : 0][PROMOTE ? 1 : 0][r]);
+        };
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) read_b(ldsB, ks);
+        read_a(0, ldsA, 0);
+        for (int kt = 0; kt < nk; ++kt) {
+            const int cur = kt & 1;
+            const int8_t* stA = ldsA + cur * A_BYTES;
+            const int8_t* stAn = ldsA + (cur ^ 1) * A_BYTES;
+            const int8_t* stBn = ldsB + (cur ^ 1) * B_BYTES;
+            load_factors(kt);
+            issue_tile_loads<B_INSTR>(baseB + min((kt + 1) * 128, klast), strideB8, voffB, tB0, wB + (cur ^ 1) * B_BYTES);
+#pragma unroll
+            for (int i = 0; i < TM - 1; ++i) {
+                read_a((i + 1) & 1, stA, i + 1);
+                __builtin_amdgcn_sched_barrier(0);
+                v16i d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i & 1][0], fbv[0][0], vzero, 0, 0, 0);
+                v16i d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i & 1][0], fbv[1][0], vzero, 0, 0, 0);
+#pragma unroll
+                for (int ks = 1; ks < 4; ++ks) {
+                    d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i & 1][ks], fbv[0][ks], d0, 0, 0, 0);
+                    d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i & 1][ks], fbv[1][ks], d1, 0, 0, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                fold(i, d0, d1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // last block row: tile kt+1 has landed, its fragments replace those of tile kt as they retire
+            __builtin_amdgcn_s_waitcnt(0);
+            __syncthreads();
+            issue_tile_loads<A_INSTR>(baseA + min((kt + 2) * 128, klast), strideA8, voffA, tA0, wA + cur * A_BYTES);
+            constexpr int LB = (TM - 1) & 1;   // buffer that holds the last block row
+            read_a(LB ^ 1, stAn, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            v16i d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[LB][0], fbv[0][0], vzero, 0, 0, 0);
+            v16i d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[LB][0], fbv[1][0], vzero, 0, 0, 0);
+            d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[LB][1], fbv[0][1], d0, 0, 0, 0);
+            d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[LB][1], fbv[1][1], d1, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            read_b(stBn, 0);
+            read_b(stBn, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[LB][2], fbv[0][2], d0, 0, 0, 0);
+            d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[LB][2], fbv[1][2], d1, 0, 0, 0);
+            d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[LB][3], fbv[0][3], d0, 0, 0, 0);
+            d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[LB][3], fbv[1][3], d1, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            read_b(stBn, 2);
+            read_b(stBn, 3);
+            __builtin_amdgcn_sched_barrier(0);
+            fold(TM - 1, d0, d1);
+            __builtin_amdgcn_sched_barrier(0);
+            // the next tile starts with block row 0 in buffer LB ^ 1; with an even number of block
+            // rows per wave that is buffer 0 again
+            static_assert(!CHAIN || ((TM - 1) & 1) == 1, "an even number of block rows keeps the A buffers in phase");
+        }
+    } else {
     load_frags(0, ldsA + a_row_off, ldsB + b_row_off, 0);
 
     auto ktile = [&](int kt) {
@@ -322,6 +402,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
                     }
             }
         }
+    }
     }
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
@@ -460,8 +541,9 @@ extern "C" int ti8_gemm_i8_nt(const int8_t* A, int64_t bsa, int64_t lda, const i
     if (int e = check_scale(fn, "A", sA, modeA)) return e;
     if (int e = check_scale(fn, "B", sB, modeB)) return e;
     if (combine < 0 || combine > 2) return fail(TI8_ERR_MODE, "%s: unknown combine %d", fn, combine);
-    if (gemm_flags & ~(TI8_GEMM_STRICT | TI8_GEMM_TILED | TI8_GEMM_SKINNY)) return fail(TI8_ERR_MODE, "%s: unknown flag 0x%x", fn, gemm_flags);
-    if ((gemm_flags & TI8_GEMM_TILED) && (gemm_flags & TI8_GEMM_SKINNY)) return fail(TI8_ERR_MODE, "%s: TI8_GEMM_TILED and TI8_GEMM_SKINNY exclude each other", fn);
+    if (gemm_flags & ~(TI8_GEMM_STRICT | TI8_GEMM_TILED | TI8_GEMM_SKINNY | TI8_GEMM_LARGE_TILES)) return fail(TI8_ERR_MODE, "%s: unknown flag 0x%x", fn, gemm_flags);
+    if ((gemm_flags & TI8_GEMM_SKINNY) && (gemm_flags & (TI8_GEMM_TILED | TI8_GEMM_LARGE_TILES)))
+        return fail(TI8_ERR_MODE, "%s: TI8_GEMM_SKINNY excludes TI8_GEMM_TILED and TI8_GEMM_LARGE_TILES", fn);
     if (acc_i32_full && (modeA != TI8_SCALE_ROW || modeB != TI8_SCALE_ROW))
         return fail(TI8_ERR_MODE, "%s: int32 accumulation over the whole K needs per-row scales on both operands", fn);
     if ((modeA == TI8_SCALE_BLOCK_K256 || modeB == TI8_SCALE_BLOCK_K256) && (K % 256))
@@ -479,7 +561,8 @@ extern "C" int ti8_gemm_i8_nt(const int8_t* A, int64_t bsa, int64_t lda, const i
     a.out_scale = out_scale; a.post_scale = post_scale;
     hipStream_t st = static_cast<hipStream_t>(stream);
     // few rows: too few 256-row tiles to fill the machine, take the kernel that splits N and K finer
-    const bool want_skinny = (gemm_flags & TI8_GEMM_SKINNY) || (!(gemm_flags & TI8_GEMM_TILED) && M <= 256);
+    const bool large = (gemm_flags & TI8_GEMM_LARGE_TILES) != 0;
+    const bool want_skinny = (gemm_flags & TI8_GEMM_SKINNY) || (!(gemm_flags & (TI8_GEMM_TILED | TI8_GEMM_LARGE_TILES)) && M <= 256);
     if (want_skinny && !a.strict && skinny_supported(a)) return launch_skinny(a, batch, acc_i32_full != 0, st);
     if (M % 128)
         return fail(TI8_ERR_SHAPE, "%s: M = %lld is not a multiple of 128, which only the few-rows kernel accepts "
@@ -496,7 +579,7 @@ extern "C" int ti8_gemm_i8_nt(const int8_t* A, int64_t bsa, int64_t lda, const i
     const int64_t tiles_256x256 = ((M + 255) / 256) * ((N + 255) / 256) * batch;
     const int64_t tiles_256x128 = ((M + 255) / 256) * (N / 128) * batch;
     if (acc_i32_full) {
-        if (tiles_256x256 < num_cu) return launch<128, 128, 2, 2, EPI_ROWS>(a, batch, st);
+        if (!large && tiles_256x256 < num_cu) return launch<128, 128, 2, 2, EPI_ROWS>(a, batch, st);
         return launch<256, 256, 2, 4, EPI_ROWS>(a, batch, st);
     }
     // the fast promotion keeps at most 256 per-K-tile factors in registers and cannot apply a
@@ -504,8 +587,11 @@ extern "C" int ti8_gemm_i8_nt(const int8_t* A, int64_t bsa, int64_t lda, const i
     const bool a_loop_per_row = (modeA == TI8_SCALE_ROW_K128);
     if (a.strict || a_loop_per_row || K > 256 * 128) return launch<128, 128, 2, 2, EPI_STRICT>(a, batch, st);
     if (modeB == TI8_SCALE_ROW_K128) return launch<256, 128, 4, 2, EPI_PROMOTE_LANE>(a, batch, st);
-    if (tiles_256x128 < num_cu) return launch<128, 128, 2, 2, EPI_PROMOTE>(a, batch, st);
-    return launch<256, 128, 4, 2, EPI_PROMOTE>(a, batch, st);
+    // 256 x 256 tiles (128 x 64 per wave, float accumulators only) where they fill the machine, else
+    // 256 x 128 (64 x 64 per wave, int32 + float accumulators), else 128 x 128
+    if (large || tiles_256x256 >= num_cu) return launch<256, 256, 2, 4, EPI_PROMOTE_CHAIN>(a, batch, st);
+    if (tiles_256x128 >= num_cu) return launch<256, 128, 4, 2, EPI_PROMOTE>(a, batch, st);
+    return launch<128, 128, 2, 2, EPI_PROMOTE>(a, batch, st);
 }
 
 extern "C" int ti8_gemm_i8_nt_i32(const int8_t* A, int64_t bsa, int64_t lda, const int8_t* B, int64_t bsb, int64_t ldb,

@@ -53,7 +53,7 @@ def _live_rows(a_q, tokens):
     with few tokens the GEMM takes any multiple of 32 rows, and the padding rows are zeros whose
     products nobody reads."""
     rows = a_q.shape[0]
-    if tokens is None or rows > 256 or ops.GEMM_PATH == "tiled" or a_q.shape[1] > 32768:
+    if tokens is None or rows > 256 or ops.GEMM_PATH in ("tiled", "large") or a_q.shape[1] > 32768:
         return rows
     return min(rows, -(-tokens // 32) * 32)
 

@@ -8,16 +8,17 @@ here, before anything is launched.
 import torch
 
 from . import _lib
-from ._lib import (COMBINE_DIV_PROD, COMBINE_MUL_MUL, COMBINE_MUL_PROD, GEMM_SKINNY, GEMM_STRICT, GEMM_TILED, INV_AMAX_DIV_127,
+from ._lib import (COMBINE_DIV_PROD, COMBINE_MUL_MUL, COMBINE_MUL_PROD, GEMM_LARGE_TILES, GEMM_SKINNY, GEMM_STRICT, GEMM_TILED, INV_AMAX_DIV_127,
                    INV_AMAX_MUL_RCP127, INV_MULTIPLIER, INV_RCP_OF_SCALE, Q_CLAMP, Q_EPS_ADD, Q_HAD128, Q_SCALE_BF16,
                    SCALE_BLOCK128, SCALE_BLOCK_K256, SCALE_ROW, SCALE_ROW_K128)
 
 __all__ = ["quant_block", "quant_block_had128", "quant_row", "quant_col_t", "quant_row_col_t", "fwht", "gemm_i8_nt", "gemm_i8_nt_i32"]
 
 
-# Which GEMM kernel `gemm_i8_nt` asks for: "auto" (the few-rows kernel for M <= 256, else the
-# LDS-tiled one), "tiled" or "skinny" (wherever it supports the scale modes).  Tests set it to
-# run the same cases through both kernels.
+# Which GEMM kernel `gemm_i8_nt` asks for: "auto" (the few-rows kernel for M <= 256, else an
+# LDS-tiled one with tiles sized to the shape), "tiled", "large" (LDS-tiled with 256 x 256 tiles
+# whatever the shape) or "skinny" (wherever it supports the scale modes).  Tests set it to run
+# the same cases through every kernel.
 GEMM_PATH = "auto"
 
 
@@ -241,7 +242,7 @@ def gemm_i8_nt(A, B, sA, modeA, sB, modeB, *, acc_i32_full=False, combine=COMBIN
               out.data_ptr(), out.stride(0), out.stride(1),
               sAv.data_ptr(), modeA, sa_bs, sa_rs, sa_ks, sBv.data_ptr(), modeB, sb_bs, sb_rs, sb_ks,
               batch, M, N, K, 1 if acc_i32_full else 0, combine, float(out_scale), float(post_scale),
-              (GEMM_STRICT if strict else 0) | {"auto": 0, "tiled": GEMM_TILED, "skinny": GEMM_SKINNY}[GEMM_PATH],
+              (GEMM_STRICT if strict else 0) | {"auto": 0, "tiled": GEMM_TILED, "skinny": GEMM_SKINNY, "large": GEMM_LARGE_TILES}[GEMM_PATH],
               _stream())
     return out
 
