@@ -206,7 +206,7 @@ def main():
     g = [a.elapsed_time(b) for a, b in rec["ti8_gemm_i8_nt"]]
     assert len(g) == 3 * args.steps
     gemm_ms = [sum(g[i::3]) / args.steps for i in range(3)]
-    kernel = "gemm_i8_kernel<256,256,2,4,EPI_ROWS>" if args.scheme == "double_channel" else "gemm_i8_kernel<256,128,4,2,EPI_PROMOTE>"
+    kernel = "gemm_i8_kernel<256,256,2,4,EPI_ROWS>" if args.scheme == "double_channel" else "gemm_i8_kernel<256,256,2,4,EPI_PROMOTE_CHAIN>"
     avg_ms = sum(gemm_ms) / len(gemm_ms)
     achieved = 2.0 * M * N * K / (avg_ms * 1e-3) / 1e12
 
@@ -227,7 +227,7 @@ def main():
 
     # HBM-side bytes per GEMM launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled on the device
     # copy above (profiles/bench_config2_*_hbm_counters.md); measured for these two schemes
-    traffic = {"block_channel": 324716454, "double_channel": 257920121}.get(args.scheme)
+    traffic = {"block_channel": 257629592, "double_channel": 257920121}.get(args.scheme)
 
     out = {
         "metric": METRIC, "value": round(tops, 2), "unit": "TOPS", "n_gpus": 1, "steps": args.steps,
