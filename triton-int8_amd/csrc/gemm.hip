@@ -7,7 +7,9 @@
 //   by row so that the 32 rows a wave reads at one k offset fall in distinct banks)
 //   --ds_read_b128--> MFMA operand registers --> int32 accumulators.
 // A K tile is exactly one 128-deep quantisation block, so the block-channel variants
-// convert and scale the int32 partial into an fp32 accumulator once per K tile.
+// convert and scale the int32 partial into an fp32 accumulator once per K tile.  Large
+// block-channel shapes use a variant of the main loop (EPI_PROMOTE_CHAIN, described where it
+// starts) that keeps no int32 accumulator from one K tile to the next.
 //
 // MFMA operand/result layout used (32x32x32 i8): lane l supplies row (l % 32) of its
 // operand and the 16 bytes k = 16*(l / 32) .. +15 of the 32-deep slice (the same map

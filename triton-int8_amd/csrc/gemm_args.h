@@ -23,7 +23,7 @@ struct GemmArgs {
     float out_scale, post_scale;
 };
 
-// EPI_PROMOTE: the per-K-tile factor is uniform over a wave's 128 x 64 tile (block or per-row scales
+// EPI_PROMOTE: the per-K-tile factor is uniform over a wave's tile (block or per-row scales
 // on both operands); EPI_PROMOTE_LANE: operand B carries one scale per (column, K tile).
 // EPI_PROMOTE_CHAIN: EPI_PROMOTE without int32 accumulators that live across K tiles (see gemm.hip).
 enum { EPI_I32 = 0, EPI_ROWS = 1, EPI_PROMOTE = 2, EPI_STRICT = 3, EPI_PROMOTE_LANE = 4, EPI_PROMOTE_CHAIN = 5 };
