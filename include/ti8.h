@@ -38,7 +38,9 @@ enum ti8_status {
 
 /* quantiser flags (bit set) */
 enum ti8_qflags {
-    TI8_Q_CLAMP = 1,        /* clamp floor(x*scale+0.5) to [-128,127] before the int8 cast */
+    TI8_Q_CLAMP = 1,        /* clamp floor(x*scale+0.5) to [-128,127] before the int8 cast.  The conversion
+                               saturates with or without this flag: the unclamped reference kernels give
+                               the same bytes on every finite input, |x*scale| <= 127 by construction */
     TI8_Q_EPS_ADD = 2,      /* amax + 1e-5 (fused kernels) instead of max(amax, 1e-4) */
     TI8_Q_SCALE_BF16 = 4,   /* round the stored scale through bf16 (TileLang copy) */
     TI8_Q_HAD128 = 8        /* ti8_quant_row only: rotate every 128-column group by H_128 (fp32

@@ -67,13 +67,14 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: keep it in an SGPR
     const int wm = wave / WN, wn = wave % WN;
 
-    // ---- tile assignment: XCD-aware remap, then groups of 8 tile rows -----------------
+    // ---- tile assignment: XCD-aware remap, then groups of GROUP tile rows -------------
     const int ntiles = g.tiles_m * g.tiles_n;
     int pid = blockIdx.x;
     if ((ntiles & 7) == 0) pid = (pid & 7) * (ntiles >> 3) + (pid >> 3);  // one contiguous range per XCD
     // tile rows per group: the 32 workgroups one XCD runs at a time then cover GROUP x 32/GROUP
-    // tiles, chosen so that the A and B panels they share are about the same size
-    constexpr int GROUP = (BM > BN) ? 4 : 8;
+    // tiles, chosen so that the A and B panels they share are about the same size (256-row tiles:
+    // 4 measured 0.4 % faster than 8 and 1 % faster than 16 on 8192 x 4096 x 4096)
+    constexpr int GROUP = (BM >= 256) ? 4 : 8;
     const int per_group = GROUP * g.tiles_n;
     const int group_id = pid / per_group;
     const int first_m = group_id * GROUP;

@@ -9,7 +9,7 @@
 namespace ti8 {
 
 struct QMode {
-    int clamp;       // TI8_Q_CLAMP
+    int clamp;       // TI8_Q_CLAMP (recorded; the byte conversion saturates either way, see qbiased)
     int eps_add;     // TI8_Q_EPS_ADD
     int scale_bf16;  // TI8_Q_SCALE_BF16
     int inv_mode;    // ti8_inv_mode
@@ -33,20 +33,44 @@ __device__ __forceinline__ float stored_scale(float amax, float scale, const QMo
     return s;
 }
 
-__device__ __forceinline__ uint32_t q1(float x, float scale, int clamp) {
-    float r = floorf(x * scale + 0.5f);  // two roundings (contraction is off)
-    if (clamp) r = fminf(fmaxf(r, -128.0f), 127.0f);
-    return static_cast<uint32_t>(static_cast<int>(r)) & 0xffu;
+// Rounding and int8 conversion.  r = floor(x*scale + 0.5) with two roundings (contraction is
+// off), then r + 128 (exact: r is integral) goes through the saturating float -> u8 conversion
+// v_cvt_pk_u8_f32, which also places the byte in a chosen position of a dword; xor 0x80 per byte
+// turns the biased byte into two's complement.  The saturation IS the [-128, 127] clamp; without
+// TI8_Q_CLAMP the reference applies no clamp, which gives the same bytes for every finite input
+// because |x*scale| <= 127 when scale = 127 / absmax of the same data.
+__device__ __forceinline__ float qbiased(float x, float scale) { return floorf(x * scale + 0.5f) + 128.0f; }
+__device__ __forceinline__ uint32_t put_u8(float t, uint32_t byte, uint32_t old) {
+    return __builtin_amdgcn_cvt_pk_u8_f32(t, byte, old);
 }
+constexpr uint32_t UNBIAS4 = 0x80808080u;
 
 // 8 bf16 (one 16-byte load) -> 8 int8 in two dwords, element 0 in the low byte
-__device__ __forceinline__ uint2 quant8(const uint4& v, float scale, int clamp) {
+__device__ __forceinline__ uint2 quant8(const uint4& v, float scale) {
+    uint32_t a = put_u8(qbiased(bf16_lo(v.x), scale), 0, 0u), b = put_u8(qbiased(bf16_lo(v.z), scale), 0, 0u);
+    a = put_u8(qbiased(bf16_hi(v.x), scale), 1, a);
+    b = put_u8(qbiased(bf16_hi(v.z), scale), 1, b);
+    a = put_u8(qbiased(bf16_lo(v.y), scale), 2, a);
+    b = put_u8(qbiased(bf16_lo(v.w), scale), 2, b);
+    a = put_u8(qbiased(bf16_hi(v.y), scale), 3, a);
+    b = put_u8(qbiased(bf16_hi(v.w), scale), 3, b);
     uint2 o;
-    o.x = q1(bf16_lo(v.x), scale, clamp) | (q1(bf16_hi(v.x), scale, clamp) << 8) |
-          (q1(bf16_lo(v.y), scale, clamp) << 16) | (q1(bf16_hi(v.y), scale, clamp) << 24);
-    o.y = q1(bf16_lo(v.z), scale, clamp) | (q1(bf16_hi(v.z), scale, clamp) << 8) |
-          (q1(bf16_lo(v.w), scale, clamp) << 16) | (q1(bf16_hi(v.w), scale, clamp) << 24);
+    o.x = a ^ UNBIAS4;
+    o.y = b ^ UNBIAS4;
     return o;
+}
+
+// the 8 elements of row j (j < 4) of a 4-row patch, each with its own column scale, into byte j of
+// w[0..7] (biased: xor UNBIAS4 once all four rows are in)
+__device__ __forceinline__ void put_row_by_cols(const uint4& v, const float (&scale)[8], uint32_t j, uint32_t (&w)[8]) {
+    w[0] = put_u8(qbiased(bf16_lo(v.x), scale[0]), j, w[0]);
+    w[1] = put_u8(qbiased(bf16_hi(v.x), scale[1]), j, w[1]);
+    w[2] = put_u8(qbiased(bf16_lo(v.y), scale[2]), j, w[2]);
+    w[3] = put_u8(qbiased(bf16_hi(v.y), scale[3]), j, w[3]);
+    w[4] = put_u8(qbiased(bf16_lo(v.z), scale[4]), j, w[4]);
+    w[5] = put_u8(qbiased(bf16_hi(v.z), scale[5]), j, w[5]);
+    w[6] = put_u8(qbiased(bf16_lo(v.w), scale[6]), j, w[6]);
+    w[7] = put_u8(qbiased(bf16_hi(v.w), scale[7]), j, w[7]);
 }
 
 __device__ __forceinline__ float absmax8(const uint4& v, float m) {
@@ -119,11 +143,15 @@ __device__ __forceinline__ float block_max_256(float v, float* red4) {
     return v;
 }
 
-// byte e (0..3) of four dwords -> one dword (row 0 in the low byte): a 4x4 byte transpose column
-__device__ __forceinline__ uint32_t gather_byte(uint32_t r0, uint32_t r1, uint32_t r2, uint32_t r3, int e) {
-    const int sh = e * 8;
-    return ((r0 >> sh) & 0xffu) | (((r1 >> sh) & 0xffu) << 8) | (((r2 >> sh) & 0xffu) << 16) |
-           (((r3 >> sh) & 0xffu) << 24);
+// 4 x 4 byte transpose: out[e] = byte e of r0, r1, r2, r3 (r0 in the low byte), two rounds of
+// v_perm_b32 (selector values 0-3 pick bytes of the second operand, 4-7 of the first)
+__device__ __forceinline__ void transpose4x4_bytes(uint32_t r0, uint32_t r1, uint32_t r2, uint32_t r3, uint32_t* out) {
+    const uint32_t t01l = __builtin_amdgcn_perm(r1, r0, 0x05010400u), t01h = __builtin_amdgcn_perm(r1, r0, 0x07030602u);
+    const uint32_t t23l = __builtin_amdgcn_perm(r3, r2, 0x05010400u), t23h = __builtin_amdgcn_perm(r3, r2, 0x07030602u);
+    out[0] = __builtin_amdgcn_perm(t23l, t01l, 0x05040100u);
+    out[1] = __builtin_amdgcn_perm(t23l, t01l, 0x07060302u);
+    out[2] = __builtin_amdgcn_perm(t23h, t01h, 0x05040100u);
+    out[3] = __builtin_amdgcn_perm(t23h, t01h, 0x07060302u);
 }
 
 // ---------------------------------------------------------------------------------
@@ -180,7 +208,7 @@ __global__ __launch_bounds__(256) void quant_block_kernel(
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) o[h][j] = quant8(v[u][h][j], scale, mode.clamp);
+            for (int j = 0; j < 4; ++j) o[h][j] = quant8(v[u][h][j], scale);
 
         if (WRITE_Q) {
             int8_t* qt = q + b * bsq + (int64_t)rb * 128 * ldq + (int64_t)cb * (128 * NSUB) + u * 128 + cc * 8;
@@ -193,12 +221,13 @@ __global__ __launch_bounds__(256) void quant_block_kernel(
         if (WRITE_QT) {  // NSUB == 1 only (checked on the host)
 #pragma unroll
             for (int h = 0; h < 2; ++h)
+            {
+                uint32_t w[8];
+                transpose4x4_bytes(o[h][0].x, o[h][1].x, o[h][2].x, o[h][3].x, w);
+                transpose4x4_bytes(o[h][0].y, o[h][1].y, o[h][2].y, o[h][3].y, w + 4);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const uint32_t w = (e < 4) ? gather_byte(o[h][0].x, o[h][1].x, o[h][2].x, o[h][3].x, e)
-                                               : gather_byte(o[h][0].y, o[h][1].y, o[h][2].y, o[h][3].y, e - 4);
-                    tileT[(cc * 8 + e) * 33 + h * 16 + rg] = w;  // [column of x][4-row group]
-                }
+                for (int e = 0; e < 8; ++e) tileT[(cc * 8 + e) * 33 + h * 16 + rg] = w[e];  // [column of x][4-row group]
+            }
             __syncthreads();
             int8_t* qtt = qT + b * bsqt + (int64_t)cb * 128 * ldqt + (int64_t)rb * 128;
 #pragma unroll
@@ -303,7 +332,7 @@ __global__ __launch_bounds__(256) void quant_block_had_kernel(
                     const float amax = amax_floor(__uint_as_float(ws[col]), mode.eps_add);
                     const float scale = 127.0f / amax;
                     if (rb == 0 && cc == 0) s[col] = stored_scale(amax, scale, mode);
-                    *reinterpret_cast<uint2*>(qcol + (int64_t)(h * 64 + rg * 4 + j) * ldq) = quant8(r, scale, mode.clamp);
+                    *reinterpret_cast<uint2*>(qcol + (int64_t)(h * 64 + rg * 4 + j) * ldq) = quant8(r, scale);
                 }
             }
         return;
@@ -327,7 +356,7 @@ __global__ __launch_bounds__(256) void quant_block_had_kernel(
     for (int h = 0; h < 2; ++h)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-            *reinterpret_cast<uint2*>(qt + (int64_t)(h * 64 + rg * 4 + j) * ldq + cc * 8) = quant8(v[h][j], scale, mode.clamp);
+            *reinterpret_cast<uint2*>(qt + (int64_t)(h * 64 + rg * 4 + j) * ldq + cc * 8) = quant8(v[h][j], scale);
 }
 
 // ---------------------------------------------------------------------------------
@@ -368,7 +397,7 @@ __global__ __launch_bounds__(256) void quant_row_kernel(const uint16_t* __restri
             amax = amax_floor(amax, mode.eps_add);
             const float scale = 127.0f / amax;
             if (c < nchunk) {
-                *reinterpret_cast<uint2*>(qr + c * 8) = quant8(v[i], scale, mode.clamp);
+                *reinterpret_cast<uint2*>(qr + c * 8) = quant8(v[i], scale);
                 if ((c & 15) == 0) s[row * ngrp + (c >> 4)] = stored_scale(amax, scale, mode);
             }
         }
@@ -387,7 +416,7 @@ __global__ __launch_bounds__(256) void quant_row_kernel(const uint16_t* __restri
 #pragma unroll
     for (int i = 0; i < NLOAD; ++i) {
         const int c = t + i * T;
-        if (c < nchunk) *reinterpret_cast<uint2*>(qr + c * 8) = quant8(v[i], scale, mode.clamp);
+        if (c < nchunk) *reinterpret_cast<uint2*>(qr + c * 8) = quant8(v[i], scale);
     }
 }
 
@@ -464,23 +493,11 @@ __global__ __launch_bounds__(256) void quant_col_t_kernel(const uint16_t* __rest
     }
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-        uint32_t qq[4][8];
+        uint32_t w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const uint4& w = v[h][j];
-            qq[j][0] = q1(bf16_lo(w.x), scale[0], mode.clamp);
-            qq[j][1] = q1(bf16_hi(w.x), scale[1], mode.clamp);
-            qq[j][2] = q1(bf16_lo(w.y), scale[2], mode.clamp);
-            qq[j][3] = q1(bf16_hi(w.y), scale[3], mode.clamp);
-            qq[j][4] = q1(bf16_lo(w.z), scale[4], mode.clamp);
-            qq[j][5] = q1(bf16_hi(w.z), scale[5], mode.clamp);
-            qq[j][6] = q1(bf16_lo(w.w), scale[6], mode.clamp);
-            qq[j][7] = q1(bf16_hi(w.w), scale[7], mode.clamp);
-        }
+        for (int j = 0; j < 4; ++j) put_row_by_cols(v[h][j], scale, j, w);
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-            tileT[(cc * 8 + e) * 33 + h * 16 + rg] =
-                qq[0][e] | (qq[1][e] << 8) | (qq[2][e] << 16) | (qq[3][e] << 24);
+        for (int e = 0; e < 8; ++e) tileT[(cc * 8 + e) * 33 + h * 16 + rg] = w[e] ^ UNBIAS4;
     }
     __syncthreads();
     int8_t* qtt = qT + (int64_t)cb * 128 * ldqt + (int64_t)rb * 128;
@@ -499,28 +516,33 @@ __global__ __launch_bounds__(256) void quant_col_t_kernel(const uint16_t* __rest
 
 // ---------------------------------------------------------------------------------
 // Row AND column absmax of x in one read (both quantisations of an operand that a training
-// step needs: by rows for one GEMM, by columns -- transposed -- for another).  Same
-// 128 x 256 tile and thread map as col_absmax_kernel; a row of the tile is spread over the
-// 32 lanes of a half-wave, whose maxima meet through lane shuffles.
+// step needs: by rows for one GEMM, by columns -- transposed -- for another).  TR x 256 tile with
+// the thread map of col_absmax_kernel; a row of the tile is spread over the 32 lanes of a
+// half-wave, whose maxima meet through lane shuffles.  Short tiles win although they issue more
+// atomics: 32 rows measured 6 % faster than 128 on 4096 x 4096 and on 8192 x 4096 (more workgroups
+// per CU, so the loads of one overlap the reductions of another).
+constexpr int ABSMAX_ROWS = 32;
+template <int TR>  // rows of x per workgroup (a multiple of 8 that divides 128)
 __global__ __launch_bounds__(256) void rowcol_absmax_kernel(const uint16_t* __restrict__ x, int64_t ldx,
                                                             unsigned int* __restrict__ ws_row,
                                                             unsigned int* __restrict__ ws_col, int64_t R, int C) {
+    constexpr int NR = TR / 8;
     __shared__ float part[8][256];
     const int tid = threadIdx.x;
     const int cc = tid & 31, rg = tid >> 5;
     const int c0 = blockIdx.x * 256 + cc * 8;
-    const int64_t r0 = (int64_t)blockIdx.y * 128;
+    const int64_t r0 = (int64_t)blockIdx.y * TR;
     float m[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    float rmax[16];
+    float rmax[NR];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) rmax[i] = 0.0f;
+    for (int i = 0; i < NR; ++i) rmax[i] = 0.0f;
     if (c0 < C) {
-        uint4 v[16];
+        uint4 v[NR];
 #pragma unroll
-        for (int i = 0; i < 16; ++i)
+        for (int i = 0; i < NR; ++i)
             v[i] = *reinterpret_cast<const uint4*>(x + (r0 + rg + 8 * i) * ldx + c0);
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
+        for (int i = 0; i < NR; ++i) {
             const float e0 = fabsf(bf16_lo(v[i].x)), e1 = fabsf(bf16_hi(v[i].x)), e2 = fabsf(bf16_lo(v[i].y)),
                         e3 = fabsf(bf16_hi(v[i].y)), e4 = fabsf(bf16_lo(v[i].z)), e5 = fabsf(bf16_hi(v[i].z)),
                         e6 = fabsf(bf16_lo(v[i].w)), e7 = fabsf(bf16_hi(v[i].w));
@@ -531,7 +553,7 @@ __global__ __launch_bounds__(256) void rowcol_absmax_kernel(const uint16_t* __re
     }
     // row maxima: over the 32 lanes (tid % 32) that hold the same rows
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
+    for (int i = 0; i < NR; ++i) {
         float a = rmax[i];
 #pragma unroll
         for (int off = 16; off >= 1; off >>= 1) a = fmaxf(a, __shfl_xor(a, off, 64));
@@ -579,28 +601,18 @@ __global__ __launch_bounds__(256) void quant_rowcol_kernel(const uint16_t* __res
     int8_t* qt = q + (int64_t)rb * 128 * ldq + (int64_t)cb * 128 + cc * 8;
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-        uint32_t qq[4][8];
+        uint32_t w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int row = h * 64 + rg * 4 + j;
             const float amax = amax_floor(ws_row[(int64_t)rb * 128 + row], mode.eps_add);
             const float rscale = 127.0f / amax;
             if (cb == 0 && cc == 0) s_row[(int64_t)rb * 128 + row] = stored_scale(amax, rscale, mode);
-            const uint4& w = v[h][j];
-            *reinterpret_cast<uint2*>(qt + (int64_t)row * ldq) = quant8(w, rscale, mode.clamp);
-            qq[j][0] = q1(bf16_lo(w.x), cscale[0], mode.clamp);
-            qq[j][1] = q1(bf16_hi(w.x), cscale[1], mode.clamp);
-            qq[j][2] = q1(bf16_lo(w.y), cscale[2], mode.clamp);
-            qq[j][3] = q1(bf16_hi(w.y), cscale[3], mode.clamp);
-            qq[j][4] = q1(bf16_lo(w.z), cscale[4], mode.clamp);
-            qq[j][5] = q1(bf16_hi(w.z), cscale[5], mode.clamp);
-            qq[j][6] = q1(bf16_lo(w.w), cscale[6], mode.clamp);
-            qq[j][7] = q1(bf16_hi(w.w), cscale[7], mode.clamp);
+            *reinterpret_cast<uint2*>(qt + (int64_t)row * ldq) = quant8(v[h][j], rscale);
+            put_row_by_cols(v[h][j], cscale, j, w);
         }
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-            tileT[(cc * 8 + e) * 33 + h * 16 + rg] =
-                qq[0][e] | (qq[1][e] << 8) | (qq[2][e] << 16) | (qq[3][e] << 24);
+        for (int e = 0; e < 8; ++e) tileT[(cc * 8 + e) * 33 + h * 16 + rg] = w[e] ^ UNBIAS4;
     }
     __syncthreads();
     int8_t* qtt = qT + (int64_t)cb * 128 * ldqt + (int64_t)rb * 128;
@@ -752,7 +764,7 @@ extern "C" int ti8_quant_row_col_t(const void* x, int64_t ldx, int8_t* q, int64_
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     unsigned int* wsu = reinterpret_cast<unsigned int*>(ws);   // [R row maxima][C column maxima]
     hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((R + C + 255) / 256)), dim3(256), 0, st, wsu, (int)(R + C), 0u);
-    hipLaunchKernelGGL(rowcol_absmax_kernel, dim3((unsigned)((C + 255) / 256), (unsigned)(R / 128)), dim3(256), 0, st, xp,
+    hipLaunchKernelGGL(rowcol_absmax_kernel<ABSMAX_ROWS>, dim3((unsigned)((C + 255) / 256), (unsigned)(R / ABSMAX_ROWS)), dim3(256), 0, st, xp,
                        ldx, wsu, wsu + R, R, (int)C);
     hipLaunchKernelGGL(quant_rowcol_kernel, dim3((unsigned)ntiles), dim3(256), 0, st, xp, ldx, q, ldq, s_row, qT, ldqt,
                        s_col, ws, ws + R, (int)(C / 128), mode);
