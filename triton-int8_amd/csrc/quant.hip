@@ -94,6 +94,35 @@ __device__ __forceinline__ float dpp_f32(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
 }
 
+// max(v, v of the lane that DPP control CTRL names) in the rows of ROW_MASK; other lanes keep v
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ float dpp_max(float v) {
+    const int i = __float_as_int(v);
+    return fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(i, i, CTRL, ROW_MASK, 0xf, false)));
+}
+
+// max over each half-wave of 32 lanes without LDS traffic; valid in lanes 16-31 and 48-63.
+// quad_perm lane^1, lane^2, then row_half_mirror and row_mirror (all 16 lanes of a row agree),
+// then row_bcast:15 into rows 1 and 3 (lane 15 of the row before).
+__device__ __forceinline__ float half_wave_max_hi(float v) {
+    v = dpp_max<0xB1>(v);
+    v = dpp_max<0x4E>(v);
+    v = dpp_max<0x141>(v);
+    v = dpp_max<0x140>(v);
+    return dpp_max<0x142, 0xA>(v);
+}
+
+// max of v over the lane pair (l, l ^ 32), in both lanes (v_permlane32_swap: one cross-half move)
+__device__ __forceinline__ float pair32_max(float v) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    const unsigned u = __float_as_uint(v);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+#else
+    return v;
+#endif
+}
+
 // 128-point Walsh-Hadamard transform of a row segment held as 8 consecutive bf16 per lane by 16
 // consecutive lanes (lane%16 = chunk index): butterflies in the fixed order stride 1, 2, 4 (in
 // registers), 8, 16, 32, 64 (lane xor 1, 2, 4, 8), fp32, un-normalised; one rounding to bf16.
@@ -471,6 +500,7 @@ __global__ __launch_bounds__(256) void quant_col_t_kernel(const uint16_t* __rest
                                                           float* __restrict__ s, const float* __restrict__ ws,
                                                           int ncb, QMode mode) {
     __shared__ uint32_t tileT[128 * 33];
+    __shared__ __attribute__((aligned(16))) float sc[128];
     const int cb = blockIdx.x % ncb;
     const int rb = blockIdx.x / ncb;
     const int tid = threadIdx.x;
@@ -484,12 +514,19 @@ __global__ __launch_bounds__(256) void quant_col_t_kernel(const uint16_t* __rest
         for (int j = 0; j < 4; ++j)
             v[h][j] = *reinterpret_cast<const uint4*>(xt + (int64_t)(h * 64 + rg * 4 + j) * ldx + cc * 8);
 
+    // the tile's 128 column scales: one division each, shared through LDS
+    if (tid < 128) {
+        const float amax = amax_floor(ws[cb * 128 + tid], mode.eps_add);
+        const float sv = 127.0f / amax;
+        sc[tid] = sv;
+        if (rb == 0) s[cb * 128 + tid] = stored_scale(amax, sv, mode);
+    }
+    __syncthreads();
     float scale[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        const float amax = amax_floor(ws[cb * 128 + cc * 8 + e], mode.eps_add);
-        scale[e] = 127.0f / amax;
-        if (rb == 0 && rg == 0) s[cb * 128 + cc * 8 + e] = stored_scale(amax, scale[e], mode);
+    {
+        const float4 c0 = *reinterpret_cast<const float4*>(&sc[cc * 8]), c1 = *reinterpret_cast<const float4*>(&sc[cc * 8 + 4]);
+        scale[0] = c0.x; scale[1] = c0.y; scale[2] = c0.z; scale[3] = c0.w;
+        scale[4] = c1.x; scale[5] = c1.y; scale[6] = c1.z; scale[7] = c1.w;
     }
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
@@ -518,7 +555,7 @@ __global__ __launch_bounds__(256) void quant_col_t_kernel(const uint16_t* __rest
 // Row AND column absmax of x in one read (both quantisations of an operand that a training
 // step needs: by rows for one GEMM, by columns -- transposed -- for another).  TR x 256 tile with
 // the thread map of col_absmax_kernel; a row of the tile is spread over the 32 lanes of a
-// half-wave, whose maxima meet through lane shuffles.  Short tiles win although they issue more
+// half-wave, whose maxima meet through DPP moves.  Short tiles win although they issue more
 // atomics: 32 rows measured 6 % faster than 128 on 4096 x 4096 and on 8192 x 4096 (more workgroups
 // per CU, so the loads of one overlap the reductions of another).
 constexpr int ABSMAX_ROWS = 32;
@@ -527,7 +564,7 @@ __global__ __launch_bounds__(256) void rowcol_absmax_kernel(const uint16_t* __re
                                                             unsigned int* __restrict__ ws_row,
                                                             unsigned int* __restrict__ ws_col, int64_t R, int C) {
     constexpr int NR = TR / 8;
-    __shared__ float part[8][256];
+    __shared__ __attribute__((aligned(16))) float part[4][256];
     const int tid = threadIdx.x;
     const int cc = tid & 31, rg = tid >> 5;
     const int c0 = blockIdx.x * 256 + cc * 8;
@@ -554,17 +591,19 @@ __global__ __launch_bounds__(256) void rowcol_absmax_kernel(const uint16_t* __re
     // row maxima: over the 32 lanes (tid % 32) that hold the same rows
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
-        float a = rmax[i];
-#pragma unroll
-        for (int off = 16; off >= 1; off >>= 1) a = fmaxf(a, __shfl_xor(a, off, 64));
-        if (cc == 0) atomicMax(ws_row + r0 + rg + 8 * i, __float_as_uint(a));
+        const float a = half_wave_max_hi(rmax[i]);
+        if (cc == 16) atomicMax(ws_row + r0 + rg + 8 * i, __float_as_uint(a));
     }
+    // column maxima: the two half-waves of a wave first, then the four waves through LDS
 #pragma unroll
-    for (int e = 0; e < 8; ++e) part[rg][cc * 8 + e] = m[e];
+    for (int e = 0; e < 8; ++e) m[e] = pair32_max(m[e]);
+    if ((tid & 32) == 0) {
+        float4* dst = reinterpret_cast<float4*>(&part[tid >> 6][cc * 8]);
+        dst[0] = make_float4(m[0], m[1], m[2], m[3]);
+        dst[1] = make_float4(m[4], m[5], m[6], m[7]);
+    }
     __syncthreads();
-    float a = part[0][tid];
-#pragma unroll
-    for (int g = 1; g < 8; ++g) a = fmaxf(a, part[g][tid]);
+    const float a = fmaxf(fmaxf(part[0][tid], part[1][tid]), fmaxf(part[2][tid], part[3][tid]));
     const int c = blockIdx.x * 256 + tid;
     if (c < C) atomicMax(ws_col + c, __float_as_uint(a));
 }
@@ -578,6 +617,7 @@ __global__ __launch_bounds__(256) void quant_rowcol_kernel(const uint16_t* __res
                                                            const float* __restrict__ ws_row,
                                                            const float* __restrict__ ws_col, int ncb, QMode mode) {
     __shared__ uint32_t tileT[128 * 33];
+    __shared__ __attribute__((aligned(16))) float sc[256];  // [0,128): row scales, [128,256): column scales
     const int cb = blockIdx.x % ncb;
     const int rb = blockIdx.x / ncb;
     const int tid = threadIdx.x;
@@ -591,12 +631,22 @@ __global__ __launch_bounds__(256) void quant_rowcol_kernel(const uint16_t* __res
         for (int j = 0; j < 4; ++j)
             v[h][j] = *reinterpret_cast<const uint4*>(xt + (int64_t)(h * 64 + rg * 4 + j) * ldx + cc * 8);
 
+    // the tile's 128 row scales and 128 column scales: one division per thread, shared through LDS
+    {
+        const bool is_row = tid < 128;
+        const int idx = tid & 127;
+        const int64_t at = is_row ? (int64_t)rb * 128 + idx : (int64_t)cb * 128 + idx;
+        const float amax = amax_floor(is_row ? ws_row[at] : ws_col[at], mode.eps_add);
+        const float scale = 127.0f / amax;
+        sc[tid] = scale;
+        if (is_row ? cb == 0 : rb == 0) (is_row ? s_row : s_col)[at] = stored_scale(amax, scale, mode);
+    }
+    __syncthreads();
     float cscale[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        const float amax = amax_floor(ws_col[cb * 128 + cc * 8 + e], mode.eps_add);
-        cscale[e] = 127.0f / amax;
-        if (rb == 0 && rg == 0) s_col[cb * 128 + cc * 8 + e] = stored_scale(amax, cscale[e], mode);
+    {
+        const float4 c0 = *reinterpret_cast<const float4*>(&sc[128 + cc * 8]), c1 = *reinterpret_cast<const float4*>(&sc[132 + cc * 8]);
+        cscale[0] = c0.x; cscale[1] = c0.y; cscale[2] = c0.z; cscale[3] = c0.w;
+        cscale[4] = c1.x; cscale[5] = c1.y; cscale[6] = c1.z; cscale[7] = c1.w;
     }
     int8_t* qt = q + (int64_t)rb * 128 * ldq + (int64_t)cb * 128 + cc * 8;
 #pragma unroll
@@ -605,10 +655,7 @@ __global__ __launch_bounds__(256) void quant_rowcol_kernel(const uint16_t* __res
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int row = h * 64 + rg * 4 + j;
-            const float amax = amax_floor(ws_row[(int64_t)rb * 128 + row], mode.eps_add);
-            const float rscale = 127.0f / amax;
-            if (cb == 0 && cc == 0) s_row[(int64_t)rb * 128 + row] = stored_scale(amax, rscale, mode);
-            *reinterpret_cast<uint2*>(qt + (int64_t)row * ldq) = quant8(v[h][j], rscale);
+            *reinterpret_cast<uint2*>(qt + (int64_t)row * ldq) = quant8(v[h][j], sc[row]);
             put_row_by_cols(v[h][j], cscale, j, w);
         }
 #pragma unroll
