@@ -94,35 +94,6 @@ __device__ __forceinline__ float dpp_f32(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
 }
 
-// max(v, v of the lane that DPP control CTRL names) in the rows of ROW_MASK; other lanes keep v
-template <int CTRL, int ROW_MASK = 0xf>
-__device__ __forceinline__ float dpp_max(float v) {
-    const int i = __float_as_int(v);
-    return fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(i, i, CTRL, ROW_MASK, 0xf, false)));
-}
-
-// max over each half-wave of 32 lanes without LDS traffic; valid in lanes 16-31 and 48-63.
-// quad_perm lane^1, lane^2, then row_half_mirror and row_mirror (all 16 lanes of a row agree),
-// then row_bcast:15 into rows 1 and 3 (lane 15 of the row before).
-__device__ __forceinline__ float half_wave_max_hi(float v) {
-    v = dpp_max<0xB1>(v);
-    v = dpp_max<0x4E>(v);
-    v = dpp_max<0x141>(v);
-    v = dpp_max<0x140>(v);
-    return dpp_max<0x142, 0xA>(v);
-}
-
-// max of v over the lane pair (l, l ^ 32), in both lanes (v_permlane32_swap: one cross-half move)
-__device__ __forceinline__ float pair32_max(float v) {
-#if defined(__HIP_DEVICE_COMPILE__)
-    const unsigned u = __float_as_uint(v);
-    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-#else
-    return v;
-#endif
-}
-
 // 128-point Walsh-Hadamard transform of a row segment held as 8 consecutive bf16 per lane by 16
 // consecutive lanes (lane%16 = chunk index): butterflies in the fixed order stride 1, 2, 4 (in
 // registers), 8, 16, 32, 64 (lane xor 1, 2, 4, 8), fp32, un-normalised; one rounding to bf16.
@@ -353,9 +324,7 @@ __global__ __launch_bounds__(256) void quant_block_had_kernel(
                 const int col = cb * 128 + h * 64 + rg * 4 + j;
                 const uint4 r = fwht128_bf16(v[h][j], lane);
                 if (SCALE == HAD_COLMAX) {
-                    float m = absmax8(r, 0.0f);
-#pragma unroll
-                    for (int off = 8; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+                    const float m = row16_max(absmax8(r, 0.0f));
                     if (cc == 0) atomicMax(ws + col, __float_as_uint(m));
                 } else {
                     const float amax = amax_floor(__uint_as_float(ws[col]), mode.eps_add);
@@ -420,10 +389,7 @@ __global__ __launch_bounds__(256) void quant_row_kernel(const uint16_t* __restri
 #pragma unroll
         for (int i = 0; i < NLOAD; ++i) {
             const int c = t + i * T;
-            float amax = absmax8(v[i], 0.0f);
-#pragma unroll
-            for (int off = 8; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
-            amax = amax_floor(amax, mode.eps_add);
+            const float amax = amax_floor(row16_max(absmax8(v[i], 0.0f)), mode.eps_add);
             const float scale = 127.0f / amax;
             if (c < nchunk) {
                 *reinterpret_cast<uint2*>(qr + c * 8) = quant8(v[i], scale);
@@ -455,7 +421,7 @@ __global__ __launch_bounds__(256) void quant_row_kernel(const uint16_t* __restri
 // into ws[] with an unsigned atomic max (non-negative floats order like their bits).
 __global__ __launch_bounds__(256) void col_absmax_kernel(const uint16_t* __restrict__ x, int64_t ldx,
                                                          unsigned int* __restrict__ ws, int64_t R, int C) {
-    __shared__ float part[8][256];
+    __shared__ __attribute__((aligned(16))) float part[4][256];
     const int tid = threadIdx.x;
     const int cc = tid & 31, rg = tid >> 5;
     const int c0 = blockIdx.x * 256 + cc * 8;
@@ -478,12 +444,16 @@ __global__ __launch_bounds__(256) void col_absmax_kernel(const uint16_t* __restr
             m[7] = fmaxf(m[7], fabsf(bf16_hi(v[i].w)));
         }
     }
+    // the two half-waves of a wave first, then the four waves through LDS
 #pragma unroll
-    for (int e = 0; e < 8; ++e) part[rg][cc * 8 + e] = m[e];
+    for (int e = 0; e < 8; ++e) m[e] = pair32_max(m[e]);
+    if ((tid & 32) == 0) {
+        float4* dst = reinterpret_cast<float4*>(&part[tid >> 6][cc * 8]);
+        dst[0] = make_float4(m[0], m[1], m[2], m[3]);
+        dst[1] = make_float4(m[4], m[5], m[6], m[7]);
+    }
     __syncthreads();
-    float a = part[0][tid];
-#pragma unroll
-    for (int g = 1; g < 8; ++g) a = fmaxf(a, part[g][tid]);
+    const float a = fmaxf(fmaxf(part[0][tid], part[1][tid]), fmaxf(part[2][tid], part[3][tid]));
     const int c = blockIdx.x * 256 + tid;
     if (c < C) atomicMax(ws + c, __float_as_uint(a));
 }

@@ -54,11 +54,49 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, ti8_bf16x2));
 }
 
-// max over the 64 lanes of a wavefront, result in every lane
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+// Reductions over lanes with DPP moves (no LDS traffic).
+// max(v, v of the lane that DPP control CTRL names) in the rows of ROW_MASK; other lanes keep v
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ float dpp_max(float v) {
+    const int i = __float_as_int(v);
+    return fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(i, i, CTRL, ROW_MASK, 0xf, false)));
+}
+
+// max over each half-wave of 32 lanes without LDS traffic; valid in lanes 16-31 and 48-63.
+// quad_perm lane^1, lane^2, then row_half_mirror and row_mirror (all 16 lanes of a row agree),
+// then row_bcast:15 into rows 1 and 3 (lane 15 of the row before).
+__device__ __forceinline__ float half_wave_max_hi(float v) {
+    v = dpp_max<0xB1>(v);
+    v = dpp_max<0x4E>(v);
+    v = dpp_max<0x141>(v);
+    v = dpp_max<0x140>(v);
+    return dpp_max<0x142, 0xA>(v);
+}
+
+// max of v over the lane pair (l, l ^ 32), in both lanes (v_permlane32_swap: one cross-half move)
+__device__ __forceinline__ float pair32_max(float v) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    const unsigned u = __float_as_uint(v);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+#else
     return v;
+#endif
+}
+
+// max over the 16 lanes of a DPP row, in all of them
+__device__ __forceinline__ float row16_max(float v) {
+    v = dpp_max<0xB1>(v);
+    v = dpp_max<0x4E>(v);
+    v = dpp_max<0x141>(v);
+    return dpp_max<0x140>(v);
+}
+
+// max over the wave, in every lane: half_wave_max_hi, row_bcast:31 into rows 2 and 3 (lane 63 then
+// holds the maximum), and a read of lane 63
+__device__ __forceinline__ float wave_max(float v) {
+    v = dpp_max<0x143, 0xC>(half_wave_max_hi(v));
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
 }  // namespace ti8
