@@ -415,49 +415,6 @@ __global__ __launch_bounds__(256) void quant_row_kernel(const uint16_t* __restri
     }
 }
 
-// ---------------------------------------------------------------------------------
-// Column absmax: workgroup = 128 rows x 256 columns; thread t reads 16-byte chunks of
-// column chunk t%32 from rows t/32 + 8i.  Partial maxima meet in LDS and are merged
-// into ws[] with an unsigned atomic max (non-negative floats order like their bits).
-__global__ __launch_bounds__(256) void col_absmax_kernel(const uint16_t* __restrict__ x, int64_t ldx,
-                                                         unsigned int* __restrict__ ws, int64_t R, int C) {
-    __shared__ __attribute__((aligned(16))) float part[4][256];
-    const int tid = threadIdx.x;
-    const int cc = tid & 31, rg = tid >> 5;
-    const int c0 = blockIdx.x * 256 + cc * 8;
-    const int64_t r0 = (int64_t)blockIdx.y * 128;
-    float m[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (c0 < C) {
-        uint4 v[16];
-#pragma unroll
-        for (int i = 0; i < 16; ++i)
-            v[i] = *reinterpret_cast<const uint4*>(x + (r0 + rg + 8 * i) * ldx + c0);
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            m[0] = fmaxf(m[0], fabsf(bf16_lo(v[i].x)));
-            m[1] = fmaxf(m[1], fabsf(bf16_hi(v[i].x)));
-            m[2] = fmaxf(m[2], fabsf(bf16_lo(v[i].y)));
-            m[3] = fmaxf(m[3], fabsf(bf16_hi(v[i].y)));
-            m[4] = fmaxf(m[4], fabsf(bf16_lo(v[i].z)));
-            m[5] = fmaxf(m[5], fabsf(bf16_hi(v[i].z)));
-            m[6] = fmaxf(m[6], fabsf(bf16_lo(v[i].w)));
-            m[7] = fmaxf(m[7], fabsf(bf16_hi(v[i].w)));
-        }
-    }
-    // the two half-waves of a wave first, then the four waves through LDS
-#pragma unroll
-    for (int e = 0; e < 8; ++e) m[e] = pair32_max(m[e]);
-    if ((tid & 32) == 0) {
-        float4* dst = reinterpret_cast<float4*>(&part[tid >> 6][cc * 8]);
-        dst[0] = make_float4(m[0], m[1], m[2], m[3]);
-        dst[1] = make_float4(m[4], m[5], m[6], m[7]);
-    }
-    __syncthreads();
-    const float a = fmaxf(fmaxf(part[0][tid], part[1][tid]), fmaxf(part[2][tid], part[3][tid]));
-    const int c = blockIdx.x * 256 + tid;
-    if (c < C) atomicMax(ws + c, __float_as_uint(a));
-}
-
 __global__ void fill_u32_kernel(unsigned int* p, int n, unsigned int v) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = v;
@@ -522,27 +479,43 @@ __global__ __launch_bounds__(256) void quant_col_t_kernel(const uint16_t* __rest
 }
 
 // ---------------------------------------------------------------------------------
-// Row AND column absmax of x in one read (both quantisations of an operand that a training
-// step needs: by rows for one GEMM, by columns -- transposed -- for another).  TR x 256 tile with
-// the thread map of col_absmax_kernel; a row of the tile is spread over the 32 lanes of a
-// half-wave, whose maxima meet through DPP moves.  Short tiles win although they issue more
-// atomics: 32 rows measured 6 % faster than 128 on 4096 x 4096 and on 8192 x 4096 (more workgroups
-// per CU, so the loads of one overlap the reductions of another).
+// Column absmax, and optionally row absmax, of x in one read (WITH_ROWS: both quantisations of
+// an operand that a training step needs, by rows for one GEMM, by columns -- transposed -- for
+// another).  Workgroup = TR rows x 256 columns; thread t reads the 16-byte chunk t%32 of rows
+// t/32 + 8i.  |x| of a bf16 is its bit pattern without the sign, and non-negative bf16 order
+// like their 16-bit patterns, so the maxima are taken on packed pairs of u16 (v_pk_max_u16: no
+// unpacking, two elements per instruction) and widened to fp32 bit patterns (<< 16) at the end,
+// where they are merged into ws[] with an unsigned atomic max.  Row maxima meet over the 32
+// lanes of a half-wave through DPP moves; column maxima over the two half-waves by a lane swap
+// and over the four waves through LDS.  Short tiles win although they issue more atomics: 32
+// rows measured 6 % faster than 128 on 4096 x 4096 and on 8192 x 4096 (more workgroups per CU,
+// so the loads of one overlap the reductions of another); 16 and 64 rows are 1-2 % slower than 32.
 constexpr int ABSMAX_ROWS = 32;
-template <int TR>  // rows of x per workgroup (a multiple of 8 that divides 128)
-__global__ __launch_bounds__(256) void rowcol_absmax_kernel(const uint16_t* __restrict__ x, int64_t ldx,
-                                                            unsigned int* __restrict__ ws_row,
-                                                            unsigned int* __restrict__ ws_col, int64_t R, int C) {
+
+typedef unsigned short ti8_u16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(ti8_u16x2, a), __builtin_bit_cast(ti8_u16x2, b)));
+}
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ uint32_t dpp_pk_max_u16(uint32_t v) {
+    return pk_max_u16(v, (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, CTRL, ROW_MASK, 0xf, false));
+}
+
+template <int TR, bool WITH_ROWS>  // TR: rows of x per workgroup (8, 16, ... 128)
+__global__ __launch_bounds__(256) void absmax_kernel(const uint16_t* __restrict__ x, int64_t ldx,
+                                                     unsigned int* __restrict__ ws_row,
+                                                     unsigned int* __restrict__ ws_col, int64_t R, int C) {
     constexpr int NR = TR / 8;
-    __shared__ __attribute__((aligned(16))) float part[4][256];
+    __shared__ uint4 part[4][32];  // [wave][chunk]: 8 column maxima (u16) per chunk
+    __shared__ uint32_t rowpart[WITH_ROWS ? TR : 1];  // row maxima of the tile (fp32 bit patterns)
     const int tid = threadIdx.x;
     const int cc = tid & 31, rg = tid >> 5;
     const int c0 = blockIdx.x * 256 + cc * 8;
     const int64_t r0 = (int64_t)blockIdx.y * TR;
-    float m[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    float rmax[NR];
+    uint32_t m[4] = {0, 0, 0, 0};  // columns c0 + 2k (low half) and c0 + 2k + 1 (high half)
+    uint32_t rmax[NR];
 #pragma unroll
-    for (int i = 0; i < NR; ++i) rmax[i] = 0.0f;
+    for (int i = 0; i < NR; ++i) rmax[i] = 0;
     if (c0 < C) {
         uint4 v[NR];
 #pragma unroll
@@ -550,32 +523,51 @@ __global__ __launch_bounds__(256) void rowcol_absmax_kernel(const uint16_t* __re
             v[i] = *reinterpret_cast<const uint4*>(x + (r0 + rg + 8 * i) * ldx + c0);
 #pragma unroll
         for (int i = 0; i < NR; ++i) {
-            const float e0 = fabsf(bf16_lo(v[i].x)), e1 = fabsf(bf16_hi(v[i].x)), e2 = fabsf(bf16_lo(v[i].y)),
-                        e3 = fabsf(bf16_hi(v[i].y)), e4 = fabsf(bf16_lo(v[i].z)), e5 = fabsf(bf16_hi(v[i].z)),
-                        e6 = fabsf(bf16_lo(v[i].w)), e7 = fabsf(bf16_hi(v[i].w));
-            m[0] = fmaxf(m[0], e0); m[1] = fmaxf(m[1], e1); m[2] = fmaxf(m[2], e2); m[3] = fmaxf(m[3], e3);
-            m[4] = fmaxf(m[4], e4); m[5] = fmaxf(m[5], e5); m[6] = fmaxf(m[6], e6); m[7] = fmaxf(m[7], e7);
-            rmax[i] = fmaxf(fmaxf(fmaxf(e0, e1), fmaxf(e2, e3)), fmaxf(fmaxf(e4, e5), fmaxf(e6, e7)));
+            const uint32_t a0 = v[i].x & 0x7fff7fffu, a1 = v[i].y & 0x7fff7fffu, a2 = v[i].z & 0x7fff7fffu,
+                           a3 = v[i].w & 0x7fff7fffu;
+            m[0] = pk_max_u16(m[0], a0);
+            m[1] = pk_max_u16(m[1], a1);
+            m[2] = pk_max_u16(m[2], a2);
+            m[3] = pk_max_u16(m[3], a3);
+            if (WITH_ROWS) rmax[i] = pk_max_u16(pk_max_u16(a0, a1), pk_max_u16(a2, a3));
         }
     }
-    // row maxima: over the 32 lanes (tid % 32) that hold the same rows
+    if (WITH_ROWS) {
+        // over the 32 lanes (tid % 32) that hold the same rows: quad_perm lane^1, lane^2,
+        // row_half_mirror, row_mirror, row_bcast:15 into rows 1 and 3 -> valid in lanes 16-31, 48-63
+        // (one step for all rows at a time: the chains are independent and interleave)
 #pragma unroll
-    for (int i = 0; i < NR; ++i) {
-        const float a = half_wave_max_hi(rmax[i]);
-        if (cc == 16) atomicMax(ws_row + r0 + rg + 8 * i, __float_as_uint(a));
-    }
-    // column maxima: the two half-waves of a wave first, then the four waves through LDS
+        for (int i = 0; i < NR; ++i) rmax[i] = dpp_pk_max_u16<0xB1>(rmax[i]);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) m[e] = pair32_max(m[e]);
-    if ((tid & 32) == 0) {
-        float4* dst = reinterpret_cast<float4*>(&part[tid >> 6][cc * 8]);
-        dst[0] = make_float4(m[0], m[1], m[2], m[3]);
-        dst[1] = make_float4(m[4], m[5], m[6], m[7]);
+        for (int i = 0; i < NR; ++i) rmax[i] = dpp_pk_max_u16<0x4E>(rmax[i]);
+#pragma unroll
+        for (int i = 0; i < NR; ++i) rmax[i] = dpp_pk_max_u16<0x141>(rmax[i]);
+#pragma unroll
+        for (int i = 0; i < NR; ++i) rmax[i] = dpp_pk_max_u16<0x140>(rmax[i]);
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+            const uint32_t a = dpp_pk_max_u16<0x142, 0xA>(rmax[i]);
+            if (cc == 16 + i) rowpart[rg + 8 * i] = max(a & 0xffffu, a >> 16) << 16;
+        }
     }
+#if defined(__HIP_DEVICE_COMPILE__)
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {  // lanes l and l ^ 32 hold the same columns
+        const auto r = __builtin_amdgcn_permlane32_swap(m[k], m[k], false, false);
+        m[k] = pk_max_u16(r[0], r[1]);
+    }
+#endif
+    if ((tid & 32) == 0) part[tid >> 6][cc] = make_uint4(m[0], m[1], m[2], m[3]);
     __syncthreads();
-    const float a = fmaxf(fmaxf(part[0][tid], part[1][tid]), fmaxf(part[2][tid], part[3][tid]));
+    // the tile's rows are consecutive words of ws_row: one atomic instruction for all of them
+    // (an instruction per row and half-wave, two lanes each, measured 2.5 us slower on 8192 x 4096)
+    if (WITH_ROWS && tid < TR) atomicMax(ws_row + r0 + tid, rowpart[tid]);
+    const uint32_t* pw = reinterpret_cast<const uint32_t*>(part);  // dword j of a wave's row: columns 2j, 2j + 1
+    const uint32_t u = pk_max_u16(pk_max_u16(pw[tid >> 1], pw[128 + (tid >> 1)]),
+                                  pk_max_u16(pw[256 + (tid >> 1)], pw[384 + (tid >> 1)]));
+    const uint32_t a = (tid & 1) ? (u >> 16) : (u & 0xffffu);
     const int c = blockIdx.x * 256 + tid;
-    if (c < C) atomicMax(ws_col + c, __float_as_uint(a));
+    if (c < C) atomicMax(ws_col + c, a << 16);
 }
 
 // Quantise a 128x128 tile of x twice: with one scale per ROW into q (same orientation) and
@@ -740,7 +732,7 @@ extern "C" int ti8_quant_col_t(const void* x, int64_t ldx, int8_t* qT, int64_t l
     if (!aligned16(x) || !aligned16(qT) || (ldx % 8) || (ldqt % 16))
         return fail(TI8_ERR_ALIGN, "ti8_quant_col_t: pointers must be 16-byte aligned and strides multiples of 16 bytes");
     const int64_t ntiles = (R / 128) * (C / 128);
-    if (ntiles > 0x7fffffffLL || R / 128 > 65535) return fail(TI8_ERR_SHAPE, "ti8_quant_col_t: too many tiles");
+    if (ntiles > 0x7fffffffLL || R / ABSMAX_ROWS > 65535) return fail(TI8_ERR_SHAPE, "ti8_quant_col_t: too many tiles");
     hipStream_t st = static_cast<hipStream_t>(stream);
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     unsigned int* wsu = reinterpret_cast<unsigned int*>(ws);
@@ -755,8 +747,8 @@ extern "C" int ti8_quant_col_t(const void* x, int64_t ldx, int8_t* qT, int64_t l
                            qT, (int64_t)0, ldqt, s, (int64_t)0, (int64_t)0, (int64_t)0, nrb, ncb, mode, wsu);
         return check_launch("ti8_quant_col_t");
     }
-    hipLaunchKernelGGL(col_absmax_kernel, dim3((unsigned)((C + 255) / 256), (unsigned)(R / 128)), dim3(256), 0, st, xp,
-                       ldx, wsu, R, (int)C);
+    hipLaunchKernelGGL((absmax_kernel<ABSMAX_ROWS, false>), dim3((unsigned)((C + 255) / 256), (unsigned)(R / ABSMAX_ROWS)),
+                       dim3(256), 0, st, xp, ldx, (unsigned int*)nullptr, wsu, R, (int)C);
     hipLaunchKernelGGL(quant_col_t_kernel, dim3((unsigned)ntiles), dim3(256), 0, st, xp, ldx, qT, ldqt, s, ws,
                        (int)(C / 128), mode);
     return check_launch("ti8_quant_col_t");
@@ -776,13 +768,13 @@ extern "C" int ti8_quant_row_col_t(const void* x, int64_t ldx, int8_t* q, int64_
     if (!aligned16(x) || !aligned16(q) || !aligned16(qT) || (ldx % 8) || (ldq % 16) || (ldqt % 16))
         return fail(TI8_ERR_ALIGN, "%s: pointers must be 16-byte aligned and strides multiples of 16 bytes", fn);
     const int64_t ntiles = (R / 128) * (C / 128);
-    if (ntiles > 0x7fffffffLL || R / 128 > 65535 || R + C > 0x7fffffffLL) return fail(TI8_ERR_SHAPE, "%s: too many tiles", fn);
+    if (ntiles > 0x7fffffffLL || R / ABSMAX_ROWS > 65535 || R + C > 0x7fffffffLL) return fail(TI8_ERR_SHAPE, "%s: too many tiles", fn);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     unsigned int* wsu = reinterpret_cast<unsigned int*>(ws);   // [R row maxima][C column maxima]
     hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((R + C + 255) / 256)), dim3(256), 0, st, wsu, (int)(R + C), 0u);
-    hipLaunchKernelGGL(rowcol_absmax_kernel<ABSMAX_ROWS>, dim3((unsigned)((C + 255) / 256), (unsigned)(R / ABSMAX_ROWS)), dim3(256), 0, st, xp,
-                       ldx, wsu, wsu + R, R, (int)C);
+    hipLaunchKernelGGL((absmax_kernel<ABSMAX_ROWS, true>), dim3((unsigned)((C + 255) / 256), (unsigned)(R / ABSMAX_ROWS)),
+                       dim3(256), 0, st, xp, ldx, wsu, wsu + R, R, (int)C);
     hipLaunchKernelGGL(quant_rowcol_kernel, dim3((unsigned)ntiles), dim3(256), 0, st, xp, ldx, q, ldq, s_row, qT, ldqt,
                        s_col, ws, ws + R, (int)(C / 128), mode);
     return check_launch(fn);

@@ -73,17 +73,6 @@ __device__ __forceinline__ float half_wave_max_hi(float v) {
     return dpp_max<0x142, 0xA>(v);
 }
 
-// max of v over the lane pair (l, l ^ 32), in both lanes (v_permlane32_swap: one cross-half move)
-__device__ __forceinline__ float pair32_max(float v) {
-#if defined(__HIP_DEVICE_COMPILE__)
-    const unsigned u = __float_as_uint(v);
-    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-#else
-    return v;
-#endif
-}
-
 // max over the 16 lanes of a DPP row, in all of them
 __device__ __forceinline__ float row16_max(float v) {
     v = dpp_max<0xB1>(v);
