@@ -43,8 +43,10 @@ enum ti8_qflags {
                                the same bytes on every finite input, |x*scale| <= 127 by construction */
     TI8_Q_EPS_ADD = 2,      /* amax + 1e-5 (fused kernels) instead of max(amax, 1e-4) */
     TI8_Q_SCALE_BF16 = 4,   /* round the stored scale through bf16 (TileLang copy) */
-    TI8_Q_HAD128 = 8        /* ti8_quant_row only: rotate every 128-column group by H_128 (fp32
+    TI8_Q_HAD128 = 8,       /* ti8_quant_row only: rotate every 128-column group by H_128 (fp32
                                butterflies, one bf16 rounding) before the absmax */
+    TI8_Q_WS_PINGPONG = 16, /* ti8_quant_row_col_t only: two-part workspace that the calls keep clear for each */
+    TI8_Q_WS_SECOND = 32    /* other, and which part this call works in (see there) */
 };
 
 /* which number is written to the scale tensor */
@@ -167,6 +169,11 @@ int ti8_quant_col_t(const void* x, int64_t ldx, int8_t* qT, int64_t ldqt, float*
  *
  *   x bf16 [R][C] (ldx) -> q int8 [R][C] (ldq), s_row[R];  qT int8 [C][R] (ldqt), s_col[C]
  *   ws: workspace of R + C floats, contents undefined afterwards.
+ *   With TI8_Q_WS_PINGPONG ws has two parts of R + C floats each and the call works in the first,
+ *   or with TI8_Q_WS_SECOND in the second: that part must be ALL ZERO on entry, and the call
+ *   zero-fills the other part.  Zero-fill the buffer once after allocating it and alternate
+ *   TI8_Q_WS_SECOND from call to call (same R and C, calls in stream order, not overlapping):
+ *   then no call needs the launch that clears the workspace.
  * R % 128 == 0, C % 128 == 0. */
 int ti8_quant_row_col_t(const void* x, int64_t ldx, int8_t* q, int64_t ldq, float* s_row,
                         int8_t* qT, int64_t ldqt, float* s_col, float* ws,

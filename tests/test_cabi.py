@@ -68,6 +68,10 @@ FAKE = 0x10000  # a 16-byte aligned non-null "device pointer"; validation never 
     (("ti8_quant_row_col_t", FAKE, 256, FAKE, 256, FAKE, FAKE, 128, FAKE, None, 128, 256, 0, 0, None), 1, "required"),
     (("ti8_quant_row_col_t", FAKE, 256, FAKE, 256, FAKE, FAKE, 128, FAKE, FAKE, 128, 200, 0, 0, None), 2, "C%128"),
     (("ti8_quant_row_col_t", FAKE, 256, FAKE, 128, FAKE, FAKE, 128, FAKE, FAKE, 128, 256, 0, 0, None), 2, "leading dimension"),
+    (("ti8_quant_row_col_t", FAKE, 256, FAKE, 256, FAKE, FAKE, 128, FAKE, FAKE, 128, 200, 16, 0, None), 2, "C%128"),
+    (("ti8_quant_row_col_t", FAKE, 256, FAKE, 256, FAKE, FAKE, 128, FAKE, FAKE, 128, 256, 32, 0, None), 4, "TI8_Q_WS_PINGPONG"),
+    (("ti8_quant_row_col_t", FAKE, 256, FAKE, 256, FAKE, FAKE, 128, FAKE, FAKE, 128, 256, 8, 0, None), 4, "Hadamard"),
+    (("ti8_quant_row", FAKE, 4096, FAKE, 4096, FAKE, 4, 4096, 0, 16, 0, None), 4, "unknown quantiser flag"),
     (("ti8_fwht", FAKE, 384, FAKE, 384, 4, 384, 384, 1.0, None), 2, "power of two"),
     (("ti8_fwht", FAKE, 256, FAKE, 256, 4, 256, 64, 1.0, None), 2, "power of two"),
     (("ti8_gemm_i8_nt", FAKE, 0, 128, FAKE, 0, 128, FAKE, 0, 128, FAKE, 0, 0, 1, 0, FAKE, 0, 0, 1, 0,

@@ -138,6 +138,33 @@ def test_row_and_col_quant_in_one_go(T, dev, R, C):
         assert bits_equal(q, qo) and bits_equal(s_row, so.flatten()) and bits_equal(qT, qTo) and bits_equal(s_col, sTo.flatten())
 
 
+def test_row_and_col_quant_workspace_modes(T, dev):
+    """The two-part workspace of ti8_quant_row_col_t (TI8_Q_WS_PINGPONG: a call works in one part and
+    clears the other for the next call) gives the same bits as the one the library clears itself,
+    call after call, and the part a call does not work in is all zero when it returns."""
+    R, C = 384, 640
+    ws2 = torch.zeros(2 * (R + C), dtype=torch.float32, device=dev)
+    for call, seed in enumerate((1, 2, 3, 4)):
+        x = randn_bf16(make_gen(seed), R, C).to(dev)
+        outs = []
+        for flags, ws in ((T._lib.Q_WS_PINGPONG | (T._lib.Q_WS_SECOND if call & 1 else 0), ws2),
+                          (0, torch.full((R + C,), float("nan"), dtype=torch.float32, device=dev))):
+            q = torch.empty((R, C), dtype=torch.int8, device=dev)
+            qT = torch.empty((C, R), dtype=torch.int8, device=dev)
+            s_row = torch.empty(R, dtype=torch.float32, device=dev)
+            s_col = torch.empty(C, dtype=torch.float32, device=dev)
+            T._lib.call("ti8_quant_row_col_t", x.data_ptr(), x.stride(0), q.data_ptr(), C, s_row.data_ptr(),
+                        qT.data_ptr(), R, s_col.data_ptr(), ws.data_ptr(), R, C, T._lib.Q_CLAMP | flags, 0,
+                        torch.cuda.current_stream().cuda_stream)
+            outs.append((q, s_row, qT, s_col))
+        torch.cuda.synchronize()
+        assert all(bits_equal(a, b) for a, b in zip(*outs))
+        halves = ws2.view(torch.int32).view(2, R + C)
+        assert not halves[1 - (call & 1)].any() and halves[call & 1].any()
+        q0, s0 = T.ops.quant_row(x, clamp=True)
+        assert torch.equal(outs[0][0], q0) and bits_equal(outs[0][1], s0)
+
+
 @pytest.mark.parametrize("n,cols", [(128, 384), (128, 4096), (256, 256), (512, 1536), (1024, 2048), (2048, 2048),
                                     (4096, 4096), (8192, 8192), (16384, 16384), (32768, 32768)])
 def test_fwht(T, dev, n, cols):

@@ -577,7 +577,8 @@ __global__ __launch_bounds__(256) void quant_rowcol_kernel(const uint16_t* __res
                                                            float* __restrict__ s_row, int8_t* __restrict__ qT,
                                                            int64_t ldqt, float* __restrict__ s_col,
                                                            const float* __restrict__ ws_row,
-                                                           const float* __restrict__ ws_col, int ncb, QMode mode) {
+                                                           const float* __restrict__ ws_col,
+                                                           float* __restrict__ ws_next, int64_t R, int ncb, QMode mode) {
     __shared__ uint32_t tileT[128 * 33];
     __shared__ __attribute__((aligned(16))) float sc[256];  // [0,128): row scales, [128,256): column scales
     const int cb = blockIdx.x % ncb;
@@ -598,6 +599,8 @@ __global__ __launch_bounds__(256) void quant_rowcol_kernel(const uint16_t* __res
         const bool is_row = tid < 128;
         const int idx = tid & 127;
         const int64_t at = is_row ? (int64_t)rb * 128 + idx : (int64_t)cb * 128 + idx;
+        // two-part workspace: clear the part that the next call will collect its maxima in
+        if (ws_next && (is_row ? cb == 0 : rb == 0)) ws_next[is_row ? at : R + at] = 0.0f;
         const float amax = amax_floor(is_row ? ws_row[at] : ws_col[at], mode.eps_add);
         const float scale = 127.0f / amax;
         sc[tid] = scale;
@@ -758,8 +761,10 @@ extern "C" int ti8_quant_row_col_t(const void* x, int64_t ldx, int8_t* q, int64_
                                    int64_t ldqt, float* s_col, float* ws, int64_t R, int64_t C, int qflags,
                                    int inv_mode, ti8_stream_t stream) {
     const char* fn = "ti8_quant_row_col_t";
+    const bool pingpong = (qflags & TI8_Q_WS_PINGPONG) != 0, second = (qflags & TI8_Q_WS_SECOND) != 0;
+    if (second && !pingpong) return fail(TI8_ERR_MODE, "%s: TI8_Q_WS_SECOND needs TI8_Q_WS_PINGPONG", fn);
     QMode mode;
-    if (int e = parse_mode(qflags, inv_mode, &mode)) return e;
+    if (int e = parse_mode(qflags & ~(TI8_Q_WS_PINGPONG | TI8_Q_WS_SECOND), inv_mode, &mode)) return e;
     if (qflags & TI8_Q_HAD128) return fail(TI8_ERR_MODE, "%s: the Hadamard rotation is not offered here", fn);
     if (!x || !q || !s_row || !qT || !s_col || !ws) return fail(TI8_ERR_NULL, "%s: x, q, s_row, qT, s_col and ws are required", fn);
     if (R <= 0 || C <= 0 || R % 128 || C % 128 || C > 0x7fffffffLL)
@@ -771,12 +776,18 @@ extern "C" int ti8_quant_row_col_t(const void* x, int64_t ldx, int8_t* q, int64_
     if (ntiles > 0x7fffffffLL || R / ABSMAX_ROWS > 65535 || R + C > 0x7fffffffLL) return fail(TI8_ERR_SHAPE, "%s: too many tiles", fn);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const uint16_t* xp = static_cast<const uint16_t*>(x);
-    unsigned int* wsu = reinterpret_cast<unsigned int*>(ws);   // [R row maxima][C column maxima]
-    hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((R + C + 255) / 256)), dim3(256), 0, st, wsu, (int)(R + C), 0u);
+    float* ws_next = nullptr;  // [R row maxima][C column maxima], once or twice
+    if (pingpong) {
+        ws_next = second ? ws : ws + R + C;
+        ws = second ? ws + R + C : ws;
+    }
+    unsigned int* wsu = reinterpret_cast<unsigned int*>(ws);
+    if (!pingpong)
+        hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((R + C + 255) / 256)), dim3(256), 0, st, wsu, (int)(R + C), 0u);
     hipLaunchKernelGGL((absmax_kernel<ABSMAX_ROWS, true>), dim3((unsigned)((C + 255) / 256), (unsigned)(R / ABSMAX_ROWS)),
                        dim3(256), 0, st, xp, ldx, wsu, wsu + R, R, (int)C);
     hipLaunchKernelGGL(quant_rowcol_kernel, dim3((unsigned)ntiles), dim3(256), 0, st, xp, ldx, q, ldq, s_row, qT, ldqt,
-                       s_col, ws, ws + R, (int)(C / 128), mode);
+                       s_col, ws, ws + R, ws_next, R, (int)(C / 128), mode);
     return check_launch(fn);
 }
 

@@ -9,7 +9,7 @@ import torch
 
 from . import _lib
 from ._lib import (COMBINE_DIV_PROD, COMBINE_MUL_MUL, COMBINE_MUL_PROD, GEMM_LARGE_TILES, GEMM_SKINNY, GEMM_STRICT, GEMM_TILED, INV_AMAX_DIV_127,
-                   INV_AMAX_MUL_RCP127, INV_MULTIPLIER, INV_RCP_OF_SCALE, Q_CLAMP, Q_EPS_ADD, Q_HAD128, Q_SCALE_BF16,
+                   INV_AMAX_MUL_RCP127, INV_MULTIPLIER, INV_RCP_OF_SCALE, Q_CLAMP, Q_EPS_ADD, Q_HAD128, Q_SCALE_BF16, Q_WS_PINGPONG, Q_WS_SECOND,
                    SCALE_BLOCK128, SCALE_BLOCK_K256, SCALE_ROW, SCALE_ROW_K128)
 
 __all__ = ["quant_block", "quant_block_had128", "quant_row", "quant_col_t", "quant_row_col_t", "fwht", "gemm_i8_nt", "gemm_i8_nt_i32"]
@@ -169,10 +169,34 @@ def quant_row_col_t(x, *, clamp=True, inv_mode=INV_RCP_OF_SCALE):
     qT = torch.empty((C, R), dtype=torch.int8, device=x.device)
     s_row = torch.empty((R,), dtype=torch.float32, device=x.device)
     s_col = torch.empty((C,), dtype=torch.float32, device=x.device)
-    ws = torch.empty((R + C,), dtype=torch.float32, device=x.device)
+    flags = _qflags(clamp, False, False)
+    stream = _stream()
+    if torch.cuda.is_current_stream_capturing():
+        # a replayed call cannot alternate: plain workspace, cleared by the library on every replay
+        ws = torch.empty((R + C,), dtype=torch.float32, device=x.device)
+    else:
+        slot = _pingpong_workspace(x.device, stream, R, C)
+        ws = slot[0]
+        flags |= Q_WS_PINGPONG | (Q_WS_SECOND if slot[1] else 0)
+        slot[1] ^= 1
     _lib.call("ti8_quant_row_col_t", x.data_ptr(), x.stride(0), q.data_ptr(), C, s_row.data_ptr(), qT.data_ptr(), R,
-              s_col.data_ptr(), ws.data_ptr(), R, C, _qflags(clamp, False, False), inv_mode, _stream())
+              s_col.data_ptr(), ws.data_ptr(), R, C, flags, inv_mode, stream)
     return q, s_row, qT, s_col
+
+
+# Two-part workspaces of quant_row_col_t: a call collects its maxima in one part and clears the
+# other for the next call, so no call needs a launch that clears memory.  One buffer (and the
+# part to use next) per device, stream and shape: calls on one stream run in order and can share
+# it; calls on different streams may overlap and get different buffers.
+_PINGPONG_WS = {}
+
+
+def _pingpong_workspace(device, stream, R, C):
+    key = (device.index, stream, R, C)
+    slot = _PINGPONG_WS.get(key)
+    if slot is None:
+        slot = _PINGPONG_WS[key] = [torch.zeros((2 * (R + C),), dtype=torch.float32, device=device), 0]
+    return slot
 
 
 def fwht(x, n=None, scale=1.0):
