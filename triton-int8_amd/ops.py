@@ -178,9 +178,10 @@ def quant_row_col_t(x, *, clamp=True, inv_mode=INV_RCP_OF_SCALE):
         slot = _pingpong_workspace(x.device, stream, R, C)
         ws = slot[0]
         flags |= Q_WS_PINGPONG | (Q_WS_SECOND if slot[1] else 0)
-        slot[1] ^= 1
     _lib.call("ti8_quant_row_col_t", x.data_ptr(), x.stride(0), q.data_ptr(), C, s_row.data_ptr(), qT.data_ptr(), R,
               s_col.data_ptr(), ws.data_ptr(), R, C, flags, inv_mode, stream)
+    if flags & Q_WS_PINGPONG:
+        slot[1] ^= 1   # only once the launches are queued: a rejected call leaves both parts as they were
     return q, s_row, qT, s_col
 
 
