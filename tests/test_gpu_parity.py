@@ -3,6 +3,7 @@
 Bar: int8 tensors, scales and int32 accumulators bit-exact; bf16 outputs bit-exact in
 strict mode and within rel-err <= 1e-2 (REL_TOL, the tolerance the task states) otherwise;
 the reference's own acceptance bar calc_diff < 1e-3 against a bf16 matmul."""
+import numpy as np
 import pytest
 import torch
 
@@ -117,7 +118,7 @@ def test_col_quant_transposed(T, dev):
     assert bits_equal(qT, qo) and bits_equal(s, so)
 
 
-@pytest.mark.parametrize("R,C", [(128, 128), (256, 384), (384, 4096), (1024, 14336)])
+@pytest.mark.parametrize("R,C", [(128, 128), (256, 384), (384, 4096), (1024, 14336), (8192, 4096)])
 def test_row_and_col_quant_in_one_go(T, dev, R, C):
     """ti8_quant_row_col_t = ti8_quant_row + ti8_quant_col_t on the same operand, bit for bit (and
     therefore equal to the oracle's per-token quantiser applied to x and to x^T)."""
@@ -131,6 +132,11 @@ def test_row_and_col_quant_in_one_go(T, dev, R, C):
         q0, s0 = T.ops.quant_row(xd, clamp=True, inv_mode=inv_mode)
         qT0, sT0 = T.ops.quant_col_t(xd, clamp=True, inv_mode=inv_mode)
         assert torch.equal(q, q0) and bits_equal(s_row, s0) and torch.equal(qT, qT0) and bits_equal(s_col, sT0)
+        if inv_mode == 1:   # scale = amax / 127: the maxima against torch's own reduction, at every size
+            a = xd.float().abs()   # numpy does the IEEE division (torch multiplies by the reciprocal of a scalar)
+            for got, dim in ((s_row, 1), (s_col, 0)):
+                want = a.amax(dim=dim).clamp_min(1e-4).cpu().numpy() / np.float32(127.0)
+                assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
     if R * C <= 384 * 4096:
         qo, so = obf.token_quant(x, True)
         qTo, sTo = obf.token_quant(x.t().contiguous(), True)
