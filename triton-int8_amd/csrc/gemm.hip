@@ -15,6 +15,7 @@
 // operand and the 16 bytes k = 16*(l / 32) .. +15 of the 32-deep slice (the same map
 // for both operands, which is all an NT dot product needs); result register r of lane
 // l is C[8*(r/4) + 4*(l/32) + r%4][l % 32] with rows from A and columns from B.
+#include <type_traits>
 #include "gemm_args.h"
 
 namespace ti8 {
@@ -419,72 +420,99 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
     constexpr int NRR = 32 / RPI;                        // rows of a 32-row block per lane
     const float* prow = g.sa.p + batch * g.sa.bs;        // per-row scales of A (unused pointer otherwise)
     const int64_t rstride = row_part ? g.sa.rs : 0;
+    // Everything that does not change from element to element is settled here, so that an
+    // element costs its multiplications and nothing else: operands without a row / column scale
+    // vector multiply by 1 (exact), the rarely used extra factors pick a copy of the loop below
+    // (compile-time flag, one uniform branch), and the output address advances by whole rows.
+    float cm[4];
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-        const int mbase = m0 + (wm * TM + i) * 32;
-        // the block's row scales: all loads go out before the slab traffic, nothing waits per row
-        float rowv[NRR];
-        if (EPI == EPI_ROWS || FAST) {
+    for (int c = 0; c < 4; ++c) cm[c] = col_part ? coln[c] : 1.0f;
+    const int row0 = m0 + wm * TM * 32 + rb_row;          // this lane's first output row
+    const bool col_ok = ncol0 < g.N;                      // N is a multiple of 4: a lane's 4 columns are all in or all out
+    const int64_t c_off = (int64_t)batch * g.bsc + (int64_t)row0 * g.ldc + ncol0;
+    const int64_t c_step = (int64_t)RPI * g.ldc;          // uniform: the output address advances by scalar adds
+    // row scales: row0 + d for d = 0, RPI, ... clamped to the last row; d * stride is uniform and
+    // the clamp is one v_min against this lane's limit (32-bit offsets: 128 rows x stride)
+    const float* prow0 = prow + (int64_t)min(row0, g.M - 1) * rstride;
+    const uint32_t rs32 = static_cast<uint32_t>(rstride);
+    const uint32_t r_lim = static_cast<uint32_t>(max(g.M - 1 - row0, 0)) * rs32;
+    auto store_tile = [&](auto extra_tag) {
+        constexpr bool EXTRA = decltype(extra_tag)::value;  // EPI_ROWS: post_scale, promotion: out_scale
+        int64_t off = c_off;
 #pragma unroll
-            for (int k = 0; k < NRR; ++k) rowv[k] = prow[(int64_t)min(mbase + rb_row + k * RPI, g.M - 1) * rstride];
-        }
+        for (int i = 0; i < TM; ++i) {
+            // the block's row scales: all loads go out before the slab traffic, nothing waits per row
+            float rm[NRR];
+            if (EPI == EPI_ROWS || FAST) {
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int rr = 8 * (r >> 2) + 4 * fr_half + (r & 3);
-                const uint32_t bits = PROMOTE ? __float_as_uint(accf[PROMOTE ? i : 0][PROMOTE ? j : 0][r])
-                                              : static_cast<uint32_t>(acc[i][j][r]);
-                slab[rr * WCOLS + j * 32 + fr_row] = bits;
+                for (int k = 0; k < NRR; ++k) rm[k] = prow0[min(static_cast<uint32_t>(i * 32 + k * RPI) * rs32, r_lim)];
             }
-        // same wave reads what it wrote: an LDS counter wait is enough, no barrier
-        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
-        __builtin_amdgcn_wave_barrier();
 #pragma unroll
-        for (int k = 0; k < NRR; ++k) {
-            const int rr = rb_row + k * RPI;
-            const int m = mbase + rr;
-            const uint4 w = *reinterpret_cast<const uint4*>(slab + rr * WCOLS + rb_col);
-            if (m >= g.M || ncol0 >= g.N) continue;  // N is a multiple of 4: a lane's 4 columns are all in or all out
-            const int64_t off = (int64_t)batch * g.bsc + (int64_t)m * g.ldc + ncol0;
-            if (EPI == EPI_I32) {
-                *reinterpret_cast<uint4*>(reinterpret_cast<int32_t*>(g.C) + off) = w;
-                continue;
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int rr = 8 * (r >> 2) + 4 * fr_half + (r & 3);
+                    const uint32_t bits = PROMOTE ? __float_as_uint(accf[PROMOTE ? i : 0][PROMOTE ? j : 0][r])
+                                                  : static_cast<uint32_t>(acc[i][j][r]);
+                    slab[rr * WCOLS + j * 32 + fr_row] = bits;
+                }
+            if (FAST) {
+                if (divide && row_part) {
+#pragma unroll
+                    for (int k = 0; k < NRR; ++k) {
+                        asm volatile("" : "+v"(rm[k]));   // not to be speculated: keeps the divisions out of the common path
+                        rm[k] = 1.0f / rm[k];
+                    }
+                }
+#pragma unroll
+                for (int k = 0; k < NRR; ++k) rm[k] = row_part ? rm[k] : 1.0f;
             }
-            float t[4];
-            const uint32_t wb[4] = {w.x, w.y, w.z, w.w};
-            if (EPI == EPI_ROWS) {
-                const float rowm = rowv[k];
+            // same wave reads what it wrote: an LDS counter wait is enough, no barrier
+            __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int k = 0; k < NRR; ++k, off += c_step) {
+                const int rr = rb_row + k * RPI;
+                const uint4 w = *reinterpret_cast<const uint4*>(slab + rr * WCOLS + rb_col);
+                if (row0 + i * 32 + k * RPI >= g.M || !col_ok) continue;
+                if (EPI == EPI_I32) {
+                    *reinterpret_cast<uint4*>(reinterpret_cast<int32_t*>(g.C) + off) = w;
+                    continue;
+                }
+                float t[4];
+                const uint32_t wb[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
-                    float v = static_cast<float>(static_cast<int32_t>(wb[c])) * rowm;
-                    v = v * coln[c];
-                    if (g.post_scale != 0.0f) v = __uint_as_float(f32_to_bf16_bits(v) << 16) * g.post_scale;
+                    float v;
+                    if (EPI == EPI_ROWS) {
+                        v = static_cast<float>(static_cast<int32_t>(wb[c])) * rm[k];
+                        v = v * cm[c];
+                        if (EXTRA) v = __uint_as_float(pack_bf16x2(v, 0.0f) << 16) * g.post_scale;
+                    } else {
+                        v = __uint_as_float(wb[c]);
+                        if (FAST) {
+                            v = v * rm[k];
+                            v = v * cm[c];
+                        }
+                        if (EXTRA) v = v * g.out_scale;
+                    }
                     t[c] = v;
                 }
-            } else {
-                float rowm = 1.0f;
-                if (FAST && row_part) {
-                    rowm = rowv[k];
-                    if (divide) rowm = 1.0f / rowm;
-                }
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    float v = __uint_as_float(wb[c]);
-                    if (FAST && row_part) v = v * rowm;
-                    if (FAST && col_part) v = v * coln[c];
-                    if (g.out_scale != 1.0f) v = v * g.out_scale;
-                    t[c] = v;
-                }
+                uint2 o;
+                o.x = pack_bf16x2(t[0], t[1]);
+                o.y = pack_bf16x2(t[2], t[3]);
+                *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(g.C) + off) = o;
             }
-            uint2 o;
-            o.x = pack_bf16x2(t[0], t[1]);
-            o.y = pack_bf16x2(t[2], t[3]);
-            *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(g.C) + off) = o;
+            static_assert(NRR * RPI == 32, "a block row advances the output by 32 rows");
+            __builtin_amdgcn_s_waitcnt(0xc07f);
+            __builtin_amdgcn_wave_barrier();
         }
-        __builtin_amdgcn_s_waitcnt(0xc07f);
-        __builtin_amdgcn_wave_barrier();
-    }
+    };
+    const bool extra = (EPI == EPI_ROWS) ? (g.post_scale != 0.0f) : (EPI != EPI_I32 && g.out_scale != 1.0f);
+    if (extra)
+        store_tile(std::true_type{});
+    else
+        store_tile(std::false_type{});
 }
 
 template <int BM, int BN, int WM, int WN, int EPI>
