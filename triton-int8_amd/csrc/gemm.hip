@@ -436,14 +436,15 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
     const float* prow0 = prow + (int64_t)min(row0, g.M - 1) * rstride;
     const uint32_t rs32 = static_cast<uint32_t>(rstride);
     const uint32_t r_lim = static_cast<uint32_t>(max(g.M - 1 - row0, 0)) * rs32;
-    auto store_tile = [&](auto extra_tag) {
+    auto store_tile = [&](auto extra_tag, auto mult_tag) {
         constexpr bool EXTRA = decltype(extra_tag)::value;  // EPI_ROWS: post_scale, promotion: out_scale
+        constexpr bool MULT = decltype(mult_tag)::value;    // promotion: some operand has a row / column scale vector
         int64_t off = c_off;
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
             // the block's row scales: all loads go out before the slab traffic, nothing waits per row
             float rm[NRR];
-            if (EPI == EPI_ROWS || FAST) {
+            if (EPI == EPI_ROWS || (FAST && MULT)) {
 #pragma unroll
                 for (int k = 0; k < NRR; ++k) rm[k] = prow0[min(static_cast<uint32_t>(i * 32 + k * RPI) * rs32, r_lim)];
             }
@@ -456,7 +457,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
                                                   : static_cast<uint32_t>(acc[i][j][r]);
                     slab[rr * WCOLS + j * 32 + fr_row] = bits;
                 }
-            if (FAST) {
+            if (FAST && MULT) {
                 if (divide && row_part) {
 #pragma unroll
                     for (int k = 0; k < NRR; ++k) {
@@ -490,7 +491,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
                         if (EXTRA) v = __uint_as_float(pack_bf16x2(v, 0.0f) << 16) * g.post_scale;
                     } else {
                         v = __uint_as_float(wb[c]);
-                        if (FAST) {
+                        if (FAST && MULT) {
                             v = v * rm[k];
                             v = v * cm[c];
                         }
@@ -509,10 +510,14 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
         }
     };
     const bool extra = (EPI == EPI_ROWS) ? (g.post_scale != 0.0f) : (EPI != EPI_I32 && g.out_scale != 1.0f);
-    if (extra)
-        store_tile(std::true_type{});
-    else
-        store_tile(std::false_type{});
+    const bool mult = FAST && (row_part || col_part);   // block scales on both operands: nothing left to multiply
+    if (extra) {
+        if (mult) store_tile(std::true_type{}, std::true_type{});
+        else store_tile(std::true_type{}, std::false_type{});
+    } else {
+        if (mult) store_tile(std::false_type{}, std::true_type{});
+        else store_tile(std::false_type{}, std::false_type{});
+    }
 }
 
 template <int BM, int BN, int WM, int WN, int EPI>
