@@ -440,14 +440,21 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
         constexpr bool EXTRA = decltype(extra_tag)::value;  // EPI_ROWS: post_scale, promotion: out_scale
         constexpr bool MULT = decltype(mult_tag)::value;    // promotion: some operand has a row / column scale vector
         int64_t off = c_off;
+        // every row scale of the tile is fetched before the first store: loads and stores share
+        // one in-order counter, so a load issued behind a block row's stores could only be waited
+        // for together with those stores
+        float rm_all[TM][NRR];
+        if (EPI == EPI_ROWS || (FAST && MULT)) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int k = 0; k < NRR; ++k) rm_all[i][k] = prow0[min(static_cast<uint32_t>(i * 32 + k * RPI) * rs32, r_lim)];
+        }
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
-            // the block's row scales: all loads go out before the slab traffic, nothing waits per row
             float rm[NRR];
-            if (EPI == EPI_ROWS || (FAST && MULT)) {
 #pragma unroll
-                for (int k = 0; k < NRR; ++k) rm[k] = prow0[min(static_cast<uint32_t>(i * 32 + k * RPI) * rs32, r_lim)];
-            }
+            for (int k = 0; k < NRR; ++k) rm[k] = rm_all[i][k];
 #pragma unroll
             for (int j = 0; j < TN; ++j)
 #pragma unroll
