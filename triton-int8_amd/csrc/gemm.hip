@@ -586,6 +586,9 @@ extern "C" int ti8_gemm_i8_nt(const int8_t* A, int64_t bsa, int64_t lda, const i
     if (int e = check_operands(fn, A, bsa, lda, B, bsb, ldb, C, ldc, batch, M, N, K, M <= 256 ? 32 : 128)) return e;
     if (int e = check_scale(fn, "A", sA, modeA)) return e;
     if (int e = check_scale(fn, "B", sB, modeB)) return e;
+    // the epilogue keeps (row within a tile) * (row stride of A's scales) in 32 bits
+    if (modeA == TI8_SCALE_ROW && (sa_rs < 0 || sa_rs > 0x00ffffff))
+        return fail(TI8_ERR_SHAPE, "%s: row stride of A's scales must be in [0, 2^24)", fn);
     if (combine < 0 || combine > 2) return fail(TI8_ERR_MODE, "%s: unknown combine %d", fn, combine);
     if (gemm_flags & ~(TI8_GEMM_STRICT | TI8_GEMM_TILED | TI8_GEMM_SKINNY | TI8_GEMM_LARGE_TILES)) return fail(TI8_ERR_MODE, "%s: unknown flag 0x%x", fn, gemm_flags);
     if ((gemm_flags & TI8_GEMM_SKINNY) && (gemm_flags & (TI8_GEMM_TILED | TI8_GEMM_LARGE_TILES)))
