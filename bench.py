@@ -227,7 +227,7 @@ def main():
 
     # HBM-side bytes per GEMM launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled on the device
     # copy above (profiles/bench_config2_*_hbm_counters.md); measured for these two schemes
-    traffic = {"block_channel": 257667232, "double_channel": 257689548}.get(args.scheme)
+    traffic = {"block_channel": 257610359, "double_channel": 257689548}.get(args.scheme)
 
     out = {
         "metric": METRIC, "value": round(tops, 2), "unit": "TOPS", "n_gpus": 1, "steps": args.steps,
