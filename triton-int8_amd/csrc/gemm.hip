@@ -197,11 +197,15 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
     for (int j = 0; j < TN; ++j) fb[j] = 1.0f;
     auto load_factors = [&](int kt) {
         const int l = kt & 63, c = kt >> 6;
-        const float v0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fvec[0]), l));
-        const float v1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fvec[1]), l));
-        const float v2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fvec[2]), l));
-        const float v3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fvec[3]), l));
-        f_cur = c == 0 ? v0 : (c == 1 ? v1 : (c == 2 ? v2 : v3));
+        if (g.K <= 64 * 128) {   // the usual case: one register holds every tile's factor
+            f_cur = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fvec[0]), l));
+        } else {
+            const float v0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fvec[0]), l));
+            const float v1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fvec[1]), l));
+            const float v2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fvec[2]), l));
+            const float v3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fvec[3]), l));
+            f_cur = c == 0 ? v0 : (c == 1 ? v1 : (c == 2 ? v2 : v3));
+        }
         if (LANEB) {  // issued before this tile's loads; consumed after its barrier (which waits for them)
 #pragma unroll
             for (int j = 0; j < TN; ++j) fb[j] = pfb[j][(int64_t)kt * g.sb.ks];

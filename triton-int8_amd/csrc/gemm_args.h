@@ -46,9 +46,14 @@ template <int NI>
 __device__ __forceinline__ void issue_tile_loads(const int8_t* base, int64_t stride8, const uint32_t (&voff)[2], int t0,
                                                  int8_t* lds) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the builtin only exists in the device pass
+    // the per-lane offsets are made opaque here so that their widening to 64 bits is not hoisted out
+    // of the caller's loop: instruction selection then sees (uniform base) + zext(32-bit offset) and
+    // uses the SGPR-base addressing form instead of a 64-bit vector add per instruction
+    uint32_t vo[2] = {voff[0], voff[1]};
+    asm volatile("" : "+v"(vo[0]), "+v"(vo[1]));
 #pragma unroll
     for (int i = 0; i < NI; ++i)
-        __builtin_amdgcn_global_load_lds(base + i * stride8 + voff[(t0 + i) & 1], lds + i * 1024, 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(base + i * stride8 + vo[(t0 + i) & 1], lds + i * 1024, 16, 0, 0);
 #else
     (void)base; (void)stride8; (void)voff; (void)t0; (void)lds;
 #endif
