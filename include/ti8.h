@@ -180,6 +180,23 @@ int ti8_quant_row_col_t(const void* x, int64_t ldx, int8_t* q, int64_t ldq, floa
                         int64_t R, int64_t C, int qflags, int inv_mode, ti8_stream_t stream);
 
 /* ---------------------------------------------------------------------------------
+ * ti8_quant_row_col_t for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): same arguments without `ws`,
+ * same bits.  It has no counterpart in the reference.  The row and column maxima are collected in
+ * a fixed array of TI8_NOALLOC_MAX_ROWS_PLUS_COLS floats (256 KiB) that lives in the library's
+ * device image: every GPU the library runs on holds its own copy until the process ends.  The call
+ * allocates and frees nothing; its launches are kernels only (the array is cleared by a fill
+ * kernel), so it may be captured.
+ *   R + C <= TI8_NOALLOC_MAX_ROWS_PLUS_COLS, else TI8_ERR_SHAPE (use the entry point above).
+ *   TI8_Q_WS_PINGPONG / TI8_Q_WS_SECOND are rejected (TI8_ERR_MODE).
+ * All calls on one GPU share that GPU's array: calls that overlap on one GPU (different streams
+ * without ordering between them) race; calls on one stream, or ordered by events, are safe. */
+#define TI8_NOALLOC_MAX_ROWS_PLUS_COLS 65536
+int ti8_quant_row_col_t_noalloc(const void* x, int64_t ldx, int8_t* q, int64_t ldq, float* s_row,
+                                int8_t* qT, int64_t ldqt, float* s_col,
+                                int64_t R, int64_t C, int qflags, int inv_mode, ti8_stream_t stream);
+
+/* ---------------------------------------------------------------------------------
  * Un-normalised Walsh-Hadamard transform along the last dim (Sylvester order):
  * replaces fast_hadamard_transform.hadamard_transform at its call sites
  * (triton/double-channle_fwd32.py:273-274,299-300; triton/double_channel_bwd33.py:

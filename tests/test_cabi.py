@@ -72,6 +72,8 @@ FAKE = 0x10000  # a 16-byte aligned non-null "device pointer"; validation never 
     (("ti8_quant_row_col_t", FAKE, 256, FAKE, 256, FAKE, FAKE, 128, FAKE, FAKE, 128, 256, 32, 0, None), 4, "TI8_Q_WS_PINGPONG"),
     (("ti8_quant_row_col_t", FAKE, 256, FAKE, 256, FAKE, FAKE, 128, FAKE, FAKE, 128, 256, 8, 0, None), 4, "Hadamard"),
     (("ti8_quant_row", FAKE, 4096, FAKE, 4096, FAKE, 4, 4096, 0, 16, 0, None), 4, "unknown quantiser flag"),
+    (("ti8_quant_row_col_t_noalloc", FAKE, 65536, FAKE, 65536, FAKE, FAKE, 128, FAKE, 128, 65536, 0, 0, None), 2, "exceeds"),
+    (("ti8_quant_row_col_t_noalloc", FAKE, 256, FAKE, 256, FAKE, FAKE, 128, FAKE, 128, 256, 16, 0, None), 4, "workspace flags"),
     (("ti8_fwht", FAKE, 384, FAKE, 384, 4, 384, 384, 1.0, None), 2, "power of two"),
     (("ti8_fwht", FAKE, 256, FAKE, 256, 4, 256, 64, 1.0, None), 2, "power of two"),
     (("ti8_gemm_i8_nt", FAKE, 0, 128, FAKE, 0, 128, FAKE, 0, 128, FAKE, 0, 0, 1, 0, FAKE, 0, 0, 1, 0,

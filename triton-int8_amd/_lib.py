@@ -20,6 +20,7 @@ PROTOTYPES = {
     "ti8_quant_row": [_vp, _i64, _vp, _i64, _vp, _i64, _i64, _int, _int, _int, _vp],
     "ti8_quant_col_t": [_vp, _i64, _vp, _i64, _vp, _vp, _i64, _i64, _int, _int, _vp],
     "ti8_quant_row_col_t": [_vp, _i64, _vp, _i64, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _int, _int, _vp],
+    "ti8_quant_row_col_t_noalloc": [_vp, _i64, _vp, _i64, _vp, _vp, _i64, _vp, _i64, _i64, _int, _int, _vp],
     "ti8_fwht": [_vp, _i64, _vp, _i64, _i64, _i64, _i64, _f32, _vp],
     "ti8_gemm_i8_nt": [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64,
                        _vp, _int, _i64, _i64, _i64, _vp, _int, _i64, _i64, _i64,
@@ -34,6 +35,7 @@ INV_RCP_OF_SCALE, INV_AMAX_DIV_127, INV_AMAX_MUL_RCP127, INV_MULTIPLIER = 0, 1, 
 SCALE_ROW, SCALE_BLOCK128, SCALE_ROW_K128, SCALE_BLOCK_K256 = 0, 1, 2, 3
 COMBINE_MUL_MUL, COMBINE_MUL_PROD, COMBINE_DIV_PROD = 0, 1, 2
 GEMM_STRICT, GEMM_TILED, GEMM_SKINNY, GEMM_LARGE_TILES = 1, 2, 4, 8
+NOALLOC_MAX_ROWS_PLUS_COLS = 65536
 
 _lib = None
 

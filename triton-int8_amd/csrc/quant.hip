@@ -4,6 +4,8 @@
 //
 // This file MUST be compiled with -ffp-contract=off: `x*scale + 0.5f` has to round
 // twice (multiply, then add) to reproduce the reference arithmetic bit for bit.
+#include <mutex>
+
 #include "ti8_common.h"
 
 namespace ti8 {
@@ -757,10 +759,10 @@ extern "C" int ti8_quant_col_t(const void* x, int64_t ldx, int8_t* qT, int64_t l
     return check_launch("ti8_quant_col_t");
 }
 
-extern "C" int ti8_quant_row_col_t(const void* x, int64_t ldx, int8_t* q, int64_t ldq, float* s_row, int8_t* qT,
-                                   int64_t ldqt, float* s_col, float* ws, int64_t R, int64_t C, int qflags,
-                                   int inv_mode, ti8_stream_t stream) {
-    const char* fn = "ti8_quant_row_col_t";
+// The launches of ti8_quant_row_col_t on a workspace the caller of this function has settled on
+static int quant_row_col_t_impl(const char* fn, const void* x, int64_t ldx, int8_t* q, int64_t ldq, float* s_row, int8_t* qT,
+                                int64_t ldqt, float* s_col, float* ws, int64_t R, int64_t C, int qflags, int inv_mode,
+                                ti8_stream_t stream) {
     const bool pingpong = (qflags & TI8_Q_WS_PINGPONG) != 0, second = (qflags & TI8_Q_WS_SECOND) != 0;
     if (second && !pingpong) return fail(TI8_ERR_MODE, "%s: TI8_Q_WS_SECOND needs TI8_Q_WS_PINGPONG", fn);
     QMode mode;
@@ -789,6 +791,58 @@ extern "C" int ti8_quant_row_col_t(const void* x, int64_t ldx, int8_t* q, int64_
     hipLaunchKernelGGL(quant_rowcol_kernel, dim3((unsigned)ntiles), dim3(256), 0, st, xp, ldx, q, ldq, s_row, qT, ldqt,
                        s_col, ws, ws + R, ws_next, R, (int)(C / 128), mode);
     return check_launch(fn);
+}
+
+extern "C" int ti8_quant_row_col_t(const void* x, int64_t ldx, int8_t* q, int64_t ldq, float* s_row, int8_t* qT,
+                                   int64_t ldqt, float* s_col, float* ws, int64_t R, int64_t C, int qflags,
+                                   int inv_mode, ti8_stream_t stream) {
+    return quant_row_col_t_impl("ti8_quant_row_col_t", x, ldx, q, ldq, s_row, qT, ldqt, s_col, ws, R, C, qflags, inv_mode, stream);
+}
+
+// ---------------------------------------------------------------------------------
+// The same operation for callers that cannot allocate: the row and column maxima are collected in
+// a fixed array in device memory that belongs to the library (one copy per GPU, held until the
+// process ends) instead of a workspace argument.
+namespace ti8 {
+static __device__ __align__(256) unsigned int scratch[TI8_NOALLOC_MAX_ROWS_PLUS_COLS];
+
+// Device address of `scratch` on the current device.  In host code the array's name is only a
+// handle for hipGetSymbolAddress, never an address a kernel can use; each GPU has its own copy at
+// its own address, looked up once per device (with that device current) and kept.
+static int scratch_address(const char* fn, float** out) {
+    constexpr int MAX_DEV = 64;
+    static std::mutex mu;
+    static float* addr[MAX_DEV] = {nullptr};
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(TI8_ERR_HIP, "%s: hipGetDevice: %s", fn, hipGetErrorString(e));
+    if (dev < 0 || dev >= MAX_DEV) return fail(TI8_ERR_HIP, "%s: device index %d out of range", fn, dev);
+    std::lock_guard<std::mutex> lock(mu);
+    if (!addr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) return fail(TI8_ERR_HIP, "%s: hipGetSymbolAddress(scratch): %s", fn, hipGetErrorString(e));
+        addr[dev] = static_cast<float*>(p);
+    }
+    *out = addr[dev];
+    return TI8_OK;
+}
+}  // namespace ti8
+
+extern "C" int ti8_quant_row_col_t_noalloc(const void* x, int64_t ldx, int8_t* q, int64_t ldq, float* s_row, int8_t* qT,
+                                           int64_t ldqt, float* s_col, int64_t R, int64_t C, int qflags,
+                                           int inv_mode, ti8_stream_t stream) {
+    const char* fn = "ti8_quant_row_col_t_noalloc";
+    if (qflags & (TI8_Q_WS_PINGPONG | TI8_Q_WS_SECOND))
+        return fail(TI8_ERR_MODE, "%s: the workspace flags belong to ti8_quant_row_col_t (there is no workspace argument here)", fn);
+    if (R > 0 && C > 0 && R + C > TI8_NOALLOC_MAX_ROWS_PLUS_COLS)
+        return fail(TI8_ERR_SHAPE, "%s: R + C = %lld exceeds the library's fixed scratch of %d floats; use ti8_quant_row_col_t with a workspace",
+                    fn, (long long)(R + C), TI8_NOALLOC_MAX_ROWS_PLUS_COLS);
+    float* ws = nullptr;
+    if (int e = scratch_address(fn, &ws)) return e;
+    // the array keeps the last call's maxima: the shared launch sequence starts with the fill kernel
+    // that zeroes the R + C words this call uses (a kernel, not a memset, so the call can be captured)
+    return quant_row_col_t_impl(fn, x, ldx, q, ldq, s_row, qT, ldqt, s_col, ws, R, C, qflags, inv_mode, stream);
 }
 
 extern "C" int ti8_quant_block_had128(const void* x, int64_t bsx, int64_t ldx, int8_t* q, int64_t bsq, int64_t ldq,
