@@ -41,22 +41,28 @@ def _expand(s, mode, rows, kb):
     return s[:, kb].to(F32).repeat_interleave(128)[:rows]   # row r uses block r // 128 (rows need not fill the last block)
 
 
-def gemm_scaled(Aq, sA, modeA, Bq, sB, modeB, out_scale=None, out_dtype=torch.bfloat16):
+def gemm_scaled(Aq, sA, modeA, Bq, sB, modeB, out_scale=None, out_dtype=torch.bfloat16, with_magnitude=False):
     """2-D NT GEMM with per-K-block promotion, literal association
     ``acc = acc + (f32(dot) * sa) * sb`` for any mix of ROW / BLOCK descriptors.
-    ``out_scale`` (a power of two) multiplies the fp32 accumulator before the store."""
+    ``out_scale`` (a power of two) multiplies the fp32 accumulator before the store.
+    ``with_magnitude`` also returns sum_kb |term_kb| (fp32, scaled like the result): what a
+    different association of the same fp32 sum can move the result by is a few 2^-24 of it."""
     M, K = Aq.shape
     N = Bq.shape[0]
     acc = torch.zeros((M, N), dtype=F32)
+    mag = torch.zeros((M, N), dtype=F32)
     for kb in range(K // 128):
         ks = slice(kb * 128, (kb + 1) * 128)
         d = int_dot_k128(Aq[:, ks], Bq[:, ks])
         t = d * _expand(sA, modeA, M, kb)[:, None]
         t = t * _expand(sB, modeB, N, kb)[None, :]
         acc = acc + t
+        if with_magnitude:
+            mag = mag + t.abs()
     if out_scale is not None:
         acc = acc * f32(out_scale)
-    return acc.to(out_dtype)
+        mag = mag * f32(out_scale)
+    return (acc.to(out_dtype), mag) if with_magnitude else acc.to(out_dtype)
 
 
 def quant2d(x, mode, clamp):

@@ -48,3 +48,19 @@ def bits_equal(a, b):
 def rel_err(a, b):
     a, b = a.double().cpu(), b.double().cpu()
     return float((a - b).norm() / b.norm().clamp_min(1e-300))
+
+
+def bf16_ulp(v):
+    """Spacing of bf16 numbers at |v| (as an fp32 tensor)."""
+    _, e = torch.frexp(v.float().abs().clamp_min(2.0 ** -126))
+    return torch.ldexp(torch.ones_like(v, dtype=torch.float32), e - 8)
+
+
+def assert_one_ulp(got, want, what="", slack=2.0 ** -18):
+    """Every element of `got` within one bf16 ulp of `want`, plus `slack` x max|want| for the elements
+    whose K-block terms cancel (re-associating the fp32 sum moves those by a few 2^-24 of the terms,
+    which are of the size of the large elements, not of the result)."""
+    got, want = got.float().cpu(), want.float().cpu()
+    assert got.shape == want.shape, what
+    bad = (got - want).abs() > bf16_ulp(want) + slack * want.abs().max()
+    assert not bool(bad.any()), f"{what}: {int(bad.sum())} of {bad.numel()} elements off by more than one bf16 ulp, first at {bad.nonzero()[0].tolist()}"

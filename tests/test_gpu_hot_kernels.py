@@ -1,0 +1,312 @@
+"""Element-by-element parity of the GEMM kernels that carry the benchmark (the promotion kernels on
+256 x 256, 256 x 128 and 128 x 128 tiles, the int32 kernel and the few-rows kernel) with the CPU
+oracle: at long contraction dims (more per-K-tile factors than one register holds), at tile counts
+that exercise the workgroup -> tile map (XCD ranges, incomplete groups of tile rows), and at the
+full benchmark shapes through sampled output tiles recomputed from the GPU-produced int8 tensors
+and scales.
+
+Bar for the default (fast) promotion arithmetic, per element:
+    |got - want| <= 1 bf16 ulp of want  +  (K/128 + 4) * 2^-23 * sum_kb |term_kb|
+The second term is what re-associating an fp32 sum of K/128 terms can move it by (it matters only
+where the terms cancel); a wrong scale, a dropped K tile or a misplaced tile is off by orders of
+magnitude more.  The literal mode (strict) and the int32 path are bit-exact."""
+import pytest
+import torch
+
+from conftest import bf16_ulp, bits_equal, make_gen, randn_bf16, rel_err
+from oracle import double_channel_fwd32 as odf
+from oracle import linear as olin
+
+pytestmark = pytest.mark.gpu
+FAST_REL_TOL = 2e-4   # Frobenius norm; the task's bar for bf16 outputs is 1e-2
+
+
+@pytest.fixture(scope="module")
+def T():
+    import triton_int8_amd
+    return triton_int8_amd
+
+
+def assert_promoted_close(got, want, mag, K, what=""):
+    got, want, mag = got.float().cpu(), want.float().cpu(), mag.float().cpu()
+    assert got.shape == want.shape, what
+    bound = bf16_ulp(want) + (K // 128 + 4) * 2.0 ** -23 * mag
+    bad = (got - want).abs() > bound
+    assert not bool(bad.any()), f"{what}: {int(bad.sum())} of {bad.numel()} elements outside one bf16 ulp, first at {bad.nonzero()[0].tolist()}"
+    assert torch.isfinite(got).all(), what
+
+
+def run_gemm(T, path, *args, **kw):
+    old = T.ops.GEMM_PATH
+    T.ops.GEMM_PATH = path
+    try:
+        return T.ops.gemm_i8_nt(*args, **kw)
+    finally:
+        T.ops.GEMM_PATH = old
+
+
+def scales(g, *shape):
+    """positive scales spread over two orders of magnitude"""
+    return torch.exp(torch.rand(*shape, generator=g) * 4.6) * 1e-4
+
+
+@pytest.mark.parametrize("K", [8192, 8320, 14336, 16384, 32768, 32896])
+@pytest.mark.parametrize("path", ["tiled", "large", "skinny"])
+def test_promotion_at_long_contraction(T, dev, K, path):
+    """K tiles 64 and up take the per-K-tile factor from the second, third and fourth register
+    (both GEMM families); K > 32768 falls back to the literal kernel."""
+    from triton_int8_amd._lib import SCALE_BLOCK128, SCALE_ROW
+    M, N, nkb = 256, 384, K // 128
+    g = make_gen(K)
+    A = torch.randint(-127, 128, (2, M, K), generator=g, dtype=torch.int8)
+    B2 = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+    B3 = torch.randint(-127, 128, (2, N, K), generator=g, dtype=torch.int8)
+    sa_row, sb_row, sb3_row = scales(g, 2, M), scales(g, N), scales(g, 2, N)
+    sa_blk, sb_blk, sb3_blk = scales(g, 2, M // 128, nkb), scales(g, N // 128, nkb), scales(g, 2, N // 128, nkb)
+    # a factor that only the last K tile of each register group carries: a stale or misindexed
+    # factor register shows as a large error
+    for kt in (63, 64, 127, 128, 191, 192, nkb - 1):
+        if kt < nkb:
+            sa_blk[:, :, kt] *= 37.0
+            sb_blk[:, kt] *= 0.031
+    Ad = A.to(dev)
+    skinny_takes_it = K <= 32768
+    for sA, mA, oA in ((sa_blk, SCALE_BLOCK128, olin.BLOCK), (sa_row, SCALE_ROW, olin.ROW)):
+        for Bq, sB, mB, oB in ((B2, sb_row, SCALE_ROW, olin.ROW), (B2, sb_blk, SCALE_BLOCK128, olin.BLOCK),
+                               (B3, sb3_row, SCALE_ROW, olin.ROW), (B3, sb3_blk, SCALE_BLOCK128, olin.BLOCK)):
+            if mA == SCALE_ROW and mB == SCALE_ROW:
+                continue
+            if path == "skinny" and not skinny_takes_it:
+                continue
+            pairs = [olin.gemm_scaled(A[b], sA[b], oA, Bq[b] if Bq.dim() == 3 else Bq, sB[b] if Bq.dim() == 3 else sB, oB,
+                                      with_magnitude=True) for b in range(2)]
+            want, mag = torch.stack([p[0] for p in pairs]), torch.stack([p[1] for p in pairs])
+            args = (Ad, Bq.to(dev), sA.to(dev), mA, sB.to(dev), mB)
+            what = f"K={K} {path} A:{oA} B:{oB}{' batched' if Bq.dim() == 3 else ''}"
+            got = run_gemm(T, path, *args)
+            assert_promoted_close(got, want, mag, K, what)
+            assert rel_err(got, want) <= FAST_REL_TOL, what
+            if path == "tiled":   # the literal kernel: bit-equal, at every K
+                assert bits_equal(run_gemm(T, path, *args, strict=True), want), what + " strict"
+    # int32 over the whole K at the same shapes: exact
+    want = odf.dequant_epilogue(odf.gemm_i32(A, B2), sa_row, sb_row)
+    if path != "skinny" or skinny_takes_it:
+        got = run_gemm(T, path, Ad, B2.to(dev), sa_row.to(dev), SCALE_ROW, sb_row.to(dev), SCALE_ROW, acc_i32_full=True)
+        assert bits_equal(got, want)
+
+
+@pytest.mark.parametrize("M,N,K,path,kernel", [
+    (1536, 1024, 1024, "large", "256x256 tiles: 6 tile rows (a group of 4 and one of 2), 24 tiles = 8 XCD ranges of 3"),
+    (1536, 1024, 640, "tiled", "128x128 tiles: 12 tile rows (a group of 8 and one of 4), 96 tiles"),
+    (4608, 2048, 512, "tiled", "256x128 tiles: 18 tile rows (four groups of 4 and one of 2), 288 tiles"),
+    (1280, 768, 384, "large", "256x256 tiles: 15 tiles, no XCD remap"),
+    (2048, 2048, 256, "large", "256x256 tiles: 64 tiles, complete groups"),
+])
+def test_tile_maps_cover_the_output(T, dev, M, N, K, path, kernel):
+    """Every element of C, against the oracle, at tile counts where the workgroup -> tile map takes
+    its XCD remap (tile count a multiple of 8) together with an incomplete last group of tile rows.
+    The output buffer starts as NaN, so a tile nobody wrote fails."""
+    from triton_int8_amd._lib import SCALE_BLOCK128, SCALE_ROW
+    g = make_gen(M + N + K)
+    A = torch.randint(-127, 128, (1, M, K), generator=g, dtype=torch.int8)
+    B = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+    sa_blk, sb_row, sb_blk, sa_row = scales(g, 1, M // 128, K // 128), scales(g, N), scales(g, N // 128, K // 128), scales(g, 1, M)
+    Ad, Bd = A.to(dev), B.to(dev)
+    for sA, mA, oA, sB, mB, oB in ((sa_blk, SCALE_BLOCK128, olin.BLOCK, sb_row, SCALE_ROW, olin.ROW),
+                                   (sa_blk, SCALE_BLOCK128, olin.BLOCK, sb_blk, SCALE_BLOCK128, olin.BLOCK),
+                                   (sa_row, SCALE_ROW, olin.ROW, sb_blk, SCALE_BLOCK128, olin.BLOCK)):
+        want, mag = olin.gemm_scaled(A[0], sA[0], oA, B, sB, oB, with_magnitude=True)
+        out = torch.full((1, M, N), float("nan"), dtype=torch.bfloat16, device=dev)
+        got = run_gemm(T, path, Ad, Bd, sA.to(dev), mA, sB.to(dev), mB, out=out)
+        assert_promoted_close(got[0], want, mag, K, f"{kernel} A:{oA} B:{oB}")
+    out = torch.full((1, M, N), float("nan"), dtype=torch.bfloat16, device=dev)
+    got = run_gemm(T, path, Ad, Bd, sa_row.to(dev), SCALE_ROW, sb_row.to(dev), SCALE_ROW, acc_i32_full=True, out=out)
+    assert bits_equal(got, odf.dequant_epilogue(odf.gemm_i32(A, B), sa_row, sb_row)), kernel
+    acc = T.ops.gemm_i8_nt_i32(Ad, Bd)
+    assert bits_equal(acc, odf.gemm_i32(A, B)), kernel
+
+
+def sample_tiles(tiles_m, tiles_n, g, count=8):
+    """first, last, the corners, and seeded others: tiles of different XCD ranges and groups"""
+    picks = {(0, 0), (tiles_m - 1, tiles_n - 1), (0, tiles_n - 1), (tiles_m - 1, 0)}
+    while len(picks) < count + 4:
+        picks.add((int(torch.randint(0, tiles_m, (1,), generator=g)), int(torch.randint(0, tiles_n, (1,), generator=g))))
+    return sorted(picks)
+
+
+def check_sampled_tiles(C, Aq, sA, oA, Bq, sB, oB, g, what, out_scale=None, exact=False, tile=256):
+    """C [M, N] (GPU) against the oracle on sampled tile x tile output tiles, recomputed on the CPU
+    from the GPU-produced int8 operands Aq [M, K], Bq [N, K] and their scales."""
+    M, K = Aq.shape
+    N = Bq.shape[0]
+    for tm, tn in sample_tiles(M // tile, N // tile, g):
+        r, c = slice(tm * tile, (tm + 1) * tile), slice(tn * tile, (tn + 1) * tile)
+        a, b = Aq[r].cpu(), Bq[c].cpu()
+        if exact:   # int32 over the whole K, per-row scales
+            want = odf.dequant_epilogue(odf.gemm_i32(a[None], b), sA[r].cpu()[None], sB[c].cpu())[0]
+            assert bits_equal(C[r, c], want), f"{what}: tile ({tm}, {tn}) differs"
+            continue
+        sa = sA[r].cpu() if oA == olin.ROW else sA[tm * tile // 128:(tm + 1) * tile // 128].cpu()
+        sb = sB[c].cpu() if oB == olin.ROW else sB[tn * tile // 128:(tn + 1) * tile // 128].cpu()
+        want, mag = olin.gemm_scaled(a, sa, oA, b, sb, oB, out_scale, with_magnitude=True)
+        assert_promoted_close(C[r, c], want, mag, K, f"{what}: tile ({tm}, {tn})")
+
+
+def config_operand(rows, cols, g, kind="normal", std=1.0, outlier_frac=0.0, outlier_mul=1.0):
+    if kind == "student_t":
+        x = torch.randn(rows, cols, generator=g) / torch.sqrt(torch.randn(3, rows, cols, generator=g).pow(2).mean(0))
+    else:
+        x = torch.randn(rows, cols, generator=g) * std
+    if outlier_frac:
+        x[:, torch.randperm(cols, generator=g)[: int(-(-cols * outlier_frac // 1))]] *= outlier_mul
+    return x.to(torch.bfloat16)
+
+
+def block_channel_step_pieces(T, X, W, dY, hadamard=None):
+    """The launches of linear_fwd_bwd(scheme="block_channel"), with the int8 operands and scales of
+    each GEMM kept: [(name, C, Aq, sA, modeA, Bq, sB, modeB, out_scale)]."""
+    from triton_int8_amd.linear import linear_backward, linear_forward
+    ops = T.ops
+    if hadamard == 128:
+        xq, xs = ops.quant_block_had128(X[None])
+        wq, ws = ops.quant_row(W, hadamard128=True)
+        dq, ds = ops.quant_block_had128(dY[None])
+        wtq, wts = ops.quant_col_t(W, hadamard128=True)
+        dyt, dyts = ops.quant_block_had128(dY[None], along_rows=True, clamp=False)
+        xt, xts = ops.quant_block_had128(X[None], along_rows=True, clamp=False)
+        Y, saved = linear_forward(X, W, "block_channel", 128)
+        dX, dW = linear_backward(dY, X, W, "block_channel", 128, saved)
+        sc = 2.0 ** -7
+        return [("Y", Y, xq[0], xs[0], olin.BLOCK, wq, ws, olin.ROW, sc),
+                ("dX", dX, dq[0], ds[0], olin.BLOCK, wtq, wts, olin.ROW, sc),
+                ("dW", dW, dyt[0], dyts[0].t(), olin.BLOCK, xt[0], xts[0].t(), olin.BLOCK, sc)]
+    xq, xqT, xs = ops.quant_block(X[None], with_transpose=True)
+    wq, ws, wtq, wts = ops.quant_row_col_t(W)
+    dq, dqT, ds = ops.quant_block(dY[None], with_transpose=True)
+    Y, saved = linear_forward(X, W, "block_channel")
+    dX, dW = linear_backward(dY, X, W, "block_channel", None, saved)
+    return [("Y", Y, xq[0], xs[0], olin.BLOCK, wq, ws, olin.ROW, None),
+            ("dX", dX, dq[0], ds[0], olin.BLOCK, wtq, wts, olin.ROW, None),
+            ("dW", dW, dqT[0], ds[0].t(), olin.BLOCK, xqT[0], xs[0].t(), olin.BLOCK, None)]
+
+
+def test_config2_sampled_tiles_per_element(T, dev):
+    """The headline workload (8192 x 4096 x 4096, block-channel, seed 1): Y, dX and dW of the layer
+    call, element by element on 12 sampled 256 x 256 tiles each, against the oracle's literal loop
+    over the GPU-produced int8 operands; the operands themselves against the oracle's quantisers on
+    sampled blocks and rows."""
+    from oracle import block_channel_fwd32 as obf
+    g = make_gen(1)
+    M, K, N = 8192, 4096, 4096
+    X = config_operand(M, K, g, outlier_frac=0.01, outlier_mul=20.0)
+    W = config_operand(N, K, g, std=0.02)
+    dY = config_operand(M, N, g, std=1e-3)
+    Xd, Wd, dYd = X.to(dev), W.to(dev), dY.to(dev)
+    pieces = block_channel_step_pieces(T, Xd, Wd, dYd)
+    for name, C, Aq, sA, oA, Bq, sB, oB, sc in pieces:
+        check_sampled_tiles(C, Aq, sA, oA, Bq, sB, oB, g, f"config 2 {name}", sc)
+    # the layer call returns these very tensors
+    Y, dX, dW = T.linear_fwd_bwd(Xd, Wd, dYd, "block_channel")
+    for (name, C, *_), got in zip(pieces, (Y, dX, dW)):
+        assert torch.equal(C, got), name
+    # quantised operands against the oracle: a band of 256 rows of X, a band of rows of W
+    xq, xs = pieces[0][2], pieces[0][3]
+    qo, so = obf.block_quant(X[None, 4096:4352], True)
+    assert bits_equal(xq[4096:4352], qo[0]) and bits_equal(xs[32:34], so[0])
+    wq, ws = pieces[0][5], pieces[0][6]
+    qo, so = obf.token_quant(W[1000:1256], True)
+    assert bits_equal(wq[1000:1256], qo) and bits_equal(ws[1000:1256], so.flatten())
+    wtq, wts = pieces[1][5], pieces[1][6]
+    qo, so = obf.token_quant(W.t().contiguous()[3840:], True)
+    assert bits_equal(wtq[3840:], qo) and bits_equal(wts[3840:], so.flatten())
+    # row_block scheme of the same workload ("per-token X, per-block W")
+    from triton_int8_amd.linear import linear_backward, linear_forward
+    ops = T.ops
+    xq, xs = ops.quant_row(Xd)
+    wq, wqT, ws = ops.quant_block(Wd[None], with_transpose=True)
+    Y, saved = linear_forward(Xd, Wd, "row_block")
+    check_sampled_tiles(Y, xq, xs, olin.ROW, wq[0], ws[0], olin.BLOCK, g, "config 2 row_block Y")
+    dX, dW = linear_backward(dYd, Xd, Wd, "row_block", None, saved)
+    dq, ds, dytq, dyts = ops.quant_row_col_t(dYd)
+    _, xqT, xs2 = ops.quant_block(Xd[None], with_transpose=True)
+    check_sampled_tiles(dX, dq, ds, olin.ROW, wqT[0], ws[0].t(), olin.BLOCK, g, "config 2 row_block dX")
+    check_sampled_tiles(dW, dytq, dyts, olin.ROW, xqT[0], xs2[0].t(), olin.BLOCK, g, "config 2 row_block dW")
+
+
+def test_config3_double_channel_llama_mlp_sampled_tiles_exact(T, dev):
+    """Config 3: 16384 tokens through 4096 -> 14336 and 14336 -> 4096 in the double-channel scheme,
+    0.5 % of the channels x50: Y, dX, dW bit-equal to the oracle on sampled 256 x 256 tiles (int32
+    accumulation is exact), quantised operands bit-equal on sampled rows."""
+    from oracle import double_channel_fwd32 as odcf
+    g = make_gen(2)
+    tokens = 16384
+    for K, N in ((4096, 14336), (14336, 4096)):
+        X = config_operand(tokens, K, g, outlier_frac=0.005, outlier_mul=50.0)
+        W = config_operand(N, K, g, std=0.02)
+        dY = config_operand(tokens, N, g, std=1e-3)
+        Xd, Wd, dYd = X.to(dev), W.to(dev), dY.to(dev)
+        Y, dX, dW = T.linear_fwd_bwd(Xd, Wd, dYd, "double_channel")
+        xq, xs, xtq, xts = T.ops.quant_row_col_t(Xd, inv_mode=1)
+        wq, ws, wtq, wts = T.ops.quant_row_col_t(Wd, inv_mode=1)
+        dq, ds, dytq, dyts = T.ops.quant_row_col_t(dYd, inv_mode=1)
+        what = f"config 3 {K}->{N}"
+        check_sampled_tiles(Y, xq, xs, None, wq, ws, None, g, what + " Y", exact=True)
+        check_sampled_tiles(dX, dq, ds, None, wtq, wts, None, g, what + " dX", exact=True)
+        check_sampled_tiles(dW, dytq, dyts, None, xtq, xts, None, g, what + " dW", exact=True)
+        r = slice(7777, 7777 + 64)
+        qo, so = odcf.row_quant(X[r], BLOCK_N=128)
+        assert bits_equal(xq[r], qo) and bits_equal(xs[r], so), what
+        c = slice(K - 128, K)
+        qo, so = odcf.row_quant(X[:, c].t().contiguous(), BLOCK_N=128)       # X^T per row = X per column
+        assert bits_equal(xtq[c], qo) and bits_equal(xts[c], so), what
+        assert float(T.calc_diff(Y, Xd @ Wd.t())) < 2e-2   # x50 outlier channels: far above the N(0,1) bar
+        del Y, dX, dW, Xd, Wd, dYd
+
+
+def test_config4_hadamard_block_channel_sampled_tiles(T, dev):
+    """Config 4: 8192^3, X Student-t(3), H_128 fused into the quantisers, block-channel scales: the
+    three GEMMs element by element on sampled tiles (contraction dim 8192 = 64 K tiles), rotated and
+    quantised operands bit-equal to the un-fused oracle on sampled bands."""
+    from oracle import block_channel_fwd32 as obf
+    from oracle import hadamard as ohad
+    g = make_gen(3)
+    S = 8192
+    X = config_operand(S, S, g, kind="student_t")
+    W = config_operand(S, S, g, std=0.02)
+    dY = config_operand(S, S, g, std=1e-3)
+    Xd, Wd, dYd = X.to(dev), W.to(dev), dY.to(dev)
+    pieces = block_channel_step_pieces(T, Xd, Wd, dYd, 128)
+    for name, C, Aq, sA, oA, Bq, sB, oB, sc in pieces:
+        check_sampled_tiles(C, Aq, sA, oA, Bq, sB, oB, g, f"config 4 {name}", sc)
+    Y, dX, dW = T.linear_fwd_bwd(Xd, Wd, dYd, "block_channel", 128)
+    for (name, C, *_), got in zip(pieces, (Y, dX, dW)):
+        assert torch.equal(C, got), name
+    band = slice(2048, 2304)
+    qo, so = obf.block_quant(ohad.hadamard128(X[None, band]), True)
+    assert bits_equal(pieces[0][2][band], qo[0]) and bits_equal(pieces[0][3][16:18], so[0])
+    qo, so = obf.token_quant(ohad.hadamard128(W[band]), True)
+    assert bits_equal(pieces[0][5][band], qo) and bits_equal(pieces[0][6][band], so.flatten())
+    # dW operands: X rotated along the tokens, transposed: columns `band` of X = rows of X^T
+    qo, so = obf.block_quant(ohad.hadamard128(X[None, :, band], dim=1), False)
+    assert bits_equal(pieces[2][5][band], qo[0].t()) and bits_equal(pieces[2][6][16:18], so[0].t())
+    # the rotation spreads the heavy tails: still close to the bf16 product
+    assert float(T.calc_diff(Y, Xd @ Wd.t())) < 1e-2
+
+
+def test_config5_down_proj_layer_sampled_tiles(T, dev):
+    """Config 5's widest linear, Int8Linear(14336 -> 4096) at 16384 tokens (block-channel): the module's
+    output and both gradients on sampled tiles against the oracle (K = 14336 for Y, 16384 for dW)."""
+    g = make_gen(4)
+    tokens, K, N = 16384, 14336, 4096
+    lin = T.Int8Linear(K, N, device=dev)
+    with torch.no_grad():
+        lin.weight.copy_(config_operand(N, K, g, std=0.02).to(dev))
+    x = config_operand(tokens, K, g).to(dev).reshape(4, 4096, K).requires_grad_(True)
+    dy = config_operand(tokens, N, g, std=1e-3).to(dev).reshape(4, 4096, N)
+    y = lin(x)
+    y.backward(dy)
+    Wd = lin.weight.detach()
+    pieces = block_channel_step_pieces(T, x.detach().reshape(tokens, K), Wd, dy.reshape(tokens, N))
+    for (name, C, Aq, sA, oA, Bq, sB, oB, sc), got in zip(pieces, (y.detach().reshape(tokens, N), x.grad.reshape(tokens, K), lin.weight.grad)):
+        assert torch.equal(C, got), name
+        check_sampled_tiles(C, Aq, sA, oA, Bq, sB, oB, g, f"config 5 down_proj {name}", sc)

@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 import torch
 
-from conftest import bits_equal, make_gen, randn_bf16, rel_err
+from conftest import assert_one_ulp, bits_equal, make_gen, randn_bf16, rel_err
 from golden_util import bf16, load, t
 from oracle import block_channel_bwd33 as obb
 from oracle import block_channel_fwd32 as obf
@@ -21,7 +21,11 @@ from oracle import tilelang_block_channel_bwd as otb
 from oracle import tilelang_block_channel_fwd as otf
 
 pytestmark = pytest.mark.gpu
-REL_TOL = 1e-2
+REL_TOL = 1e-2     # the tolerance the task states for bf16 outputs
+FAST_TOL = 2e-4    # Frobenius bound for the default (re-associated fp32) promotion arithmetic, beside the
+                   # element-wise one-ulp bound (assert_one_ulp); 33 of 393216 elements one bf16 ulp off, the
+                   # large ones of outlier channels, already make 1.2e-4, and the literal arithmetic is no
+                   # closer to the exact sum than the re-associated one (27 against 16 such elements)
 
 
 @pytest.fixture(scope="module")
@@ -248,7 +252,8 @@ def test_entry_points_match_oracle(T, dev, module, fn, oracle_fn, three_d, gemm_
     C = getattr(getattr(T, module), fn)(a.to(dev), b.to(dev))
     Co = oracle_fn(a, b)
     assert C.dtype == torch.bfloat16 and C.shape == Co.shape
-    assert rel_err(C, Co) <= REL_TOL
+    assert rel_err(C, Co) <= FAST_TOL
+    assert_one_ulp(C, Co, f"{module}.{fn}")
     if module.startswith("double_channel"):
         assert bits_equal(C, Co)          # integer accumulation + literal epilogue: exact
     ref = torch.matmul(a.float(), b.float().transpose(-1, -2))
@@ -321,7 +326,8 @@ def test_bwd33_on_transposed_views(T, dev, gemm_path):
     at = randn_bf16(g, 1, 1024, 256).transpose(1, 2)
     bt = randn_bf16(g, 1, 1024, 384).transpose(1, 2)
     C = T.block_channel_bwd33.bwd_33(at.to(dev), bt.to(dev))
-    assert rel_err(C, obb.bwd_33(at, bt)) <= REL_TOL
+    assert rel_err(C, obb.bwd_33(at, bt)) <= FAST_TOL
+    assert_one_ulp(C, obb.bwd_33(at, bt))
 
 
 @pytest.mark.parametrize("scheme,h", [("block_channel", None), ("row_block", None), ("double_channel", None),
@@ -335,7 +341,8 @@ def test_linear_fwd_bwd(T, dev, scheme, h, gemm_path):
     Y, dX, dW = T.linear_fwd_bwd(X.to(dev), W.to(dev), dY.to(dev), scheme, h)
     Yo, dXo, dWo = olin.linear_fwd_bwd(X, W, dY, scheme, h)
     for got, want in ((Y, Yo), (dX, dXo), (dW, dWo)):
-        assert got.shape == want.shape and rel_err(got, want) <= REL_TOL
+        assert got.shape == want.shape and rel_err(got, want) <= FAST_TOL
+        assert_one_ulp(got, want, f"{scheme} hadamard={h}")
         if scheme == "double_channel":
             assert bits_equal(got, want)
     for got, ref in ((Y, X.float() @ W.float().t()), (dX, dY.float() @ W.float()),
@@ -388,7 +395,8 @@ def test_skinny_and_ragged_token_counts(T, dev, tokens, gemm_path):
         got = T.linear_fwd_bwd(X.to(dev), W.to(dev), dY.to(dev), scheme)
         want = olin.linear_fwd_bwd(X, W, dY, scheme)
         for a, b in zip(got, want):
-            assert a.shape == b.shape and rel_err(a, b) <= REL_TOL
+            assert a.shape == b.shape and rel_err(a, b) <= FAST_TOL
+            assert_one_ulp(a, b, f"{scheme} {tokens} tokens")
             if scheme == "double_channel":
                 assert bits_equal(a, b)
 
@@ -480,7 +488,8 @@ def test_golden_vectors_on_gpu(T, dev, gemm_path):
         tag = scheme + ("_h128" if h else "")
         Y, dX, dW = T.linear_fwd_bwd(X, W, dY, scheme, h)
         for got, key in ((Y, "_Y"), (dX, "_dX"), (dW, "_dW")):
-            assert rel_err(got, bf16(z[tag + key])) <= REL_TOL
+            assert rel_err(got, bf16(z[tag + key])) <= FAST_TOL
+            assert_one_ulp(got, bf16(z[tag + key]), tag + key)
 
 
 def test_full_size_properties(T, dev):
