@@ -1,0 +1,316 @@
+// Host-side walk over the launches of libti8's kernels: for the geometry an entry point would
+// launch, visit every (workgroup, wave, lane, iteration) and check each global-memory access
+// against the number of elements that lie between the pointer the caller passed and the end of
+// its allocation.  The offsets come from triton-int8_amd/csrc/index_math.h, the same functions the
+// kernels call; what is mirrored by hand here is only the order in which a kernel combines them
+// (each such place cites the kernel's lines).  Built with g++ by tests/test_kernel_bounds.py: no
+// GPU, no HIP.
+//
+// Every walk_* function returns 0 when all accesses are in bounds (and, for the GEMM, when every
+// element of C is stored exactly once), else 1 with a description of the first violation in msg.
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <vector>
+
+#include "index_math.h"
+
+using namespace ti8::idx;
+
+namespace {
+
+struct Report {
+    char* msg;
+    int len;
+    bool bad = false;
+    int64_t checked = 0;
+    void fail(const char* fmt, ...) {
+        if (bad) return;
+        bad = true;
+        va_list ap;
+        va_start(ap, fmt);
+        vsnprintf(msg, len, fmt, ap);
+        va_end(ap);
+    }
+    // access of `n` elements at element offset `off` of a buffer with `size` elements
+    bool access(const char* what, int64_t off, int64_t n, int64_t size, int64_t a = -1, int64_t b = -1, int64_t c = -1, int64_t d = -1) {
+        ++checked;
+        if (off < 0 || off + n > size) {
+            fail("%s: elements [%lld, %lld) outside the buffer of %lld (at %lld, %lld, %lld, %lld)", what, (long long)off,
+                 (long long)(off + n), (long long)size, (long long)a, (long long)b, (long long)c, (long long)d);
+            return false;
+        }
+        return true;
+    }
+};
+
+}  // namespace
+
+extern "C" {
+
+// ti8_fwht -> fwht_kernel<NT> (fwht.hip): bf16 x [rows][cols] (ldx) -> y (ldy)
+int walk_fwht(int64_t ldx, int64_t ldy, int64_t rows, int64_t cols, int64_t n, int64_t x_elems, int64_t y_elems,
+              int64_t lds_bytes_limit, int64_t* n_checked, char* msg, int msglen) {
+    Report r{msg, msglen};
+    const int64_t L = fwht_segment_len(cols, n);
+    const int NT = fwht_threads(L);
+    const int64_t nblocks = rows * (cols / L);
+    const int64_t lds_words = fwht_lds_words(L);
+    if (lds_words * 4 > lds_bytes_limit) r.fail("fwht: %lld bytes of LDS requested, limit %lld", (long long)(lds_words * 4), (long long)lds_bytes_limit);
+    int logn = 0;
+    while ((1LL << logn) < n) ++logn;
+    const int segs_per_row = (int)(cols / L);
+    // LDS indices do not depend on the workgroup: walk them once
+    for (int tid = 0; tid < NT && !r.bad; ++tid) {
+        for (int vt = tid; vt < (L >> 4); vt += NT)
+            for (int e = 0; e < 16; ++e) r.access("fwht lds first pass", vt * 17 + e, 1, lds_words, tid, vt, e);
+        auto pass = [&](int p, int rb) {   // pass_in_lds<RB, NT>
+            const int ngroups = (int)(L >> rb);
+            for (int vt = tid; vt < ngroups; vt += NT) {
+                const int base = fwht_group_base(vt, p, rb);
+                for (int e = 0; e < (1 << rb); ++e) r.access("fwht lds pass", fwht_padded(base + (e << p)), 1, lds_words, tid, vt, e, p);
+            }
+        };
+        const int rb1 = imin(4, logn - 4);
+        pass(4, rb1);
+        int rem = logn - 8;
+        if (rem > 0) {
+            const int rb2 = rem <= 5 ? rem : (rem + 1) / 2;
+            pass(8, rb2);
+            rem -= rb2;
+            if (rem > 0) pass(8 + rb2, rem);
+        }
+        for (int c = tid; c < (L >> 3); c += NT) r.access("fwht lds read-back", fwht_padded(c * 8), 8, lds_words, tid, c);
+    }
+    for (int64_t block = 0; block < nblocks && !r.bad; ++block) {
+        const int64_t xo = fwht_segment_offset(block, segs_per_row, ldx, (int)L);
+        const int64_t yo = fwht_segment_offset(block, segs_per_row, ldy, (int)L);
+        for (int tid = 0; tid < NT; ++tid) {
+            for (int vt = tid; vt < (L >> 4); vt += NT) {   // two 16-byte loads: elements vt*16 .. +16
+                r.access("fwht x", xo + vt * 16, 8, x_elems, block, tid, vt);
+                r.access("fwht x", xo + vt * 16 + 8, 8, x_elems, block, tid, vt);
+            }
+            for (int c = tid; c < (L >> 3); c += NT) r.access("fwht y", yo + c * 8, 8, y_elems, block, tid, c);
+        }
+    }
+    *n_checked = r.checked;
+    return r.bad;
+}
+
+// ti8_quant_row -> quant_row_kernel<NLOAD, WG_ROW, GROUP16, HAD> (quant.hip)
+int walk_quant_row(int64_t ldx, int64_t ldq, int64_t rows, int64_t cols, int group, int64_t x_elems, int64_t q_elems,
+                   int64_t s_elems, int64_t* n_checked, char* msg, int msglen) {
+    Report r{msg, msglen};
+    const int nchunk = (int)(cols / 8);
+    const QRowConfig cfg = qrow_config(nchunk, group == 128);
+    const int64_t grid = cfg.wg_row ? rows : (rows + 3) / 4;
+    const int T = cfg.wg_row ? 256 : 64;
+    const int ngrp = (int)(cols >> 7);
+    std::vector<uint8_t> seen((size_t)rows, 0);
+    for (int64_t block = 0; block < grid && !r.bad; ++block)
+        for (int tid = 0; tid < 256; ++tid) {
+            const int t = cfg.wg_row ? tid : (tid & 63);
+            const int64_t row = qrow_row(block, tid >> 6, cfg.wg_row);
+            if (row >= rows) continue;
+            if (t == 0) ++seen[(size_t)row];
+            for (int i = 0; i < cfg.nload; ++i) {
+                const int c = qrow_chunk(t, i, T);
+                if (c >= nchunk) continue;
+                r.access("quant_row x", row * ldx + c * 8, 8, x_elems, block, tid, i);
+                r.access("quant_row q", row * ldq + c * 8, 8, q_elems, block, tid, i);
+                if (group == 128 && (c & 15) == 0) r.access("quant_row s", row * ngrp + (c >> 4), 1, s_elems, block, tid, i);
+            }
+            if (group != 128 && t == 0) r.access("quant_row s", row, 1, s_elems, block, tid);
+        }
+    // every chunk of a row is taken by exactly one (thread, load): T * NLOAD covers the row
+    if ((int64_t)T * cfg.nload < nchunk) r.fail("quant_row: %d threads x %d loads do not cover %d chunks", T, cfg.nload, nchunk);
+    for (int64_t row = 0; row < rows && !r.bad; ++row)
+        if (seen[(size_t)row] != 1) r.fail("quant_row: row %lld handled %d times", (long long)row, (int)seen[(size_t)row]);
+    *n_checked = r.checked;
+    return r.bad;
+}
+
+// ti8_quant_block -> quant_block_kernel<NSUB, WRITE_Q, WRITE_QT> (quant.hip)
+int walk_quant_block(int64_t bsx, int64_t ldx, int has_q, int64_t bsq, int64_t ldq, int has_qt, int64_t bsqt, int64_t ldqt,
+                     int64_t ssb, int64_t ssr, int64_t ssc, int64_t B, int64_t R, int64_t C, int group_c, int64_t x_elems,
+                     int64_t q_elems, int64_t qt_elems, int64_t s_elems, int64_t* n_checked, char* msg, int msglen) {
+    Report r{msg, msglen};
+    const int nsub = group_c / 128;
+    const int nrb = (int)(R / 128), ncb = (int)(C / group_c);
+    const int64_t ntiles = B * nrb * ncb;
+    for (int64_t block = 0; block < ntiles && !r.bad; ++block) {
+        const TileId t = qblock_tile((int)block, nrb, ncb);
+        const int64_t xo = qblock_origin(t.b, bsx, t.rb, ldx, t.cb, 128 * nsub);
+        r.access("quant_block s", t.b * ssb + t.rb * ssr + t.cb * ssc, 1, s_elems, block);
+        for (int tid = 0; tid < 256; ++tid) {
+            for (int u = 0; u < nsub; ++u)
+                for (int h = 0; h < 2; ++h)
+                    for (int j = 0; j < 4; ++j) {
+                        const int row = qblock_row(tid, h, j);
+                        r.access("quant_block x", xo + (int64_t)row * ldx + u * 128 + qblock_col(tid), 8, x_elems, block, tid, h, j);
+                        if (has_q)
+                            r.access("quant_block q", qblock_origin(t.b, bsq, t.rb, ldq, t.cb, 128 * nsub) + u * 128 + qblock_col(tid) + (int64_t)row * ldq,
+                                     8, q_elems, block, tid, h, j);
+                    }
+            if (has_qt) {
+                const int64_t qo = qblock_origin(t.b, bsqt, t.cb, ldqt, t.rb, 128);
+                for (int p = 0; p < 4; ++p) r.access("quant_block qT", qo + (int64_t)qblock_t_row(tid, p) * ldqt + qblock_t_col(tid), 16, qt_elems, block, tid, p);
+            }
+        }
+    }
+    *n_checked = r.checked;
+    return r.bad;
+}
+
+struct ScaleArg {
+    int mode;
+    int64_t bs, rs, ks, elems;
+};
+
+// ti8_gemm_i8_nt / ti8_gemm_i8_nt_i32 -> gemm_i8_kernel<BM, BN, WM, WN, EPI> (gemm.hip); the
+// tile shape and epilogue kind are chosen as the entry point chooses them (raw_i32 = 1: the
+// int32-output entry point, always 256 x 256 tiles).  epi: 0 raw int32, 1 rows, 2 promote,
+// 3 literal, 4 per-lane B factors, 5 chained promote.
+int walk_gemm(int64_t bsa, int64_t lda, int64_t bsb, int64_t ldb, int64_t bsc, int64_t ldc, const ScaleArg* sa_in,
+              const ScaleArg* sb_in, int64_t batch, int64_t M, int64_t N, int64_t K, int acc_i32_full, int strict, int large,
+              int raw_i32, int num_cu, int64_t a_elems, int64_t b_elems, int64_t c_elems, int* picked, int64_t* n_checked,
+              char* msg, int msglen) {
+    Report r{msg, msglen};
+    ScaleArg sa = sa_in ? *sa_in : ScaleArg{0, 0, 0, 0, 0}, sb = sb_in ? *sb_in : ScaleArg{0, 0, 0, 0, 0};
+    GemmConfig cfg = raw_i32 ? GemmConfig{256, 256, 2, 4, 0}
+                             : gemm_config(M, N, K, batch, acc_i32_full != 0, strict != 0, sa.mode, sb.mode, large != 0, num_cu);
+    picked[0] = cfg.bm; picked[1] = cfg.bn; picked[2] = cfg.epi;
+    const int BM = cfg.bm, BN = cfg.bn, WM = cfg.wm, WN = cfg.wn, EPI = cfg.epi;
+    const int NW = WM * WN, TM = BM / WM / 32, TN = BN / WN / 32, A_INSTR = BM / 8 / NW, B_INSTR = BN / 8 / NW;
+    const int A_BYTES = BM * 128, B_BYTES = BN * 128;
+    const bool CHAIN = EPI == 5, LANEB = EPI == 4, FAST = EPI == 2 || EPI == 4 || EPI == 5;
+    const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
+    const int nk = (int)(K >> 7), klast = (nk - 1) * 128;
+    const int WCOLS = TN * 32, LPR = WCOLS / 4, RPI = 64 / LPR, NRR = 32 / RPI;
+    const int GROUP = gemm_group_rows(BM);
+    (void)CHAIN;
+    std::vector<uint8_t> stored(c_elems <= (int64_t)1 << 30 ? (size_t)c_elems : 0, 0);
+    std::vector<uint8_t> tile_seen((size_t)tiles_m * tiles_n, 0);
+    // K tiles whose loads are checked: offsets grow with kt up to the clamp, so the first two and
+    // the clamped ones (nk - 1, nk, nk + 1: the loop fetches up to two tiles ahead) cover all
+    const int kts[5] = {0, 1, nk - 1, nk, nk + 1};
+    for (int64_t by = 0; by < batch && !r.bad; ++by) {
+        std::fill(tile_seen.begin(), tile_seen.end(), 0);
+        for (int bx = 0; bx < tiles_m * tiles_n && !r.bad; ++bx) {
+            const TileCoord tc = gemm_tile_of(bx, tiles_m, tiles_n, GROUP);
+            if (tc.tile_m < 0 || tc.tile_m >= tiles_m || tc.tile_n < 0 || tc.tile_n >= tiles_n) {
+                r.fail("gemm: workgroup %d maps to tile (%d, %d) outside %d x %d", bx, tc.tile_m, tc.tile_n, tiles_m, tiles_n);
+                break;
+            }
+            ++tile_seen[(size_t)tc.tile_m * tiles_n + tc.tile_n];
+            const int m0 = tc.tile_m * BM, n0 = tc.tile_n * BN;
+            for (int wave = 0; wave < NW; ++wave) {
+                const int wm = wave / WN, wn = wave % WN;
+                const int rA0 = gemm_wave_first_row(m0, wave, A_INSTR, (int)M), rB0 = gemm_wave_first_row(n0, wave, B_INSTR, (int)N);
+                const int tA0 = wave * A_INSTR, tB0 = wave * B_INSTR;
+                for (int lane = 0; lane < 64; ++lane) {
+                    // ---- global -> LDS loads (gemm.hip: voffA/voffB, baseA/baseB, issue_tile_loads)
+                    for (int q = 0; q < 5; ++q) {
+                        const int koff = gemm_k_offset(kts[q], klast);
+                        for (int i = 0; i < A_INSTR; ++i) {
+                            const uint32_t vo = gemm_lane_offset_bytes(lane, (tA0 + i) & 1, (int)lda);
+                            r.access("gemm A", by * bsa + gemm_load_offset_bytes(rA0, lda, koff, i, vo), 16, a_elems, bx, wave, lane, kts[q]);
+                            const int64_t lds = (int64_t)wave * A_INSTR * 1024 + i * 1024 + lane * 16;
+                            r.access("gemm LDS A", lds, 16, A_BYTES, bx, wave, lane, i);
+                        }
+                        for (int i = 0; i < B_INSTR; ++i) {
+                            const uint32_t vo = gemm_lane_offset_bytes(lane, (tB0 + i) & 1, (int)ldb);
+                            r.access("gemm B", by * bsb + gemm_load_offset_bytes(rB0, ldb, koff, i, vo), 16, b_elems, bx, wave, lane, kts[q]);
+                            const int64_t lds = (int64_t)wave * B_INSTR * 1024 + i * 1024 + lane * 16;
+                            r.access("gemm LDS B", lds, 16, B_BYTES, bx, wave, lane, i);
+                        }
+                    }
+                    const int fr_row = lane & 31, fr_half = lane >> 5;
+                    // ---- per-K-tile factors of the fast promotion (gemm.hip: fraw_a / fraw_b, pfb)
+                    if (FAST) {
+                        const bool a_in = sa.mode != 0, b_in = sb.mode != 0;
+                        const int sha = sa.mode == 3 ? 1 : 0, shb = sb.mode == 3 ? 1 : 0;
+                        const int rowblk = gemm_factor_block(m0 + wm * TM * 32, (int)M), colblk = gemm_factor_block(n0 + wn * TN * 32, (int)N);
+                        const int64_t ska = a_in ? sa.ks : 0, skb = (b_in && !LANEB) ? sb.ks : 0;
+                        for (int c = 0; c < 4; ++c) {
+                            const int kt = gemm_factor_kt(c, lane, nk);
+                            r.access("gemm factor A", gemm_factor_index(by, sa.bs, rowblk, sa.rs, kt, sha, ska), 1, sa.elems, bx, wave, lane, c);
+                            r.access("gemm factor B", gemm_factor_index(by, sb.bs, colblk, sb.rs, kt, shb, skb), 1, sb.elems, bx, wave, lane, c);
+                        }
+                        if (LANEB)
+                            for (int j = 0; j < TN; ++j) {
+                                const int64_t base = epi_col_scale_index(by, sb.bs, n0 + (wn * TN + j) * 32 + fr_row, (int)N, sb.rs);
+                                for (int kt = 0; kt < nk; ++kt) r.access("gemm lane factor B", base + (int64_t)kt * sb.ks, 1, sb.elems, bx, wave, lane, kt);
+                            }
+                    }
+                    // ---- literal promotion: one scale per element and K tile (gemm.hip: EPI_STRICT block)
+                    if (EPI == 3) {
+                        const int kk[2] = {0, nk - 1};
+                        for (int q = 0; q < 2; ++q)
+                            for (int i = 0; i < TM; ++i)
+                                for (int j = 0; j < TN; ++j) {
+                                    const int col = imin(n0 + (wn * TN + j) * 32 + fr_row, (int)N - 1);
+                                    r.access("gemm strict B scale", scale_index(sb.mode, sb.bs, sb.rs, sb.ks, by, col, kk[q]), 1, sb.elems, bx, wave, lane, kk[q]);
+                                    for (int e = 0; e < 16; ++e) {
+                                        const int mrow = imin(m0 + (wm * TM + i) * 32 + 8 * (e >> 2) + 4 * fr_half + (e & 3), (int)M - 1);
+                                        r.access("gemm strict A scale", scale_index(sa.mode, sa.bs, sa.rs, sa.ks, by, mrow, kk[q]), 1, sa.elems, bx, wave, lane, kk[q]);
+                                    }
+                                }
+                    }
+                    // ---- epilogue (gemm.hip: coln, prow0 / rm_all, store_tile)
+                    const int rb_col = epi_col_of_lane(lane, WCOLS), rb_row = epi_row_of_lane(lane, WCOLS);
+                    const int ncol0 = n0 + wn * WCOLS + rb_col;
+                    const bool col_part = EPI == 1 || (FAST && sb.mode == 0), row_part = EPI == 1 || (FAST && sa.mode == 0);
+                    if (EPI == 1 || FAST) {
+                        const int64_t cs = col_part ? sb.rs : 0;
+                        for (int c = 0; c < 4; ++c) r.access("gemm column scale", epi_col_scale_index(by, sb.bs, ncol0 + c, (int)N, cs), 1, sb.elems, bx, wave, lane, c);
+                    }
+                    const int64_t rstride = row_part ? sa.rs : 0;
+                    const int row0 = m0 + wm * TM * 32 + rb_row;
+                    const bool col_ok = ncol0 < N;
+                    const uint32_t rs32 = (uint32_t)rstride;
+                    const uint32_t r_lim = epi_row_scale_limit(row0, (int)M, rs32);
+                    const bool mult = FAST && (row_part || col_part);
+                    if (EPI == 1 || (FAST && mult)) {
+                        const int64_t base = epi_row_scale_base(by, sa.bs, row0, (int)M, rstride);
+                        for (int i = 0; i < TM; ++i)
+                            for (int k = 0; k < NRR; ++k)
+                                r.access("gemm row scale", base + epi_row_scale_rel(i * 32 + k * RPI, rs32, r_lim), 1, sa.elems, bx, wave, lane, i * NRR + k);
+                    }
+                    int64_t off = epi_out_offset(by, bsc, row0, ldc, ncol0);
+                    const int64_t c_step = (int64_t)RPI * ldc;
+                    for (int i = 0; i < TM; ++i)
+                        for (int k = 0; k < NRR; ++k, off += c_step) {
+                            if (row0 + i * 32 + k * RPI >= M || !col_ok) continue;
+                            if (r.access("gemm C", off, 4, c_elems, bx, wave, lane, i * NRR + k) && !stored.empty())
+                                for (int c = 0; c < 4; ++c) ++stored[(size_t)(off + c)];
+                        }
+                }
+            }
+        }
+        for (size_t t = 0; t < tile_seen.size() && !r.bad; ++t)
+            if (tile_seen[t] != 1) r.fail("gemm: tile %zu of batch %lld is computed %d times", t, (long long)by, (int)tile_seen[t]);
+    }
+    // every element of C [batch][M][N] stored exactly once, nothing else touched
+    if (!stored.empty() && !r.bad) {
+        int64_t expect = 0;
+        for (int64_t b = 0; b < batch && !r.bad; ++b)
+            for (int64_t m = 0; m < M && !r.bad; ++m)
+                for (int64_t n = 0; n < N; ++n) {
+                    const int64_t o = b * bsc + m * ldc + n;
+                    if (stored[(size_t)o] != 1) {
+                        r.fail("gemm: C[%lld][%lld][%lld] stored %d times", (long long)b, (long long)m, (long long)n, (int)stored[(size_t)o]);
+                        break;
+                    }
+                    ++expect;
+                }
+        int64_t total = 0;
+        for (size_t i = 0; i < stored.size(); ++i) total += stored[i];
+        if (!r.bad && total != expect) r.fail("gemm: %lld stores, %lld elements of C", (long long)total, (long long)expect);
+    }
+    *n_checked = r.checked;
+    return r.bad;
+}
+
+}  // extern "C"

@@ -108,3 +108,20 @@ def test_python_surface_rejects_bad_inputs_without_gpu():
         T.block_channel_fwd32.triton_per_token_quant(torch.zeros(4, 100, dtype=torch.bfloat16))
     with pytest.raises(ValueError, match="bfloat16"):
         T.block_channel_fwd32.triton_gemm(None, None, None, None, out_dtype=torch.float16)
+
+
+def test_latency_harness_refuses_shapes_it_has_not_completed():
+    """No GPU needed: the shape checks come before anything touches the device.  The bwd_33 half is
+    limited to small shapes (its bf16 baseline faulted the GPU at large ones), the fwd_32 half to
+    the reference's own shape."""
+    import triton_int8_amd as T
+    with pytest.raises(ValueError, match="bwd half"):
+        T.latency.main(["--batch", "4", "--m", "8192", "--n", "8192", "--k", "8192"])
+    with pytest.raises(ValueError, match="bwd half"):
+        T.latency.main(["--halves", "bwd", "--batch", "2", "--m", "8192", "--n", "4096", "--k", "4096"])
+    with pytest.raises(ValueError, match="fwd half"):
+        T.latency.main(["--halves", "fwd", "--batch", "8", "--m", "8192", "--n", "8192", "--k", "8192"])
+    with pytest.raises(ValueError, match="multiples of 128"):
+        T.latency.check_shape(1, 100, 128, 128)
+    T.latency.check_shape(4, 8192, 8192, 8192, "fwd")
+    T.latency.check_shape(2, 256, 512, 2048, "bwd")

@@ -447,6 +447,20 @@ def test_decoder_layer_step_matches_bf16_twin(T, dev):
     assert cos(outs[0][4], outs[1][4]) > 0.3
 
 
+@pytest.mark.parametrize("scheme", ["block_channel", "double_channel", "fused", "tilelang"])
+def test_latency_harness(T, dev, scheme, capsys):
+    """The test.py-protocol harness end to end at a small shape: both halves run (the bf16 3-D x 2-D and
+    3-D x 3-D products beside fwd_32 / bwd_33), print test.py's lines and report both clocks."""
+    rep = T.latency.main(["--scheme", scheme, "--batch", "2", "--m", "256", "--n", "512", "--k", "2048", "--repeat", "6", "--warmup", "2", "--json"])
+    out = capsys.readouterr().out
+    for half in ("fwd32", "bwd33"):
+        assert f"{half}_bf16 time:" in out and f"{half}_int8 time:" in out and f"{half}_speedup:" in out
+        for leg in ("bf16", "int8"):
+            r = rep[half][leg]
+            assert r["calls"] == 4 and 0 < r["device_ms"] <= r["wall_ms"] * 1.5
+    assert T.latency.measure_latency(lambda: None, total_repeat=3, warmup=1, device=dev) >= 0
+
+
 def test_golden_vectors_on_gpu(T, dev, gemm_path):
     z = load("quant_256x256.npz")
     x = bf16(z["x"]).to(dev)

@@ -1,0 +1,189 @@
+"""Host-side bounds model of the kernels (no GPU).
+
+The kernels take every global-memory offset from triton-int8_amd/csrc/index_math.h, which also
+compiles with g++.  tests/kernel_bounds/walk.cpp walks (workgroup, wave, lane, iteration) of the
+launch an entry point would make and checks every access against the allocation it goes to.  Here
+the Python pipelines (fwd_32 / bwd_33 of every scheme) run on host tensors with the C-ABI calls
+RECORDED instead of executed, so the geometry, strides and allocation sizes are the ones the
+wrappers of ops.py produce; each recorded call is then walked.
+
+Shapes: the reference's own acceptance / latency shape B = 4, M = N = K = 8192
+(triton/block_channel_fwd32.py:257-272, test.py:32-45) and smaller ragged ones."""
+import ctypes
+import os
+import subprocess
+
+import pytest
+import torch
+
+from conftest import ROOT
+
+CSRC = os.path.join(ROOT, "triton-int8_amd", "csrc")
+SRC = os.path.join(ROOT, "tests", "kernel_bounds", "walk.cpp")
+LDS_LIMIT = 160 * 1024     # bytes of LDS per workgroup on gfx950
+NUM_CU = 256
+
+
+class ScaleArg(ctypes.Structure):
+    _fields_ = [("mode", ctypes.c_int), ("bs", ctypes.c_int64), ("rs", ctypes.c_int64), ("ks", ctypes.c_int64),
+                ("elems", ctypes.c_int64)]
+
+
+@pytest.fixture(scope="module")
+def walker(tmp_path_factory):
+    so = str(tmp_path_factory.mktemp("bounds") / "libwalk.so")
+    subprocess.run(["g++", "-O2", "-std=c++17", "-shared", "-fPIC", "-I", CSRC, "-o", so, SRC], check=True)
+    lib = ctypes.CDLL(so)
+    i64, ci, cp = ctypes.c_int64, ctypes.c_int, ctypes.c_char_p
+    p64 = ctypes.POINTER(ctypes.c_int64)
+    lib.walk_fwht.argtypes = [i64] * 8 + [p64, cp, ci]
+    lib.walk_quant_row.argtypes = [i64] * 4 + [ci] + [i64] * 3 + [p64, cp, ci]
+    lib.walk_quant_block.argtypes = [i64, i64, ci, i64, i64, ci, i64, i64, i64, i64, i64, i64, i64, i64, ci, i64, i64, i64, i64, p64, cp, ci]
+    lib.walk_gemm.argtypes = [i64] * 6 + [ctypes.POINTER(ScaleArg)] * 2 + [i64] * 4 + [ci] * 5 + [i64] * 3 + [ctypes.POINTER(ci), p64, cp, ci]
+    return lib
+
+
+class Allocations:
+    """Host stand-ins for device allocations: start address -> bytes."""
+
+    def __init__(self):
+        self.blocks = []
+        self.keep = []
+
+    def add(self, t):
+        self.blocks.append((t.data_ptr(), t.numel() * t.element_size()))
+        self.keep.append(t)
+        return t
+
+    def room(self, ptr, elem_size):
+        """Elements of `elem_size` bytes between `ptr` and the end of the allocation that holds it."""
+        if ptr is None:
+            return 0
+        for start, nbytes in self.blocks:
+            if start <= ptr < start + nbytes:
+                return (start + nbytes - ptr) // elem_size
+        raise AssertionError(f"pointer {ptr:#x} belongs to no recorded allocation")
+
+
+@pytest.fixture
+def recorded(monkeypatch):
+    """Run the Python surface on host tensors with every C-ABI call recorded instead of executed."""
+    import triton_int8_amd as T
+    allocs, calls = Allocations(), []
+    real_empty = torch.empty
+    monkeypatch.setattr(torch, "empty", lambda *a, **k: allocs.add(real_empty(*a, **k)))
+    monkeypatch.setattr(torch, "zeros", lambda *a, **k: allocs.add(real_empty(*a, **k)))   # untouched pages: no memory used
+    monkeypatch.setattr(T.ops, "_on_gpu", lambda t: True)
+    monkeypatch.setattr(T.ops, "_stream", lambda: None)
+    monkeypatch.setattr(torch.cuda, "set_device", lambda d: None)
+    monkeypatch.setattr(torch.Tensor, "cuda", lambda self, *a, **k: self)
+    monkeypatch.setattr(T._lib, "call", lambda name, *args: calls.append((name, args)))
+    yield T, allocs, calls
+
+
+def walk(lib, allocs, name, a):
+    """Walk one recorded call; returns the number of accesses checked."""
+    msg = ctypes.create_string_buffer(512)
+    n = ctypes.c_int64(0)
+    if name == "ti8_fwht":
+        x, ldx, y, ldy, rows, cols, nn = a[:7]
+        rc = lib.walk_fwht(ldx, ldy, rows, cols, nn, allocs.room(x, 2), allocs.room(y, 2), LDS_LIMIT, ctypes.byref(n), msg, 512)
+    elif name == "ti8_quant_row":
+        x, ldx, q, ldq, s, rows, cols, group = a[:8]
+        rc = lib.walk_quant_row(ldx, ldq, rows, cols, group, allocs.room(x, 2), allocs.room(q, 1), allocs.room(s, 4), ctypes.byref(n), msg, 512)
+    elif name == "ti8_quant_block":
+        x, bsx, ldx, q, bsq, ldq, qT, bsqt, ldqt, s, ssb, ssr, ssc, B, R, C, group_c = a[:17]
+        rc = lib.walk_quant_block(bsx, ldx, q is not None, bsq, ldq, qT is not None, bsqt, ldqt, ssb, ssr, ssc, B, R, C, group_c,
+                                  allocs.room(x, 2), allocs.room(q, 1), allocs.room(qT, 1), allocs.room(s, 4), ctypes.byref(n), msg, 512)
+    elif name in ("ti8_gemm_i8_nt", "ti8_gemm_i8_nt_i32"):
+        picked = (ctypes.c_int * 3)()
+        if name == "ti8_gemm_i8_nt":
+            (A, bsa, lda, B, bsb, ldb, C, bsc, ldc, sA, mA, sa_bs, sa_rs, sa_ks, sB, mB, sb_bs, sb_rs, sb_ks,
+             batch, M, N, K, acc, combine, out_scale, post_scale, flags) = a[:28]
+            sa = ScaleArg(mA, sa_bs, sa_rs, sa_ks, allocs.room(sA, 4))
+            sb = ScaleArg(mB, sb_bs, sb_rs, sb_ks, allocs.room(sB, 4))
+            rc = lib.walk_gemm(bsa, lda, bsb, ldb, bsc, ldc, ctypes.byref(sa), ctypes.byref(sb), batch, M, N, K, acc, flags & 1, (flags >> 3) & 1, 0,
+                               NUM_CU, allocs.room(A, 1), allocs.room(B, 1), allocs.room(C, 2), picked, ctypes.byref(n), msg, 512)
+        else:
+            A, bsa, lda, B, bsb, ldb, C, bsc, ldc, batch, M, N, K = a[:13]
+            rc = lib.walk_gemm(bsa, lda, bsb, ldb, bsc, ldc, None, None, batch, M, N, K, 0, 0, 0, 1,
+                               NUM_CU, allocs.room(A, 1), allocs.room(B, 1), allocs.room(C, 4), picked, ctypes.byref(n), msg, 512)
+    else:
+        raise AssertionError(f"no walker for {name}")
+    assert rc == 0, f"{name}: {msg.value.decode()}"
+    assert n.value > 0
+    return n.value
+
+
+PIPELINES = [("double_channel_fwd32", "fwd_32", False), ("double_channel_bwd33", "bwd_33", True),
+             ("block_channel_fwd32", "fwd_32", False), ("block_channel_bwd33", "bwd_33", True),
+             ("fused_fwd32", "fwd_32", False), ("fused_bwd33", "bwd_33", True),
+             ("tilelang_block_channel_fwd", "fwd_32", False), ("tilelang_block_channel_bwd", "bwd_33", True)]
+
+
+@pytest.mark.parametrize("module,fn,three_d", PIPELINES)
+@pytest.mark.parametrize("B,M,N,K", [(4, 8192, 8192, 8192), (2, 384, 640, 2048)])
+def test_every_access_of_a_pipeline_is_in_bounds(walker, recorded, module, fn, three_d, B, M, N, K):
+    """Every kernel launch of fwd_32 / bwd_33: all global accesses inside their allocations, every
+    tile computed once, every element of C stored once.  B = 4, M = N = K = 8192 is the shape of
+    the reference's self-checks and of its latency script."""
+    T, allocs, calls = recorded
+    a = torch.empty(B, M, K, dtype=torch.bfloat16)
+    b = torch.empty(B, N, K, dtype=torch.bfloat16) if three_d else torch.empty(N, K, dtype=torch.bfloat16)
+    out = getattr(getattr(T, module), fn)(a, b)
+    assert tuple(out.shape) == (B, M, N)
+    names = [c[0] for c in calls]
+    assert "ti8_gemm_i8_nt" in names and len(names) >= 3
+    total = sum(walk(walker, allocs, name, args) for name, args in calls)
+    assert total > 1000
+
+
+def test_walker_sees_an_access_past_the_end(walker):
+    """The model is not vacuous: the same launches against buffers one row too short fail."""
+    msg = ctypes.create_string_buffer(512)
+    n = ctypes.c_int64(0)
+    rows, cols = 512, 8192
+    assert walker.walk_fwht(cols, cols, rows, cols, cols, rows * cols, rows * cols, LDS_LIMIT, ctypes.byref(n), msg, 512) == 0
+    assert walker.walk_fwht(cols, cols, rows, cols, cols, rows * cols - 8, rows * cols, LDS_LIMIT, ctypes.byref(n), msg, 512) == 1
+    assert b"fwht x" in msg.value
+    assert walker.walk_fwht(cols, cols, rows, 32768, 32768, rows * 32768, rows * 32768, 64 * 1024, ctypes.byref(n), msg, 512) == 1   # LDS
+    assert walker.walk_quant_row(cols, cols, rows, cols, 0, rows * cols, rows * cols, rows, ctypes.byref(n), msg, 512) == 0
+    assert walker.walk_quant_row(cols, cols, rows, cols, 0, rows * cols, rows * cols, rows - 1, ctypes.byref(n), msg, 512) == 1
+    assert b"quant_row s" in msg.value
+    M = N = K = 512
+    sa, sb = ScaleArg(0, M, 1, 0, M), ScaleArg(0, 0, 1, 0, N)
+    picked = (ctypes.c_int * 3)()
+    ok = lambda a_el, c_el, large: walker.walk_gemm(M * K, K, 0, K, M * N, N, ctypes.byref(sa), ctypes.byref(sb), 1, M, N, K, 1, 0, large, 0, NUM_CU,
+                                                    a_el, N * K, c_el, picked, ctypes.byref(n), msg, 512)
+    assert ok(M * K, M * N, 0) == 0 and tuple(picked) == (128, 128, 1)
+    assert ok(M * K, M * N, 1) == 0 and tuple(picked) == (256, 256, 1)
+    assert ok(M * K - 16, M * N, 1) == 1 and b"gemm A" in msg.value
+    assert ok(M * K, M * N - 4, 0) == 1 and b"gemm C" in msg.value
+
+
+@pytest.mark.parametrize("M,N,K,batch,mA,mB,acc,flags", [
+    (8192, 4096, 4096, 1, 1, 0, 0, 0),      # config 2 Y / dX: chained promotion kernel on 256 x 256 tiles
+    (4096, 4096, 8192, 1, 1, 1, 0, 0),      # config 2 dW: block x block
+    (16384, 14336, 4096, 1, 0, 0, 1, 0),    # config 3 gate/up: int32 kernel
+    (14336, 4096, 16384, 1, 1, 1, 0, 0),    # config 5 down_proj dW: K = 16384
+    (1536, 1024, 1024, 1, 1, 0, 0, 8),      # incomplete group of tile rows + XCD remap, 256 x 256 tiles
+    (4608, 2048, 512, 1, 0, 1, 0, 0),       # 256 x 128 tiles
+    (640, 384, 640, 3, 1, 1, 0, 0),         # 128 x 128 tiles, tiles that hang over M and N
+    (640, 384, 640, 3, 1, 1, 0, 8),         # the same on 256 x 256 tiles: the re-read of the valid half
+    (384, 256, 33024, 2, 1, 0, 0, 0),       # K > 32768: literal kernel
+    (256, 384, 1024, 2, 1, 2, 0, 2),        # per-(column, K tile) scales of B
+])
+def test_gemm_launch_geometries(walker, M, N, K, batch, mA, mB, acc, flags):
+    """The GEMM kernels at the benchmark shapes and at shapes whose tiles hang over the edges."""
+    nkb = K // 128
+    def desc(mode, rows, batched):
+        per_batch = {0: rows, 1: -(-rows // 128) * nkb, 2: rows * nkb, 3: -(-rows // 128) * (nkb // 2)}[mode]
+        rs = {0: 1, 1: nkb, 2: nkb, 3: nkb // 2}[mode]
+        return ScaleArg(mode, per_batch if batched else 0, rs, 0 if mode == 0 else 1, per_batch * (batch if batched else 1))
+    sa, sb = desc(mA, M, True), desc(mB, N, False)
+    msg = ctypes.create_string_buffer(512)
+    n = ctypes.c_int64(0)
+    picked = (ctypes.c_int * 3)()
+    rc = walker.walk_gemm(M * K, K, 0, K, M * N, N, ctypes.byref(sa), ctypes.byref(sb), batch, M, N, K, acc, flags & 1, (flags >> 3) & 1, 0,
+                          NUM_CU, batch * M * K, N * K, batch * M * N, picked, ctypes.byref(n), msg, 512)
+    assert rc == 0, msg.value.decode()

@@ -17,10 +17,11 @@
 // Compile with -ffp-contract=off (the optional scale multiply must not fuse with a
 // butterfly).
 #include "ti8_common.h"
+#include "index_math.h"
 
 namespace ti8 {
 
-__device__ __forceinline__ int padded(int i) { return i + (i >> 4); }
+__device__ __forceinline__ int padded(int i) { return idx::fwht_padded(i); }
 
 template <int RB>
 __device__ __forceinline__ void butterflies(float (&a)[1 << RB]) {
@@ -41,9 +42,7 @@ __device__ __forceinline__ void pass_in_lds(float* lds, int L, int p, int tid) {
     constexpr int RAD = 1 << RB;
     const int ngroups = L >> RB;
     for (int vt = tid; vt < ngroups; vt += NT) {
-        const int lo = vt & ((1 << p) - 1);
-        const int hi = vt >> p;
-        const int base = (hi << (p + RB)) | lo;
+        const int base = idx::fwht_group_base(vt, p, RB);
         float a[RAD];
 #pragma unroll
         for (int e = 0; e < RAD; ++e) a[e] = lds[padded(base + (e << p))];
@@ -73,10 +72,8 @@ __global__ __launch_bounds__(NT) void fwht_kernel(const uint16_t* __restrict__ x
     extern __shared__ float lds[];
     const int tid = threadIdx.x;
     const int segs_per_row = cols / L;
-    const int64_t row = blockIdx.x / segs_per_row;
-    const int seg = blockIdx.x % segs_per_row;
-    const uint16_t* xr = x + row * ldx + (int64_t)seg * L;
-    uint16_t* yr = y + row * ldy + (int64_t)seg * L;
+    const uint16_t* xr = x + idx::fwht_segment_offset(blockIdx.x, segs_per_row, ldx, L);
+    uint16_t* yr = y + idx::fwht_segment_offset(blockIdx.x, segs_per_row, ldy, L);
 
     // pass over bits 0..3 (n >= 128, so all four stages belong to every group)
     for (int vt = tid; vt < (L >> 4); vt += NT) {
@@ -132,21 +129,14 @@ extern "C" int ti8_fwht(const void* x, int64_t ldx, void* y, int64_t ldy, int64_
     if (!x || !y) return fail(TI8_ERR_NULL, "ti8_fwht: x and y are required");
     if (n < 128 || n > 32768 || (n & (n - 1))) return fail(TI8_ERR_SHAPE, "ti8_fwht: n must be a power of two in [128, 32768], got %lld", (long long)n);
     if (rows <= 0 || cols <= 0 || cols % n) return fail(TI8_ERR_SHAPE, "ti8_fwht: need rows>0 and cols%%n==0; got rows=%lld cols=%lld n=%lld", (long long)rows, (long long)cols, (long long)n);
-    // elements per workgroup: a whole group when n >= 2048, else as many groups as divide
-    // both the row and 2048
-    int64_t L = n;
-    if (n < 2048) {
-        int64_t a = cols, b = 2048;
-        while (b) { const int64_t t = a % b; a = b; b = t; }
-        L = a;  // gcd(cols, 2048), a multiple of n because n divides both
-    }
+    const int64_t L = idx::fwht_segment_len(cols, n);   // elements per workgroup
     if (ldx < cols || ldy < cols) return fail(TI8_ERR_SHAPE, "ti8_fwht: leading dimension smaller than cols");
     if (!aligned16(x) || !aligned16(y) || (ldx % 8) || (ldy % 8)) return fail(TI8_ERR_ALIGN, "ti8_fwht: pointers must be 16-byte aligned and strides multiples of 16 bytes");
     const int64_t nblocks = rows * (cols / L);
     if (nblocks > 0x7fffffffLL) return fail(TI8_ERR_SHAPE, "ti8_fwht: too many segments");
     int logn = 0;
     while ((1LL << logn) < n) ++logn;
-    const size_t shmem = (size_t)(L + L / 16) * sizeof(float);
+    const size_t shmem = (size_t)idx::fwht_lds_words(L) * sizeof(float);
     static thread_local int attr_set_for = -1;
     int dev = 0;
     (void)hipGetDevice(&dev);
@@ -155,7 +145,7 @@ extern "C" int ti8_fwht(const void* x, int64_t ldx, void* y, int64_t ldy, int64_
         if (e != hipSuccess) return fail(TI8_ERR_HIP, "ti8_fwht: cannot raise the LDS limit: %s", hipGetErrorString(e));
         attr_set_for = dev;
     }
-    if (L >= 16384)
+    if (idx::fwht_threads(L) == 1024)
         hipLaunchKernelGGL(fwht_kernel<1024>, dim3((unsigned)nblocks), dim3(1024), shmem, static_cast<hipStream_t>(stream),
                            static_cast<const uint16_t*>(x), ldx, static_cast<uint16_t*>(y), ldy, (int)cols, logn, (int)L, scale);
     else

@@ -69,21 +69,14 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
     const int wm = wave / WN, wn = wave % WN;
 
     // ---- tile assignment: XCD-aware remap, then groups of GROUP tile rows -------------
-    const int ntiles = g.tiles_m * g.tiles_n;
-    int pid = blockIdx.x;
-    if ((ntiles & 7) == 0) pid = (pid & 7) * (ntiles >> 3) + (pid >> 3);  // one contiguous range per XCD
-    // tile rows per group: the 32 workgroups one XCD runs at a time then cover GROUP x 32/GROUP
-    // tiles, chosen so that the A and B panels they share are about the same size (256-row tiles:
-    // 4 measured 0.4 % faster than 8 and 1 % faster than 16 on 8192 x 4096 x 4096)
-    constexpr int GROUP = (BM >= 256) ? 4 : 8;
-    const int per_group = GROUP * g.tiles_n;
-    const int group_id = pid / per_group;
-    const int first_m = group_id * GROUP;
-    const int gsz = min(g.tiles_m - first_m, GROUP);
-    const int tile_m = first_m + (pid % per_group) % gsz;
-    const int tile_n = (pid % per_group) / gsz;
+    // one contiguous range of tiles per XCD, then groups of GROUP tile rows: the 32 workgroups one
+    // XCD runs at a time then cover GROUP x 32/GROUP tiles, chosen so that the A and B panels they
+    // share are about the same size (256-row tiles: 4 measured 0.4 % faster than 8 and 1 % faster
+    // than 16 on 8192 x 4096 x 4096)
+    constexpr int GROUP = idx::gemm_group_rows(BM);
+    const idx::TileCoord tc = idx::gemm_tile_of(blockIdx.x, g.tiles_m, g.tiles_n, GROUP);
     const int batch = blockIdx.y;
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int m0 = tc.tile_m * BM, n0 = tc.tile_n * BN;
 
     const int8_t* Ab = g.A + (int64_t)batch * g.bsa;
     const int8_t* Bb = g.B + (int64_t)batch * g.bsb;
@@ -95,20 +88,16 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
     // then sit in 16 distinct 16-byte bank groups.
     // Address = (uniform row base of the instruction, SGPRs) + (per-lane 32-bit offset, one
     // VGPR per parity of t): keeps the loop's address registers to four VGPRs.
-    const int ld_row = lane >> 3;
     uint32_t voffA[2], voffB[2];
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
-        const int ch = (lane & 7) ^ ld_row ^ p;
-        voffA[p] = (uint32_t)(ld_row * (int)g.lda + ch * 16);
-        voffB[p] = (uint32_t)(ld_row * (int)g.ldb + ch * 16);
+        voffA[p] = idx::gemm_lane_offset_bytes(lane, p, (int)g.lda);
+        voffB[p] = idx::gemm_lane_offset_bytes(lane, p, (int)g.ldb);
     }
     // a wave's instructions cover A_INSTR*8 consecutive tile rows (a divisor of 128): if they
     // start past M (a multiple of 128) they re-read the valid half; those results are masked
     static_assert(128 % (A_INSTR * 8) == 0 && 128 % (B_INSTR * 8) == 0, "a wave's rows must not straddle a 128-row boundary");
-    int rA0 = m0 + wave * A_INSTR * 8, rB0 = n0 + wave * B_INSTR * 8;
-    if (rA0 >= g.M) rA0 -= 128;
-    if (rB0 >= g.N) rB0 -= 128;
+    const int rA0 = idx::gemm_wave_first_row(m0, wave, A_INSTR, g.M), rB0 = idx::gemm_wave_first_row(n0, wave, B_INSTR, g.N);
     const int8_t* const baseA = Ab + (int64_t)rA0 * g.lda;  // wave-uniform
     const int8_t* const baseB = Bb + (int64_t)rB0 * g.ldb;
     const int64_t strideA8 = 8 * g.lda, strideB8 = 8 * g.ldb;
@@ -156,32 +145,29 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
     const float* pfb[TN];  // LANEB: this lane's column of B's scale grid
     if (FAST) {
         static_assert(!FAST || (128 % (TM * 32) == 0 && 128 % (TN * 32) == 0), "a wave tile must lie inside one 128 x 128 scale block");
-        const int rowblk = min(m0 + wm * TM * 32, g.M - 1) >> 7;
-        const float* pa = g.sa.p + batch * g.sa.bs + (int64_t)rowblk * g.sa.rs;
-        const int colblk = min(n0 + wn * TN * 32, g.N - 1) >> 7;
-        const float* pb = g.sb.p + batch * g.sb.bs + (int64_t)colblk * g.sb.rs;
+        const int rowblk = idx::gemm_factor_block(m0 + wm * TM * 32, g.M);
+        const int colblk = idx::gemm_factor_block(n0 + wn * TN * 32, g.N);
         const int nkt = g.K >> 7;
         // unconditional loads (an operand without in-loop factors is read with stride 0 and its
         // value dropped): a load under a branch is waited for on the spot, one after the other
         const int64_t ska = a_in ? g.sa.ks : 0, skb = (b_in && !LANEB) ? g.sb.ks : 0;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            const int kt = min(c * 64 + lane, nkt - 1);
-            fraw_a[c] = pa[(int64_t)(kt >> sha) * ska];
-            fraw_b[c] = pb[(int64_t)(kt >> shb) * skb];
+            const int kt = idx::gemm_factor_kt(c, lane, nkt);
+            fraw_a[c] = g.sa.p[idx::gemm_factor_index(batch, g.sa.bs, rowblk, g.sa.rs, kt, sha, ska)];
+            fraw_b[c] = g.sb.p[idx::gemm_factor_index(batch, g.sb.bs, colblk, g.sb.rs, kt, shb, skb)];
         }
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-            const int col = min(n0 + (wn * TN + j) * 32 + fr_row, g.N - 1);
-            pfb[j] = g.sb.p + batch * g.sb.bs + (int64_t)col * g.sb.rs;
+            pfb[j] = g.sb.p + idx::epi_col_scale_index(batch, g.sb.bs, n0 + (wn * TN + j) * 32 + fr_row, g.N, g.sb.rs);
         }
     }
     // column scale vector of the epilogue (4 columns per lane there), fetched now for the same reason
     constexpr int WCOLS = TN * 32;                       // columns of the wave tile
     constexpr int LPR = WCOLS / 4;                       // lanes per row in the epilogue's read-back
     constexpr int RPI = 64 / LPR;                        // rows per wave instruction there
-    const int rb_col = (lane % LPR) * 4;
-    const int rb_row = lane / LPR;
+    const int rb_col = idx::epi_col_of_lane(lane, WCOLS);
+    const int rb_row = idx::epi_row_of_lane(lane, WCOLS);
     const int ncol0 = n0 + wn * WCOLS + rb_col;          // first of this lane's 4 columns
     const bool col_part = EPI == EPI_ROWS || (FAST && g.sb.mode == TI8_SCALE_ROW);
     const bool row_part = EPI == EPI_ROWS || (FAST && g.sa.mode == TI8_SCALE_ROW);
@@ -189,7 +175,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
     if (EPI == EPI_ROWS || FAST) {
         const int64_t cs = col_part ? g.sb.rs : 0;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) coln[c] = g.sb.p[batch * g.sb.bs + (int64_t)min(ncol0 + c, g.N - 1) * cs];
+        for (int c = 0; c < 4; ++c) coln[c] = g.sb.p[idx::epi_col_scale_index(batch, g.sb.bs, ncol0 + c, g.N, cs)];
     }
     float f_cur = 1.0f;   // wave-uniform factor of the K tile being accumulated
     float fb[TN];         // LANEB only: per-lane factors of that tile
@@ -268,10 +254,10 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     const int klast = (nk - 1) * 128;  // loads past the last K tile re-read it into a free buffer: no branches in the loop
-    issue_tile_loads<A_INSTR>(baseA + min(128, klast), strideA8, voffA, tA0, wA + A_BYTES);
+    issue_tile_loads<A_INSTR>(baseA + idx::gemm_k_offset(1, klast), strideA8, voffA, tA0, wA + A_BYTES);
     // (the chained kernel issues the B half of tile kt+1 at the top of iteration kt instead: with
     // both halves behind its barrier it measured 1 % slower, the other kernels 2.5 % faster)
-    if constexpr (!CHAIN) issue_tile_loads<B_INSTR>(baseB + min(128, klast), strideB8, voffB, tB0, wB + B_BYTES);
+    if constexpr (!CHAIN) issue_tile_loads<B_INSTR>(baseB + idx::gemm_k_offset(1, klast), strideB8, voffB, tB0, wB + B_BYTES);
     if constexpr (CHAIN) {
         // Promotion without int32 accumulators that outlive a K tile: a 32 x 32 block's four MFMAs of
         // a K tile chain into a temporary (two blocks of one block row interleaved, so that
@@ -305,7 +291,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
             const int8_t* stAn = ldsA + (cur ^ 1) * A_BYTES;
             const int8_t* stBn = ldsB + (cur ^ 1) * B_BYTES;
             load_factors(kt);
-            issue_tile_loads<B_INSTR>(baseB + min((kt + 1) * 128, klast), strideB8, voffB, tB0, wB + (cur ^ 1) * B_BYTES);
+            issue_tile_loads<B_INSTR>(baseB + idx::gemm_k_offset(kt + 1, klast), strideB8, voffB, tB0, wB + (cur ^ 1) * B_BYTES);
 #pragma unroll
             for (int i = 0; i < TM - 1; ++i) {
                 read_a((i + 1) & 1, stA, i + 1);
@@ -324,7 +310,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
             // last block row: tile kt+1 has landed, its fragments replace those of tile kt as they retire
             __builtin_amdgcn_s_waitcnt(0);
             __syncthreads();
-            issue_tile_loads<A_INSTR>(baseA + min((kt + 2) * 128, klast), strideA8, voffA, tA0, wA + cur * A_BYTES);
+            issue_tile_loads<A_INSTR>(baseA + idx::gemm_k_offset(kt + 2, klast), strideA8, voffA, tA0, wA + cur * A_BYTES);
             constexpr int LB = (TM - 1) & 1;   // buffer that holds the last block row
             read_a(LB ^ 1, stAn, 0);
             __builtin_amdgcn_sched_barrier(0);
@@ -373,8 +359,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
         __builtin_amdgcn_s_waitcnt(0);  // tile kt+1 landed; every read of buffer `cur` returned
         __syncthreads();
         // k-step 3
-        issue_tile_loads<A_INSTR>(baseA + min((kt + 2) * 128, klast), strideA8, voffA, tA0, wA + cur * A_BYTES);
-        issue_tile_loads<B_INSTR>(baseB + min((kt + 2) * 128, klast), strideB8, voffB, tB0, wB + cur * B_BYTES);
+        issue_tile_loads<A_INSTR>(baseA + idx::gemm_k_offset(kt + 2, klast), strideA8, voffA, tA0, wA + cur * A_BYTES);
+        issue_tile_loads<B_INSTR>(baseB + idx::gemm_k_offset(kt + 2, klast), strideB8, voffB, tB0, wB + cur * B_BYTES);
         load_frags(0, ldsA + (cur ^ 1) * A_BYTES + a_row_off, ldsB + (cur ^ 1) * B_BYTES + b_row_off, 0);
         if (FAST) {
             mfmas_promote(1);
@@ -425,8 +411,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
     static_assert(WCOLS * 32 * 4 * NW <= 2 * (A_BYTES + B_BYTES), "epilogue slab does not fit");
     uint32_t* slab = reinterpret_cast<uint32_t*>(smem) + wave * (32 * WCOLS);
     constexpr int NRR = 32 / RPI;                        // rows of a 32-row block per lane
-    const float* prow = g.sa.p + batch * g.sa.bs;        // per-row scales of A (unused pointer otherwise)
-    const int64_t rstride = row_part ? g.sa.rs : 0;
+    const int64_t rstride = row_part ? g.sa.rs : 0;      // per-row scales of A (read with stride 0 and dropped otherwise)
     // Everything that does not change from element to element is settled here, so that an
     // element costs its multiplications and nothing else: operands without a row / column scale
     // vector multiply by 1 (exact), the rarely used extra factors pick a copy of the loop below
@@ -436,13 +421,13 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
     for (int c = 0; c < 4; ++c) cm[c] = col_part ? coln[c] : 1.0f;
     const int row0 = m0 + wm * TM * 32 + rb_row;          // this lane's first output row
     const bool col_ok = ncol0 < g.N;                      // N is a multiple of 4: a lane's 4 columns are all in or all out
-    const int64_t c_off = (int64_t)batch * g.bsc + (int64_t)row0 * g.ldc + ncol0;
+    const int64_t c_off = idx::epi_out_offset(batch, g.bsc, row0, g.ldc, ncol0);
     const int64_t c_step = (int64_t)RPI * g.ldc;          // uniform: the output address advances by scalar adds
     // row scales: row0 + d for d = 0, RPI, ... clamped to the last row; d * stride is uniform and
     // the clamp is one v_min against this lane's limit (32-bit offsets: 128 rows x stride)
-    const float* prow0 = prow + (int64_t)min(row0, g.M - 1) * rstride;
+    const float* prow0 = g.sa.p + idx::epi_row_scale_base(batch, g.sa.bs, row0, g.M, rstride);
     const uint32_t rs32 = static_cast<uint32_t>(rstride);
-    const uint32_t r_lim = static_cast<uint32_t>(max(g.M - 1 - row0, 0)) * rs32;
+    const uint32_t r_lim = idx::epi_row_scale_limit(row0, g.M, rs32);
     auto store_tile = [&](auto extra_tag, auto mult_tag) {
         constexpr bool EXTRA = decltype(extra_tag)::value;  // EPI_ROWS: post_scale, promotion: out_scale
         constexpr bool MULT = decltype(mult_tag)::value;    // promotion: some operand has a row / column scale vector
@@ -455,7 +440,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int k = 0; k < NRR; ++k) rm_all[i][k] = prow0[min(static_cast<uint32_t>(i * 32 + k * RPI) * rs32, r_lim)];
+                for (int k = 0; k < NRR; ++k) rm_all[i][k] = prow0[idx::epi_row_scale_rel(i * 32 + k * RPI, rs32, r_lim)];
         }
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
@@ -629,22 +614,18 @@ extern "C" int ti8_gemm_i8_nt(const int8_t* A, int64_t bsa, int64_t lda, const i
         (void)hipGetDevice(&dev);
         num_cu = (hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
     }
-    const int64_t tiles_256x256 = ((M + 255) / 256) * ((N + 255) / 256) * batch;
-    const int64_t tiles_256x128 = ((M + 255) / 256) * (N / 128) * batch;
-    if (acc_i32_full) {
-        if (!large && tiles_256x256 < num_cu) return launch<128, 128, 2, 2, EPI_ROWS>(a, batch, st);
-        return launch<256, 256, 2, 4, EPI_ROWS>(a, batch, st);
-    }
-    // the fast promotion keeps at most 256 per-K-tile factors in registers and cannot apply a
-    // factor that varies per row of A inside the loop: those cases take the literal kernel
-    const bool a_loop_per_row = (modeA == TI8_SCALE_ROW_K128);
-    if (a.strict || a_loop_per_row || K > 256 * 128) return launch<128, 128, 2, 2, EPI_STRICT>(a, batch, st);
-    if (modeB == TI8_SCALE_ROW_K128) return launch<256, 128, 4, 2, EPI_PROMOTE_LANE>(a, batch, st);
-    // 256 x 256 tiles (128 x 64 per wave, float accumulators only) where they fill the machine, else
-    // 256 x 128 (64 x 64 per wave, int32 + float accumulators), else 128 x 128
-    if (large || tiles_256x256 >= num_cu) return launch<256, 256, 2, 4, EPI_PROMOTE_CHAIN>(a, batch, st);
-    if (tiles_256x128 >= num_cu) return launch<256, 128, 4, 2, EPI_PROMOTE>(a, batch, st);
-    return launch<128, 128, 2, 2, EPI_PROMOTE>(a, batch, st);
+    const idx::GemmConfig c = idx::gemm_config(M, N, K, batch, acc_i32_full != 0, a.strict != 0, modeA, modeB, large, num_cu);
+#define TI8_GEMM_CASE(BM, BN, WM, WN, EPI) \
+    if (c.bm == BM && c.bn == BN && c.epi == EPI) return launch<BM, BN, WM, WN, EPI>(a, batch, st)
+    TI8_GEMM_CASE(128, 128, 2, 2, EPI_ROWS);
+    TI8_GEMM_CASE(256, 256, 2, 4, EPI_ROWS);
+    TI8_GEMM_CASE(128, 128, 2, 2, EPI_STRICT);
+    TI8_GEMM_CASE(256, 128, 4, 2, EPI_PROMOTE_LANE);
+    TI8_GEMM_CASE(256, 256, 2, 4, EPI_PROMOTE_CHAIN);
+    TI8_GEMM_CASE(256, 128, 4, 2, EPI_PROMOTE);
+    TI8_GEMM_CASE(128, 128, 2, 2, EPI_PROMOTE);
+#undef TI8_GEMM_CASE
+    return fail(TI8_ERR_MODE, "%s: no kernel for tile %d x %d, epilogue %d", fn, c.bm, c.bn, c.epi);
 }
 
 extern "C" int ti8_gemm_i8_nt_i32(const int8_t* A, int64_t bsa, int64_t lda, const int8_t* B, int64_t bsb, int64_t ldb,

@@ -1,6 +1,7 @@
 // Argument block, scale descriptors and epilogue kinds shared by the INT8 GEMM kernels.
 #pragma once
 #include "ti8_common.h"
+#include "index_math.h"
 
 namespace ti8 {
 
@@ -31,12 +32,7 @@ enum { EPI_I32 = 0, EPI_ROWS = 1, EPI_PROMOTE = 2, EPI_STRICT = 3, EPI_PROMOTE_L
 
 // scale of operand row `row` at K block kb
 __device__ __forceinline__ float scale_at(const ScaleDesc& d, int64_t batch, int row, int kb) {
-    switch (d.mode) {
-        case TI8_SCALE_ROW: return d.p[batch * d.bs + (int64_t)row * d.rs];
-        case TI8_SCALE_BLOCK128: return d.p[batch * d.bs + (int64_t)(row >> 7) * d.rs + (int64_t)kb * d.ks];
-        case TI8_SCALE_ROW_K128: return d.p[batch * d.bs + (int64_t)row * d.rs + (int64_t)kb * d.ks];
-        default: return d.p[batch * d.bs + (int64_t)(row >> 7) * d.rs + (int64_t)(kb >> 1) * d.ks];
-    }
+    return d.p[idx::scale_index(d.mode, d.bs, d.rs, d.ks, batch, row, kb)];
 }
 
 // One wave's share of a K tile: NI global->LDS instructions of 64 x 16 bytes; instruction i
@@ -53,7 +49,7 @@ __device__ __forceinline__ void issue_tile_loads(const int8_t* base, int64_t str
     asm volatile("" : "+v"(vo[0]), "+v"(vo[1]));
 #pragma unroll
     for (int i = 0; i < NI; ++i)
-        __builtin_amdgcn_global_load_lds(base + i * stride8 + vo[(t0 + i) & 1], lds + i * 1024, 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(base + i * stride8 + vo[(t0 + i) & 1], lds + i * 1024, 16, 0, 0);   // = idx::gemm_load_offset_bytes
 #else
     (void)base; (void)stride8; (void)voff; (void)t0; (void)lds;
 #endif

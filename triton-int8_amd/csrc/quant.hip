@@ -7,6 +7,7 @@
 #include <mutex>
 
 #include "ti8_common.h"
+#include "index_math.h"
 
 namespace ti8 {
 
@@ -170,17 +171,14 @@ __global__ __launch_bounds__(256) void quant_block_kernel(
     __shared__ float red4[4];
     __shared__ uint32_t tileT[WRITE_QT ? 128 * 33 : 1];
 
-    int tile = blockIdx.x;
-    const int cb = tile % ncb;
-    tile /= ncb;
-    const int rb = tile % nrb;
-    const int b = tile / nrb;
+    const idx::TileId tl = idx::qblock_tile(blockIdx.x, nrb, ncb);
+    const int b = tl.b, rb = tl.rb, cb = tl.cb;
 
     const int tid = threadIdx.x;
     const int cc = tid & 15;   // 8-column chunk
     const int rg = tid >> 4;   // 4-row group
 
-    const uint16_t* xt = x + b * bsx + (int64_t)rb * 128 * ldx + (int64_t)cb * (128 * NSUB);
+    const uint16_t* xt = x + idx::qblock_origin(b, bsx, rb, ldx, cb, 128 * NSUB);
     uint4 v[NSUB][2][4];
 #pragma unroll
     for (int u = 0; u < NSUB; ++u)
@@ -188,8 +186,8 @@ __global__ __launch_bounds__(256) void quant_block_kernel(
         for (int h = 0; h < 2; ++h)
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const int row = h * 64 + rg * 4 + j;
-                v[u][h][j] = *reinterpret_cast<const uint4*>(xt + (int64_t)row * ldx + u * 128 + cc * 8);
+                const int row = idx::qblock_row(tid, h, j);
+                v[u][h][j] = *reinterpret_cast<const uint4*>(xt + (int64_t)row * ldx + u * 128 + idx::qblock_col(tid));
             }
 
     float amax = 0.0f;
@@ -213,12 +211,12 @@ __global__ __launch_bounds__(256) void quant_block_kernel(
             for (int j = 0; j < 4; ++j) o[h][j] = quant8(v[u][h][j], scale);
 
         if (WRITE_Q) {
-            int8_t* qt = q + b * bsq + (int64_t)rb * 128 * ldq + (int64_t)cb * (128 * NSUB) + u * 128 + cc * 8;
+            int8_t* qt = q + idx::qblock_origin(b, bsq, rb, ldq, cb, 128 * NSUB) + u * 128 + idx::qblock_col(tid);
 #pragma unroll
             for (int h = 0; h < 2; ++h)
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
-                    *reinterpret_cast<uint2*>(qt + (int64_t)(h * 64 + rg * 4 + j) * ldq) = o[h][j];
+                    *reinterpret_cast<uint2*>(qt + (int64_t)idx::qblock_row(tid, h, j) * ldq) = o[h][j];
         }
         if (WRITE_QT) {  // NSUB == 1 only (checked on the host)
 #pragma unroll
@@ -231,11 +229,11 @@ __global__ __launch_bounds__(256) void quant_block_kernel(
                 for (int e = 0; e < 8; ++e) tileT[(cc * 8 + e) * 33 + h * 16 + rg] = w[e];  // [column of x][4-row group]
             }
             __syncthreads();
-            int8_t* qtt = qT + b * bsqt + (int64_t)cb * 128 * ldqt + (int64_t)rb * 128;
+            int8_t* qtt = qT + idx::qblock_origin(b, bsqt, cb, ldqt, rb, 128);   // tile (cb, rb) of the transposed tensor
 #pragma unroll
             for (int p = 0; p < 4; ++p) {
-                const int tr = p * 32 + (tid >> 3);  // row of the transposed tile = column of x
-                const int tc = tid & 7;              // 16-byte chunk along the original rows
+                const int tr = idx::qblock_t_row(tid, p);  // row of the transposed tile = column of x
+                const int tc = tid & 7;                    // 16-byte chunk along the original rows
                 uint4 w;
                 w.x = tileT[tr * 33 + tc * 4 + 0];
                 w.y = tileT[tr * 33 + tc * 4 + 1];
@@ -372,7 +370,7 @@ __global__ __launch_bounds__(256) void quant_row_kernel(const uint16_t* __restri
     __shared__ float red4[4];
     constexpr int T = WG_ROW ? 256 : 64;
     const int t = WG_ROW ? threadIdx.x : (threadIdx.x & 63);
-    const int64_t row = WG_ROW ? (int64_t)blockIdx.x : (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t row = idx::qrow_row(blockIdx.x, threadIdx.x >> 6, WG_ROW);
     if (row >= rows) return;  // whole wave (or workgroup) leaves together
     const int nchunk = cols >> 3;
     const uint16_t* xr = x + row * ldx;
@@ -380,7 +378,7 @@ __global__ __launch_bounds__(256) void quant_row_kernel(const uint16_t* __restri
     uint4 v[NLOAD];
 #pragma unroll
     for (int i = 0; i < NLOAD; ++i) {
-        const int c = t + i * T;
+        const int c = idx::qrow_chunk(t, i, T);
         v[i] = (c < nchunk) ? *reinterpret_cast<const uint4*>(xr + c * 8) : make_uint4(0, 0, 0, 0);
         // chunks c, c^1, ... c^15 of a 128-column group sit in 16 consecutive lanes (T % 16 == 0)
         if (HAD) v[i] = fwht128_bf16(v[i], threadIdx.x & 63);
@@ -412,7 +410,7 @@ __global__ __launch_bounds__(256) void quant_row_kernel(const uint16_t* __restri
     if (t == 0) s[row] = stored_scale(amax, scale, mode);
 #pragma unroll
     for (int i = 0; i < NLOAD; ++i) {
-        const int c = t + i * T;
+        const int c = idx::qrow_chunk(t, i, T);
         if (c < nchunk) *reinterpret_cast<uint2*>(qr + c * 8) = quant8(v[i], scale);
     }
 }
@@ -711,17 +709,19 @@ extern "C" int ti8_quant_row(const void* x, int64_t ldx, int8_t* q, int64_t ldq,
 #define TI8_LAUNCH_QR(NL, WG, G16, GRID) \
     do { if (had) hipLaunchKernelGGL((quant_row_kernel<NL, WG, G16, true>), dim3((unsigned)(GRID)), dim3(256), 0, st, xp, ldx, q, ldq, s, rows, c, mode); \
          else hipLaunchKernelGGL((quant_row_kernel<NL, WG, G16, false>), dim3((unsigned)(GRID)), dim3(256), 0, st, xp, ldx, q, ldq, s, rows, c, mode); } while (0)
-    const int64_t g4 = (rows + 3) / 4;
+    const idx::QRowConfig cfg = idx::qrow_config(nchunk, group == 128);
+    const int64_t grid = cfg.wg_row ? rows : (rows + 3) / 4;
     if (group == 128) {
-        if (nchunk <= 64 * 8) TI8_LAUNCH_QR(8, false, true, g4);
-        else if (nchunk <= 256 * 8) TI8_LAUNCH_QR(8, true, true, rows);
-        else TI8_LAUNCH_QR(16, true, true, rows);
-    } else if (nchunk <= 64 * 2) TI8_LAUNCH_QR(2, false, false, g4);
-    else if (nchunk <= 64 * 4) TI8_LAUNCH_QR(4, false, false, g4);
-    else if (nchunk <= 64 * 8) TI8_LAUNCH_QR(8, false, false, g4);
-    else if (nchunk <= 256 * 4) TI8_LAUNCH_QR(4, true, false, rows);
-    else if (nchunk <= 256 * 8) TI8_LAUNCH_QR(8, true, false, rows);
-    else TI8_LAUNCH_QR(16, true, false, rows);
+        if (!cfg.wg_row) TI8_LAUNCH_QR(8, false, true, grid);
+        else if (cfg.nload == 8) TI8_LAUNCH_QR(8, true, true, grid);
+        else TI8_LAUNCH_QR(16, true, true, grid);
+    } else if (!cfg.wg_row) {
+        if (cfg.nload == 2) TI8_LAUNCH_QR(2, false, false, grid);
+        else if (cfg.nload == 4) TI8_LAUNCH_QR(4, false, false, grid);
+        else TI8_LAUNCH_QR(8, false, false, grid);
+    } else if (cfg.nload == 4) TI8_LAUNCH_QR(4, true, false, grid);
+    else if (cfg.nload == 8) TI8_LAUNCH_QR(8, true, false, grid);
+    else TI8_LAUNCH_QR(16, true, false, grid);
 #undef TI8_LAUNCH_QR
     return check_launch("ti8_quant_row");
 }

@@ -26,13 +26,19 @@ def _stream():
     return torch.cuda.current_stream().cuda_stream
 
 
+def _on_gpu(t):
+    """Whether a tensor lives in device memory.  One place, so that a host-side model of the launches
+    (tests that record the C-ABI calls these wrappers make, without a GPU) can stand in for it."""
+    return t.is_cuda
+
+
 def _need(cond, msg):
     if not cond:
         raise ValueError(msg)
 
 
 def _check_bf16(x, name):
-    _need(isinstance(x, torch.Tensor) and x.is_cuda, f"{name} must be a tensor on the GPU")
+    _need(isinstance(x, torch.Tensor) and _on_gpu(x), f"{name} must be a tensor on the GPU")
     _need(x.dtype == torch.bfloat16, f"{name} must be bfloat16, got {x.dtype}")
 
 
@@ -223,7 +229,7 @@ def _k_contig(t):
 
 def _scale_desc(s, mode, rows, nkb, batch, batched, who):
     """(ptr, batch stride, row stride, k stride) of a scale tensor for operand `who`."""
-    _need(s.dtype == torch.float32 and s.is_cuda, f"{who} scale must be a float32 GPU tensor")
+    _need(s.dtype == torch.float32 and _on_gpu(s), f"{who} scale must be a float32 GPU tensor")
     if mode == SCALE_ROW:
         shape = (batch, rows) if batched else (rows,)
         _need(s.numel() == batch * rows if batched else s.numel() == rows,
@@ -246,7 +252,7 @@ def _scale_desc(s, mode, rows, nkb, batch, batched, who):
 def gemm_i8_nt(A, B, sA, modeA, sB, modeB, *, acc_i32_full=False, combine=COMBINE_MUL_MUL, out_scale=1.0,
                post_scale=0.0, strict=False, out=None):
     """C[b] = dequant(A[b] @ B[b]^T): A int8 [batch, M, K]; B int8 [N, K] (shared) or [batch, N, K]."""
-    _need(A.dtype == torch.int8 and B.dtype == torch.int8 and A.is_cuda and B.is_cuda, "A and B must be int8 GPU tensors")
+    _need(A.dtype == torch.int8 and B.dtype == torch.int8 and _on_gpu(A) and _on_gpu(B), "A and B must be int8 GPU tensors")
     _need(A.dim() == 3 and B.dim() in (2, 3), "A must be [batch, M, K]; B [N, K] or [batch, N, K]")
     batch, M, K = A.shape
     N = B.shape[-2]
@@ -274,7 +280,7 @@ def gemm_i8_nt(A, B, sA, modeA, sB, modeB, *, acc_i32_full=False, combine=COMBIN
 
 def gemm_i8_nt_i32(A, B):
     """Raw int32 accumulators of A[b] @ B[b]^T over the whole K."""
-    _need(A.dtype == torch.int8 and B.dtype == torch.int8 and A.is_cuda and B.is_cuda, "A and B must be int8 GPU tensors")
+    _need(A.dtype == torch.int8 and B.dtype == torch.int8 and _on_gpu(A) and _on_gpu(B), "A and B must be int8 GPU tensors")
     _need(A.dim() == 3 and B.dim() in (2, 3), "A must be [batch, M, K]; B [N, K] or [batch, N, K]")
     batch, M, K = A.shape
     N = B.shape[-2]
