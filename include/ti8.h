@@ -12,6 +12,12 @@
  *     Arguments are validated on the host before anything is launched.
  *   - bf16 tensors are passed as void* / uint16_t bit patterns.
  *
+ *   - Non-finite inputs of the quantisers, one rule for all of them: a NaN element is left out of
+ *     its group's absmax (as v_max_f32 and the reference's tl.max leave it out; a group of nothing
+ *     but NaN has absmax 0) and converts to -128; an infinite element is its group's absmax like any
+ *     other number, so the group's multiplier is 0, its finite elements convert to 0, the infinity
+ *     to -128 (inf * 0 = NaN) and the stored scale is infinite.  Nothing is rejected or reported.
+ *
  * The reference has no FFI: its boundary is a set of Python functions, each a host
  * wrapper around one Triton kernel.  Each entry point below names the reference
  * wrapper + kernel it replaces (paths relative to the reference checkout).
@@ -46,7 +52,14 @@ enum ti8_qflags {
     TI8_Q_HAD128 = 8,       /* ti8_quant_row only: rotate every 128-column group by H_128 (fp32
                                butterflies, one bf16 rounding) before the absmax */
     TI8_Q_WS_PINGPONG = 16, /* ti8_quant_row_col_t only: two-part workspace that the calls keep clear for each */
-    TI8_Q_WS_SECOND = 32    /* other, and which part this call works in (see there) */
+    TI8_Q_WS_SECOND = 32,   /* other, and which part this call works in (see there) */
+    TI8_Q_TORCH_ROUND = 64, /* ti8_quant_block (128 x 128 groups, q only) and ti8_quant_row (group = 0): the arithmetic of the
+                               reference's pure-torch quantisers instead of its Triton kernels' -- scale =
+                               reciprocal(max(amax, 1e-4)) * 127, q = clamp(round_half_even(x * scale), -127, 127), stored
+                               scale = reciprocal(scale) (per_block_cast_to_int8 of tilelang/block_channel_bwd.py:96-104) */
+    TI8_Q_TORCH_BF16 = 128  /* the same with every intermediate rounded to bf16, the product x * scale included: what torch
+                               computes when the input is bf16 and nothing widens it (per_token_cast_to_int8 /
+                               per_block_cast_to_int8 of tilelang/block_channel_fwd.py:215-230) */
 };
 
 /* which number is written to the scale tensor */

@@ -56,7 +56,12 @@ FAKE = 0x10000  # a 16-byte aligned non-null "device pointer"; validation never 
     (("ti8_quant_block", FAKE, 0, 128, FAKE, 0, 128, None, 0, 0, FAKE, 0, 1, 1, 1, 128, 128, 64, 0, 0, None), 4, "group_c"),
     (("ti8_quant_block", FAKE, 0, 128, FAKE, 0, 128, FAKE, 0, 128, FAKE, 0, 1, 1, 1, 128, 256, 256, 0, 0, None), 4, "transposed"),
     (("ti8_quant_block", FAKE + 2, 0, 128, FAKE, 0, 128, None, 0, 0, FAKE, 0, 1, 1, 1, 128, 128, 128, 0, 0, None), 3, "aligned"),
-    (("ti8_quant_block", FAKE, 0, 128, FAKE, 0, 128, None, 0, 0, FAKE, 0, 1, 1, 1, 128, 128, 128, 64, 0, None), 4, "flag"),
+    (("ti8_quant_block", FAKE, 0, 128, FAKE, 0, 128, None, 0, 0, FAKE, 0, 1, 1, 1, 128, 128, 128, 256, 0, None), 4, "flag"),
+    (("ti8_quant_block", FAKE, 0, 256, FAKE, 0, 256, None, 0, 0, FAKE, 0, 1, 1, 1, 128, 256, 256, 64, 0, None), 4, "torch arithmetic"),
+    (("ti8_quant_block", FAKE, 0, 128, FAKE, 0, 128, FAKE, 0, 128, FAKE, 0, 1, 1, 1, 128, 128, 128, 128, 0, None), 4, "torch arithmetic"),
+    (("ti8_quant_row", FAKE, 4096, FAKE, 4096, FAKE, 4, 4096, 128, 64, 0, None), 4, "torch arithmetic"),
+    (("ti8_quant_row", FAKE, 4096, FAKE, 4096, FAKE, 4, 4096, 0, 64, 1, None), 4, "torch arithmetic"),
+    (("ti8_quant_col_t", FAKE, 256, FAKE, 128, FAKE, FAKE, 128, 256, 64, 0, None), 4, "unknown quantiser flag"),
     (("ti8_quant_block", FAKE, 0, 128, FAKE, 0, 128, None, 0, 0, FAKE, 0, 1, 1, 1, 128, 128, 128, 8, 0, None), 4, "had128"),
     (("ti8_quant_block_had128", FAKE, 0, 128, FAKE, 0, 128, FAKE, 0, 1, 1, 1, 128, 100, 0, 1, 0, None), 2, "C%128"),
     (("ti8_quant_block_had128", FAKE, 0, 128, None, 0, 128, FAKE, 0, 1, 1, 1, 128, 128, 1, 1, 0, None), 1, "required"),

@@ -175,6 +175,43 @@ def test_row_and_col_quant_workspace_modes(T, dev):
         assert torch.equal(outs[0][0], q0) and bits_equal(outs[0][1], s0)
 
 
+def test_row_and_col_quant_workspace_cache_is_bounded(T, dev):
+    """The per-(stream, shape) two-part workspaces of ops.quant_row_col_t are a small LRU: shapes that
+    fall out and come back, and calls from several threads on one stream, still give the bits of the
+    separate quantisers."""
+    import threading
+    xs = [randn_bf16(make_gen(60 + i), 128, 128 * (i + 1)).to(dev) for i in range(T.ops._PINGPONG_SLOTS + 4)]
+    want = [(T.ops.quant_row(x), T.ops.quant_col_t(x)) for x in xs]
+
+    def check(x, w):
+        q, sr, qT, sc = T.ops.quant_row_col_t(x)
+        assert torch.equal(q, w[0][0]) and bits_equal(sr, w[0][1]) and torch.equal(qT, w[1][0]) and bits_equal(sc, w[1][1])
+
+    for _ in range(3):                       # every shape is evicted and re-created between its uses
+        for x, w in zip(xs, want):
+            check(x, w)
+    assert len(T.ops._PINGPONG_WS) <= T.ops._PINGPONG_SLOTS
+    errors = []
+
+    same_shape = [randn_bf16(make_gen(90 + i), 128, 512, std=10.0 ** i).to(dev) for i in range(4)]   # maxima orders of magnitude apart
+    same_want = [(T.ops.quant_row(x), T.ops.quant_col_t(x)) for x in same_shape]
+
+    def worker(i):
+        try:
+            for _ in range(20):
+                check(same_shape[i], same_want[i])
+        except Exception as e:               # noqa: BLE001 - reported below
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(4)]   # all on the default stream, one workspace
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors[0]
+
+
 @pytest.mark.parametrize("n,cols", [(128, 384), (128, 4096), (256, 256), (512, 1536), (1024, 2048), (2048, 2048),
                                     (4096, 4096), (8192, 8192), (16384, 16384), (32768, 32768)])
 def test_fwht(T, dev, n, cols):
@@ -445,6 +482,80 @@ def test_decoder_layer_step_matches_bf16_twin(T, dev):
     # 128x128 block, so most of it quantises to zero: int8 noise of the scheme, not of the kernels
     # (the same layers match the CPU oracle in test_linear_fwd_bwd)
     assert cos(outs[0][4], outs[1][4]) > 0.3
+
+
+def test_nan_and_inf_inputs(T, dev):
+    """One rule for every quantiser (include/ti8.h, "Non-finite inputs"): a NaN element is left out of
+    its group's absmax, as the reference's tl.max leaves it out, and converts to -128; an infinite
+    element is its group's absmax like any other number, which makes the multiplier 0 (codes 0, the
+    infinity itself -128 through inf * 0 = NaN) and the stored scale infinite."""
+    x = randn_bf16(make_gen(50), 256, 384)
+    clean = x.clone()
+    x[7, 9] = float("nan")
+    clean[7, 9] = 0
+    xd, cd = x.to(dev), clean.to(dev)
+
+    def same_but(q, q0, pos):
+        q0 = q0.clone()
+        q0[pos] = -128
+        return torch.equal(q, q0)
+
+    q, s = T.ops.quant_block(xd[None])
+    q0, s0 = T.ops.quant_block(cd[None])
+    assert same_but(q[0], q0[0], (7, 9)) and bits_equal(s, s0)
+    q, s = T.ops.quant_row(xd)
+    q0, s0 = T.ops.quant_row(cd)
+    assert same_but(q, q0, (7, 9)) and bits_equal(s, s0)
+    qT, s = T.ops.quant_col_t(xd)
+    qT0, s0 = T.ops.quant_col_t(cd)
+    assert same_but(qT, qT0, (9, 7)) and bits_equal(s, s0)
+    q, sr, qT, sc = T.ops.quant_row_col_t(xd)
+    q0, sr0, qT0, sc0 = T.ops.quant_row_col_t(cd)
+    assert same_but(q, q0, (7, 9)) and same_but(qT, qT0, (9, 7)) and bits_equal(sr, sr0) and bits_equal(sc, sc0)
+    q, s = T.ops.quant_block_had128(xd[None])          # the rotation spreads the NaN over its group of 128, and no further
+    assert bool((q[0, 7, :128] == -128).all()) and bool((q[0, 7, 128:] != -128).any()) and bool((q[0, 8] != -128).any())
+    # a row / column of nothing but NaN counts as all zero: the epsilon scale
+    y = clean.clone()
+    y[5] = float("nan")
+    q, sr, qT, sc = T.ops.quant_row_col_t(y.to(dev))
+    q0, sr0 = T.ops.quant_row(y.to(dev))
+    assert bits_equal(sr, sr0) and float(sr[5]) == float(sr0[5]) and torch.equal(q, q0) and bool((q[5] == -128).all())
+    # infinity
+    z = clean.clone()
+    z[3, 5] = float("inf")
+    zd = z.to(dev)
+    for q, s, row, col in ((*T.ops.quant_row(zd), 3, 5), (*T.ops.quant_col_t(zd), 5, 3)):
+        assert torch.isinf(s[row]) and int(q[row, col]) == -128 and int(q[row].int().abs().sum()) == 128
+    q, s = T.ops.quant_block(zd[None])
+    assert torch.isinf(s[0, 0, 0]) and int(q[0, 3, 5]) == -128 and int(q[0, :128, :128].int().abs().sum()) == 128
+    assert not torch.isinf(s[0, 1, 1])
+
+
+def test_torch_form_cast_quantisers(T, dev):
+    """per_token_cast_to_int8 / per_block_cast_to_int8 of both TileLang files (the reference author's
+    pure-torch quantisers: round half to even, clamp +-127, bf16 or fp32 intermediates) as HIP kernels,
+    bit for bit against torch's own evaluation of the reference expressions on the CPU."""
+    x = planted(30, 2, 256, 384)
+    x[1, 128:256, 256:384] = torch.tensor([0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 127.0, 3.0] * 16).to(torch.bfloat16)   # exact ties
+    xd = x.to(dev)
+    q, s = T.tilelang_block_channel_fwd.per_block_cast_to_int8(xd)
+    qo, so = otf.per_block_cast_to_int8(x)
+    assert s.dtype == torch.bfloat16 and bits_equal(q, qo) and bits_equal(s, so)
+    q, s = T.tilelang_block_channel_bwd.per_block_cast_to_int8(xd)
+    qo, so = otb.per_block_cast_to_int8(x)
+    assert s.dtype == torch.float32 and bits_equal(q, qo) and bits_equal(s, so)
+    for cols in (128, 1024, 6144, 14336):
+        xr = randn_bf16(make_gen(cols), 37, cols)
+        xr[3] = 0
+        xr[5, :8] = torch.tensor([0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 127.0, 3.0]).to(torch.bfloat16)
+        xr[5, 8:] = 0
+        q, s = T.tilelang_block_channel_fwd.per_token_cast_to_int8(xr.to(dev))
+        qo, so = otf.per_token_cast_to_int8(xr)
+        assert s.shape == (37, 1) and bits_equal(q, qo) and bits_equal(s, so)
+    # the reference's self-checks of the TileLang kernels, at the reference's shapes
+    assert T.tilelang_block_channel_fwd.assert_tl_gemm_correctness(4, 1024, 1024, 8192, 128, "int8", "bfloat16", "int32") < 1e-3
+    assert T.tilelang_block_channel_bwd.assert_tl_gemm_correctness(10, 1024, 1024, 8192, 128, "int8", "bfloat16", "int32") < 1e-3
+    assert T.tilelang_block_channel_bwd.ceildiv(129, 128) == 2
 
 
 @pytest.mark.parametrize("scheme", ["block_channel", "double_channel", "fused", "tilelang"])

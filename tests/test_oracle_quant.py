@@ -141,3 +141,48 @@ def test_reference_torch_quantisers_differ_only_on_ties():
     q_ref, _ = otf.per_token_cast_to_int8(x)
     q, _ = obf.triton_per_token_quant(x)
     assert int((q_ref.int() - q.int()).abs().max()) <= 1
+
+
+def _bf16_round(a):
+    """fp32 numpy array -> nearest bf16 (ties to even), as fp32."""
+    u = np.asarray(a, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    u = (u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000
+    return u.astype(np.uint32).view(np.float32)
+
+
+def test_torch_cast_quantisers_closed_form():
+    """The reference's pure-torch quantisers, pinned against a numpy evaluation with every rounding
+    written out: torch turns ``127.0 / amax`` into reciprocal(amax) * 127 (two roundings), rounds half
+    to even, and on a bf16 tensor rounds every intermediate (x * scale included) to bf16.  This is
+    the arithmetic the HIP kernels implement for TI8_Q_TORCH_ROUND / TI8_Q_TORCH_BF16."""
+    from oracle import tilelang_block_channel_bwd as otb
+    x = randn_bf16(make_gen(31), 2, 256, 384)
+    x[0, :128, :128] = 0                       # all-zero block: the 1e-4 floor
+    x[1, 130, 200] = 37.25
+    # planted exact ties of x * scale: the block maximum 127 makes scale exactly 1
+    x[1, 128:256, 256:384] = torch.tensor([0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 127.0, 3.0] * 16).to(torch.bfloat16)
+    xf = x.float().numpy()
+    blocks = xf.reshape(2, 2, 128, 3, 128)
+    amax = np.abs(blocks).max(axis=(2, 4), keepdims=True)
+    # fp32 variant (tilelang/block_channel_bwd.py:96-104)
+    a32 = np.maximum(amax, np.float32(1e-4))
+    scale = (np.float32(1.0) / a32) * np.float32(127.0)
+    q = np.clip(np.rint(blocks * scale), -127, 127).astype(np.int8).reshape(2, 256, 384)
+    s = (np.float32(1.0) / scale).reshape(2, 2, 3)
+    qo, so = otb.per_block_cast_to_int8(x)
+    assert so.dtype == torch.float32 and np.array_equal(qo.numpy(), q) and np.array_equal(so.numpy().view(np.uint32), s.view(np.uint32))
+    assert qo[1, 128, 256:264].tolist() == [0, 2, 2, 0, -2, -2, 127, 3]       # half to even (the kernels' floor(x + 0.5): 1, 2, 3, 0, -1, -2)
+    # bf16 variant (tilelang/block_channel_fwd.py:222-230)
+    ab = np.maximum(amax, _bf16_round(np.float32(1e-4)))
+    scale = _bf16_round(_bf16_round(np.float32(1.0) / ab) * np.float32(127.0))
+    q = np.clip(np.rint(_bf16_round(blocks * scale)), -127, 127).astype(np.int8).reshape(2, 256, 384)
+    s = _bf16_round(np.float32(1.0) / scale).reshape(2, 2, 3)
+    qo, so = otf.per_block_cast_to_int8(x)
+    assert so.dtype == torch.bfloat16 and np.array_equal(qo.numpy(), q) and np.array_equal(so.float().numpy(), s)
+    # per row, bf16 (tilelang/block_channel_fwd.py:215-220)
+    rows = xf[1]
+    ab = np.maximum(np.abs(rows).max(axis=1, keepdims=True), _bf16_round(np.float32(1e-4)))
+    scale = _bf16_round(_bf16_round(np.float32(1.0) / ab) * np.float32(127.0))
+    q = np.clip(np.rint(_bf16_round(rows * scale)), -127, 127).astype(np.int8)
+    qo, so = otf.per_token_cast_to_int8(x[1])
+    assert np.array_equal(qo.numpy(), q) and np.array_equal(so.float().numpy(), _bf16_round(np.float32(1.0) / scale))

@@ -35,3 +35,17 @@ class StageTimer:
         if self.verbose:
             torch.cuda.synchronize(self.device)
             print(f"{label}:{(time.time() - self.t0) * 1000} ms")
+
+
+def bf16_reference_nt(a, b):
+    """bf16 ``a @ b^T`` over the last two dims, the product the reference's self-checks compare with
+    (``torch.matmul(a, b.T)`` / ``torch.bmm(a, b.transpose(1, 2))``).  With a 3-D ``b`` it is
+    evaluated batch by batch as 2-D products rather than as one batched call."""
+    if b.dim() == 2:
+        return torch.matmul(a, b.t())
+    return torch.stack([torch.matmul(a[i], b[i].t()) for i in range(a.shape[0])])
+
+
+def ceildiv(a, b):
+    """tilelang/block_channel_bwd.py:91-92."""
+    return (a + b - 1) // b

@@ -30,7 +30,7 @@ PROTOTYPES = {
 EXPORTS = ["ti8_version", "ti8_last_error", "ti8_arch"] + list(PROTOTYPES)
 
 # enums of include/ti8.h
-Q_CLAMP, Q_EPS_ADD, Q_SCALE_BF16, Q_HAD128, Q_WS_PINGPONG, Q_WS_SECOND = 1, 2, 4, 8, 16, 32
+Q_CLAMP, Q_EPS_ADD, Q_SCALE_BF16, Q_HAD128, Q_WS_PINGPONG, Q_WS_SECOND, Q_TORCH_ROUND, Q_TORCH_BF16 = 1, 2, 4, 8, 16, 32, 64, 128
 INV_RCP_OF_SCALE, INV_AMAX_DIV_127, INV_AMAX_MUL_RCP127, INV_MULTIPLIER = 0, 1, 2, 3
 SCALE_ROW, SCALE_BLOCK128, SCALE_ROW_K128, SCALE_BLOCK_K256 = 0, 1, 2, 3
 COMBINE_MUL_MUL, COMBINE_MUL_PROD, COMBINE_DIV_PROD = 0, 1, 2

@@ -18,6 +18,33 @@ struct QMode {
     int inv_mode;    // ti8_inv_mode
 };
 
+// Arithmetic of the conversion.  ARITH_KERNEL is that of the reference's Triton kernels.  The
+// other two are those of its pure-torch quantisers per_token_cast_to_int8 / per_block_cast_to_int8
+// (tilelang/block_channel_fwd.py:215-230, tilelang/block_channel_bwd.py:96-104), evaluated the way
+// torch evaluates them: `127.0 / amax` is reciprocal(amax) * 127 (two roundings), round() is
+// half-to-even, the clamp is [-127, 127], the returned scale is reciprocal(scale); in the bf16
+// variant (bf16 input, no .float() anywhere) every intermediate is rounded to bf16, the product
+// x * scale included.
+enum { ARITH_KERNEL = 0, ARITH_TORCH_F32 = 1, ARITH_TORCH_BF16 = 2 };
+
+__device__ __forceinline__ float round_bf16(float f) { return __uint_as_float(f32_to_bf16_bits(f) << 16); }
+
+template <int ARITH>
+__device__ __forceinline__ float group_multiplier(float amax) {   // amax already floored
+    if (ARITH == ARITH_KERNEL) return 127.0f / amax;
+    float r = 1.0f / amax;
+    if (ARITH == ARITH_TORCH_BF16) r = round_bf16(r);
+    r = r * 127.0f;
+    return ARITH == ARITH_TORCH_BF16 ? round_bf16(r) : r;
+}
+template <int ARITH>
+__device__ __forceinline__ float amax_floor_arith(float amax, int eps_add) {
+    if (ARITH == ARITH_KERNEL) return eps_add ? (amax + 1e-5f) : (amax > 1e-4f ? amax : 1e-4f);
+    // torch clamp(min=1e-4) compares in the tensor's dtype: the constant is rounded to bf16 there
+    const float e = ARITH == ARITH_TORCH_BF16 ? round_bf16(1e-4f) : 1e-4f;
+    return amax > e ? amax : e;
+}
+
 __device__ __forceinline__ float amax_floor(float amax, int eps_add) {
     // triton/block_channel_fwd32.py:182 `where(amax > 1e-4, amax, 1e-4)`;
     // triton/fused_triton_fwd32.py:49 `max|x| + 1e-5`
@@ -35,6 +62,12 @@ __device__ __forceinline__ float stored_scale(float amax, float scale, const QMo
     if (m.scale_bf16) s = __uint_as_float(f32_to_bf16_bits(s) << 16);
     return s;
 }
+template <int ARITH>
+__device__ __forceinline__ float stored_scale_arith(float amax, float scale, const QMode& m) {
+    if (ARITH == ARITH_KERNEL) return stored_scale(amax, scale, m);
+    const float s = 1.0f / scale;   // torch: (1.0 / scale) = reciprocal(scale) * 1.0
+    return ARITH == ARITH_TORCH_BF16 ? round_bf16(s) : s;
+}
 
 // Rounding and int8 conversion.  r = floor(x*scale + 0.5) with two roundings (contraction is
 // off), then r + 128 (exact: r is integral) goes through the saturating float -> u8 conversion
@@ -42,21 +75,30 @@ __device__ __forceinline__ float stored_scale(float amax, float scale, const QMo
 // turns the biased byte into two's complement.  The saturation IS the [-128, 127] clamp; without
 // TI8_Q_CLAMP the reference applies no clamp, which gives the same bytes for every finite input
 // because |x*scale| <= 127 when scale = 127 / absmax of the same data.
-__device__ __forceinline__ float qbiased(float x, float scale) { return floorf(x * scale + 0.5f) + 128.0f; }
+template <int ARITH = ARITH_KERNEL>
+__device__ __forceinline__ float qbiased(float x, float scale) {
+    if (ARITH == ARITH_KERNEL) return floorf(x * scale + 0.5f) + 128.0f;
+    float t = x * scale;
+    if (ARITH == ARITH_TORCH_BF16) t = round_bf16(t);
+    t = rintf(t);                                       // half to even
+    t = fminf(fmaxf(t, -127.0f), 127.0f);
+    return t + 128.0f;
+}
 __device__ __forceinline__ uint32_t put_u8(float t, uint32_t byte, uint32_t old) {
     return __builtin_amdgcn_cvt_pk_u8_f32(t, byte, old);
 }
 constexpr uint32_t UNBIAS4 = 0x80808080u;
 
 // 8 bf16 (one 16-byte load) -> 8 int8 in two dwords, element 0 in the low byte
+template <int ARITH = ARITH_KERNEL>
 __device__ __forceinline__ uint2 quant8(const uint4& v, float scale) {
-    uint32_t a = put_u8(qbiased(bf16_lo(v.x), scale), 0, 0u), b = put_u8(qbiased(bf16_lo(v.z), scale), 0, 0u);
-    a = put_u8(qbiased(bf16_hi(v.x), scale), 1, a);
-    b = put_u8(qbiased(bf16_hi(v.z), scale), 1, b);
-    a = put_u8(qbiased(bf16_lo(v.y), scale), 2, a);
-    b = put_u8(qbiased(bf16_lo(v.w), scale), 2, b);
-    a = put_u8(qbiased(bf16_hi(v.y), scale), 3, a);
-    b = put_u8(qbiased(bf16_hi(v.w), scale), 3, b);
+    uint32_t a = put_u8(qbiased<ARITH>(bf16_lo(v.x), scale), 0, 0u), b = put_u8(qbiased<ARITH>(bf16_lo(v.z), scale), 0, 0u);
+    a = put_u8(qbiased<ARITH>(bf16_hi(v.x), scale), 1, a);
+    b = put_u8(qbiased<ARITH>(bf16_hi(v.z), scale), 1, b);
+    a = put_u8(qbiased<ARITH>(bf16_lo(v.y), scale), 2, a);
+    b = put_u8(qbiased<ARITH>(bf16_lo(v.w), scale), 2, b);
+    a = put_u8(qbiased<ARITH>(bf16_hi(v.y), scale), 3, a);
+    b = put_u8(qbiased<ARITH>(bf16_hi(v.w), scale), 3, b);
     uint2 o;
     o.x = a ^ UNBIAS4;
     o.y = b ^ UNBIAS4;
@@ -163,7 +205,7 @@ __device__ __forceinline__ void transpose4x4_bytes(uint32_t r0, uint32_t r1, uin
 // a wave load instruction covers whole 256-byte row segments, and the 4-row patches
 // transpose in registers for the optional transposed output (staged through LDS so
 // that the global writes of qT are 128-byte rows too).
-template <int NSUB, bool WRITE_Q, bool WRITE_QT>
+template <int NSUB, bool WRITE_Q, bool WRITE_QT, int ARITH = ARITH_KERNEL>
 __global__ __launch_bounds__(256) void quant_block_kernel(
     const uint16_t* __restrict__ x, int64_t bsx, int64_t ldx, int8_t* __restrict__ q, int64_t bsq, int64_t ldq,
     int8_t* __restrict__ qT, int64_t bsqt, int64_t ldqt, float* __restrict__ s, int64_t ssb, int64_t ssr,
@@ -198,9 +240,9 @@ __global__ __launch_bounds__(256) void quant_block_kernel(
 #pragma unroll
             for (int j = 0; j < 4; ++j) amax = absmax8(v[u][h][j], amax);
     amax = block_max_256(amax, red4);
-    amax = amax_floor(amax, mode.eps_add);
-    const float scale = 127.0f / amax;
-    if (tid == 0) s[b * ssb + rb * ssr + cb * ssc] = stored_scale(amax, scale, mode);
+    amax = amax_floor_arith<ARITH>(amax, mode.eps_add);
+    const float scale = group_multiplier<ARITH>(amax);
+    if (tid == 0) s[b * ssb + rb * ssr + cb * ssc] = stored_scale_arith<ARITH>(amax, scale, mode);
 
 #pragma unroll
     for (int u = 0; u < NSUB; ++u) {
@@ -208,7 +250,7 @@ __global__ __launch_bounds__(256) void quant_block_kernel(
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) o[h][j] = quant8(v[u][h][j], scale);
+            for (int j = 0; j < 4; ++j) o[h][j] = quant8<ARITH>(v[u][h][j], scale);
 
         if (WRITE_Q) {
             int8_t* qt = q + idx::qblock_origin(b, bsq, rb, ldq, cb, 128 * NSUB) + u * 128 + idx::qblock_col(tid);
@@ -362,7 +404,7 @@ __global__ __launch_bounds__(256) void quant_block_had_kernel(
 // workgroup); WG_ROW = true: one 256-thread workgroup per row.  Each thread keeps
 // NLOAD 16-byte chunks of its row in registers.  GROUP16: one scale per 16 chunks
 // (128 columns) instead of per row.
-template <int NLOAD, bool WG_ROW, bool GROUP16, bool HAD>
+template <int NLOAD, bool WG_ROW, bool GROUP16, bool HAD, int ARITH = ARITH_KERNEL>
 __global__ __launch_bounds__(256) void quant_row_kernel(const uint16_t* __restrict__ x, int64_t ldx,
                                                         int8_t* __restrict__ q, int64_t ldq,
                                                         float* __restrict__ s, int64_t rows, int cols,
@@ -405,13 +447,13 @@ __global__ __launch_bounds__(256) void quant_row_kernel(const uint16_t* __restri
         amax = block_max_256(amax, red4);
     else
         amax = wave_max(amax);
-    amax = amax_floor(amax, mode.eps_add);
-    const float scale = 127.0f / amax;
-    if (t == 0) s[row] = stored_scale(amax, scale, mode);
+    amax = amax_floor_arith<ARITH>(amax, mode.eps_add);
+    const float scale = group_multiplier<ARITH>(amax);
+    if (t == 0) s[row] = stored_scale_arith<ARITH>(amax, scale, mode);
 #pragma unroll
     for (int i = 0; i < NLOAD; ++i) {
         const int c = idx::qrow_chunk(t, i, T);
-        if (c < nchunk) *reinterpret_cast<uint2*>(qr + c * 8) = quant8(v[i], scale);
+        if (c < nchunk) *reinterpret_cast<uint2*>(qr + c * 8) = quant8<ARITH>(v[i], scale);
     }
 }
 
@@ -483,22 +525,36 @@ __global__ __launch_bounds__(256) void quant_col_t_kernel(const uint16_t* __rest
 // an operand that a training step needs, by rows for one GEMM, by columns -- transposed -- for
 // another).  Workgroup = TR rows x 256 columns; thread t reads the 16-byte chunk t%32 of rows
 // t/32 + 8i.  |x| of a bf16 is its bit pattern without the sign, and non-negative bf16 order
-// like their 16-bit patterns, so the maxima are taken on packed pairs of u16 (v_pk_max_u16: no
+// like their 16-bit patterns, so the maxima are taken on packed pairs of 16-bit integers (no
 // unpacking, two elements per instruction) and widened to fp32 bit patterns (<< 16) at the end,
-// where they are merged into ws[] with an unsigned atomic max.  Row maxima meet over the 32
+// where they are merged into ws[] with an unsigned atomic max.
+// NaN elements are left out of the maxima, as the float maxima of the other quantisers (v_max_f32)
+// and the reference's tl.max leave them out: the patterns are biased by 0x7f, which moves the NaN
+// patterns 0x7f81 .. 0x7fff -- and only those -- to 0x8000 and above, and compared as SIGNED
+// 16-bit values (v_pk_max_i16), where those are negative and lose against every number, infinity
+// included; a group of nothing but NaN ends below the biased zero and counts as zero.
+// Row maxima meet over the 32
 // lanes of a half-wave through DPP moves; column maxima over the two half-waves by a lane swap
 // and over the four waves through LDS.  Short tiles win although they issue more atomics: 32
 // rows measured 6 % faster than 128 on 4096 x 4096 and on 8192 x 4096 (more workgroups per CU,
 // so the loads of one overlap the reductions of another); 16 and 64 rows are 1-2 % slower than 32.
 constexpr int ABSMAX_ROWS = 32;
+constexpr uint32_t ABS_BIAS2 = 0x007f007fu;   // the bias of both halves = the biased zero
 
-typedef unsigned short ti8_u16x2 __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
-    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(ti8_u16x2, a), __builtin_bit_cast(ti8_u16x2, b)));
+typedef short ti8_i16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pk_max_i16(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(ti8_i16x2, a), __builtin_bit_cast(ti8_i16x2, b)));
+}
+// |x| patterns of two bf16, biased
+__device__ __forceinline__ uint32_t abs_biased2(uint32_t w) { return (w & 0x7fff7fffu) + ABS_BIAS2; }
+// biased maxima of both halves -> the larger |x| pattern (0 if everything was NaN)
+__device__ __forceinline__ uint32_t unbias_max2(uint32_t m) {
+    const int lo = static_cast<short>(m & 0xffffu), hi = static_cast<short>(m >> 16);
+    return static_cast<uint32_t>(max(max(lo, hi), 0x7f) - 0x7f);
 }
 template <int CTRL, int ROW_MASK = 0xf>
-__device__ __forceinline__ uint32_t dpp_pk_max_u16(uint32_t v) {
-    return pk_max_u16(v, (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, CTRL, ROW_MASK, 0xf, false));
+__device__ __forceinline__ uint32_t dpp_pk_max_i16(uint32_t v) {
+    return pk_max_i16(v, (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, CTRL, ROW_MASK, 0xf, false));
 }
 
 template <int TR, bool WITH_ROWS>  // TR: rows of x per workgroup (8, 16, ... 128)
@@ -506,16 +562,16 @@ __global__ __launch_bounds__(256) void absmax_kernel(const uint16_t* __restrict_
                                                      unsigned int* __restrict__ ws_row,
                                                      unsigned int* __restrict__ ws_col, int64_t R, int C) {
     constexpr int NR = TR / 8;
-    __shared__ uint4 part[4][32];  // [wave][chunk]: 8 column maxima (u16) per chunk
+    __shared__ uint4 part[4][32];  // [wave][chunk]: 8 biased column maxima per chunk
     __shared__ uint32_t rowpart[WITH_ROWS ? TR : 1];  // row maxima of the tile (fp32 bit patterns)
     const int tid = threadIdx.x;
     const int cc = tid & 31, rg = tid >> 5;
     const int c0 = blockIdx.x * 256 + cc * 8;
     const int64_t r0 = (int64_t)blockIdx.y * TR;
-    uint32_t m[4] = {0, 0, 0, 0};  // columns c0 + 2k (low half) and c0 + 2k + 1 (high half)
+    uint32_t m[4] = {ABS_BIAS2, ABS_BIAS2, ABS_BIAS2, ABS_BIAS2};  // columns c0 + 2k (low half) and c0 + 2k + 1 (high half)
     uint32_t rmax[NR];
 #pragma unroll
-    for (int i = 0; i < NR; ++i) rmax[i] = 0;
+    for (int i = 0; i < NR; ++i) rmax[i] = ABS_BIAS2;
     if (c0 < C) {
         uint4 v[NR];
 #pragma unroll
@@ -523,13 +579,12 @@ __global__ __launch_bounds__(256) void absmax_kernel(const uint16_t* __restrict_
             v[i] = *reinterpret_cast<const uint4*>(x + (r0 + rg + 8 * i) * ldx + c0);
 #pragma unroll
         for (int i = 0; i < NR; ++i) {
-            const uint32_t a0 = v[i].x & 0x7fff7fffu, a1 = v[i].y & 0x7fff7fffu, a2 = v[i].z & 0x7fff7fffu,
-                           a3 = v[i].w & 0x7fff7fffu;
-            m[0] = pk_max_u16(m[0], a0);
-            m[1] = pk_max_u16(m[1], a1);
-            m[2] = pk_max_u16(m[2], a2);
-            m[3] = pk_max_u16(m[3], a3);
-            if (WITH_ROWS) rmax[i] = pk_max_u16(pk_max_u16(a0, a1), pk_max_u16(a2, a3));
+            const uint32_t a0 = abs_biased2(v[i].x), a1 = abs_biased2(v[i].y), a2 = abs_biased2(v[i].z), a3 = abs_biased2(v[i].w);
+            m[0] = pk_max_i16(m[0], a0);
+            m[1] = pk_max_i16(m[1], a1);
+            m[2] = pk_max_i16(m[2], a2);
+            m[3] = pk_max_i16(m[3], a3);
+            if (WITH_ROWS) rmax[i] = pk_max_i16(pk_max_i16(a0, a1), pk_max_i16(a2, a3));
         }
     }
     if (WITH_ROWS) {
@@ -537,24 +592,24 @@ __global__ __launch_bounds__(256) void absmax_kernel(const uint16_t* __restrict_
         // row_half_mirror, row_mirror, row_bcast:15 into rows 1 and 3 -> valid in lanes 16-31, 48-63
         // (one step for all rows at a time: the chains are independent and interleave)
 #pragma unroll
-        for (int i = 0; i < NR; ++i) rmax[i] = dpp_pk_max_u16<0xB1>(rmax[i]);
+        for (int i = 0; i < NR; ++i) rmax[i] = dpp_pk_max_i16<0xB1>(rmax[i]);
 #pragma unroll
-        for (int i = 0; i < NR; ++i) rmax[i] = dpp_pk_max_u16<0x4E>(rmax[i]);
+        for (int i = 0; i < NR; ++i) rmax[i] = dpp_pk_max_i16<0x4E>(rmax[i]);
 #pragma unroll
-        for (int i = 0; i < NR; ++i) rmax[i] = dpp_pk_max_u16<0x141>(rmax[i]);
+        for (int i = 0; i < NR; ++i) rmax[i] = dpp_pk_max_i16<0x141>(rmax[i]);
 #pragma unroll
-        for (int i = 0; i < NR; ++i) rmax[i] = dpp_pk_max_u16<0x140>(rmax[i]);
+        for (int i = 0; i < NR; ++i) rmax[i] = dpp_pk_max_i16<0x140>(rmax[i]);
 #pragma unroll
         for (int i = 0; i < NR; ++i) {
-            const uint32_t a = dpp_pk_max_u16<0x142, 0xA>(rmax[i]);
-            if (cc == 16 + i) rowpart[rg + 8 * i] = max(a & 0xffffu, a >> 16) << 16;
+            const uint32_t a = dpp_pk_max_i16<0x142, 0xA>(rmax[i]);
+            if (cc == 16 + i) rowpart[rg + 8 * i] = unbias_max2(a) << 16;
         }
     }
 #if defined(__HIP_DEVICE_COMPILE__)
 #pragma unroll
     for (int k = 0; k < 4; ++k) {  // lanes l and l ^ 32 hold the same columns
         const auto r = __builtin_amdgcn_permlane32_swap(m[k], m[k], false, false);
-        m[k] = pk_max_u16(r[0], r[1]);
+        m[k] = pk_max_i16(r[0], r[1]);
     }
 #endif
     if ((tid & 32) == 0) part[tid >> 6][cc] = make_uint4(m[0], m[1], m[2], m[3]);
@@ -563,9 +618,10 @@ __global__ __launch_bounds__(256) void absmax_kernel(const uint16_t* __restrict_
     // (an instruction per row and half-wave, two lanes each, measured 2.5 us slower on 8192 x 4096)
     if (WITH_ROWS && tid < TR) atomicMax(ws_row + r0 + tid, rowpart[tid]);
     const uint32_t* pw = reinterpret_cast<const uint32_t*>(part);  // dword j of a wave's row: columns 2j, 2j + 1
-    const uint32_t u = pk_max_u16(pk_max_u16(pw[tid >> 1], pw[128 + (tid >> 1)]),
-                                  pk_max_u16(pw[256 + (tid >> 1)], pw[384 + (tid >> 1)]));
-    const uint32_t a = (tid & 1) ? (u >> 16) : (u & 0xffffu);
+    const uint32_t u = pk_max_i16(pk_max_i16(pw[tid >> 1], pw[128 + (tid >> 1)]),
+                                  pk_max_i16(pw[256 + (tid >> 1)], pw[384 + (tid >> 1)]));
+    const int b = static_cast<short>((tid & 1) ? (u >> 16) : (u & 0xffffu));   // biased, signed
+    const uint32_t a = static_cast<uint32_t>(max(b, 0x7f) - 0x7f);
     const int c = blockIdx.x * 256 + tid;
     if (c < C) atomicMax(ws_col + c, a << 16);
 }
@@ -641,6 +697,11 @@ __global__ __launch_bounds__(256) void quant_rowcol_kernel(const uint16_t* __res
     }
 }
 
+// arithmetic variant a flag set asks for (only ti8_quant_block and ti8_quant_row take the flags)
+static int arith_of(int qflags) {
+    return (qflags & TI8_Q_TORCH_BF16) ? ARITH_TORCH_BF16 : ((qflags & TI8_Q_TORCH_ROUND) ? ARITH_TORCH_F32 : ARITH_KERNEL);
+}
+
 static int parse_mode(int qflags, int inv_mode, QMode* m) {
     if (qflags & ~(TI8_Q_CLAMP | TI8_Q_EPS_ADD | TI8_Q_SCALE_BF16 | TI8_Q_HAD128)) return fail(TI8_ERR_MODE, "unknown quantiser flag 0x%x", qflags);
     if (inv_mode < 0 || inv_mode > 3) return fail(TI8_ERR_MODE, "unknown inv_mode %d", inv_mode);
@@ -660,7 +721,11 @@ extern "C" int ti8_quant_block(const void* x, int64_t bsx, int64_t ldx, int8_t* 
                                int64_t ssc, int64_t B, int64_t R, int64_t C, int group_c, int qflags,
                                int inv_mode, ti8_stream_t stream) {
     QMode mode;
+    const int arith = arith_of(qflags);
+    qflags &= ~(TI8_Q_TORCH_ROUND | TI8_Q_TORCH_BF16);
     if (int e = parse_mode(qflags, inv_mode, &mode)) return e;
+    if (arith != ARITH_KERNEL && (group_c != 128 || qT || (qflags & (TI8_Q_EPS_ADD | TI8_Q_SCALE_BF16)) || inv_mode != TI8_INV_RCP_OF_SCALE))
+        return fail(TI8_ERR_MODE, "ti8_quant_block: the torch arithmetic goes with group_c = 128, q only, no other flag and TI8_INV_RCP_OF_SCALE");
     if (qflags & TI8_Q_HAD128) return fail(TI8_ERR_MODE, "ti8_quant_block: use ti8_quant_block_had128 for the Hadamard rotation");
     if (!x || !s || (!q && !qT)) return fail(TI8_ERR_NULL, "ti8_quant_block: x, s and one of q/qT are required");
     if (group_c != 128 && group_c != 256) return fail(TI8_ERR_MODE, "ti8_quant_block: group_c must be 128 or 256, got %d", group_c);
@@ -681,7 +746,11 @@ extern "C" int ti8_quant_block(const void* x, int64_t bsx, int64_t ldx, int8_t* 
 #define TI8_LAUNCH_QB(NSUB, WQ, WQT)                                                                          \
     hipLaunchKernelGGL((quant_block_kernel<NSUB, WQ, WQT>), grid, block, 0, st, xp, bsx, ldx, q, bsq, ldq, qT, \
                        bsqt, ldqt, s, ssb, ssr, ssc, nrb, ncb, mode)
-    if (group_c == 256) TI8_LAUNCH_QB(2, true, false);
+    if (arith == ARITH_TORCH_F32)
+        hipLaunchKernelGGL((quant_block_kernel<1, true, false, ARITH_TORCH_F32>), grid, block, 0, st, xp, bsx, ldx, q, bsq, ldq, qT, bsqt, ldqt, s, ssb, ssr, ssc, nrb, ncb, mode);
+    else if (arith == ARITH_TORCH_BF16)
+        hipLaunchKernelGGL((quant_block_kernel<1, true, false, ARITH_TORCH_BF16>), grid, block, 0, st, xp, bsx, ldx, q, bsq, ldq, qT, bsqt, ldqt, s, ssb, ssr, ssc, nrb, ncb, mode);
+    else if (group_c == 256) TI8_LAUNCH_QB(2, true, false);
     else if (q && qT) TI8_LAUNCH_QB(1, true, true);
     else if (q) TI8_LAUNCH_QB(1, true, false);
     else TI8_LAUNCH_QB(1, false, true);
@@ -692,7 +761,11 @@ extern "C" int ti8_quant_block(const void* x, int64_t bsx, int64_t ldx, int8_t* 
 extern "C" int ti8_quant_row(const void* x, int64_t ldx, int8_t* q, int64_t ldq, float* s, int64_t rows,
                              int64_t cols, int group, int qflags, int inv_mode, ti8_stream_t stream) {
     QMode mode;
+    const int arith = arith_of(qflags);
+    qflags &= ~(TI8_Q_TORCH_ROUND | TI8_Q_TORCH_BF16);
     if (int e = parse_mode(qflags, inv_mode, &mode)) return e;
+    if (arith != ARITH_KERNEL && (group != 0 || (qflags & (TI8_Q_EPS_ADD | TI8_Q_SCALE_BF16 | TI8_Q_HAD128)) || inv_mode != TI8_INV_RCP_OF_SCALE))
+        return fail(TI8_ERR_MODE, "ti8_quant_row: the torch arithmetic goes with group = 0, no other flag and TI8_INV_RCP_OF_SCALE");
     if (!x || !q || !s) return fail(TI8_ERR_NULL, "ti8_quant_row: x, q and s are required");
     if (group != 0 && group != 128) return fail(TI8_ERR_MODE, "ti8_quant_row: group must be 0 or 128, got %d", group);
     if (rows <= 0 || cols <= 0 || cols % 128 || cols > 32768 || rows > 0x7fffffffLL)
@@ -707,7 +780,9 @@ extern "C" int ti8_quant_row(const void* x, int64_t ldx, int8_t* q, int64_t ldq,
     const int c = (int)cols;
     const bool had = (qflags & TI8_Q_HAD128) != 0;
 #define TI8_LAUNCH_QR(NL, WG, G16, GRID) \
-    do { if (had) hipLaunchKernelGGL((quant_row_kernel<NL, WG, G16, true>), dim3((unsigned)(GRID)), dim3(256), 0, st, xp, ldx, q, ldq, s, rows, c, mode); \
+    do { if (!G16 && arith == ARITH_TORCH_F32) hipLaunchKernelGGL((quant_row_kernel<NL, WG, false, false, ARITH_TORCH_F32>), dim3((unsigned)(GRID)), dim3(256), 0, st, xp, ldx, q, ldq, s, rows, c, mode); \
+         else if (!G16 && arith == ARITH_TORCH_BF16) hipLaunchKernelGGL((quant_row_kernel<NL, WG, false, false, ARITH_TORCH_BF16>), dim3((unsigned)(GRID)), dim3(256), 0, st, xp, ldx, q, ldq, s, rows, c, mode); \
+         else if (had) hipLaunchKernelGGL((quant_row_kernel<NL, WG, G16, true>), dim3((unsigned)(GRID)), dim3(256), 0, st, xp, ldx, q, ldq, s, rows, c, mode); \
          else hipLaunchKernelGGL((quant_row_kernel<NL, WG, G16, false>), dim3((unsigned)(GRID)), dim3(256), 0, st, xp, ldx, q, ldq, s, rows, c, mode); } while (0)
     const idx::QRowConfig cfg = idx::qrow_config(nchunk, group == 128);
     const int64_t grid = cfg.wg_row ? rows : (rows + 3) / 4;

@@ -5,11 +5,15 @@ current torch stream and never synchronises.  Arguments the kernels cannot take
 (wrong dtype/device, sizes that are not multiples of the tile) raise ``ValueError``
 here, before anything is launched.
 """
+import collections
+import threading
+
 import torch
 
 from . import _lib
 from ._lib import (COMBINE_DIV_PROD, COMBINE_MUL_MUL, COMBINE_MUL_PROD, GEMM_LARGE_TILES, GEMM_SKINNY, GEMM_STRICT, GEMM_TILED, INV_AMAX_DIV_127,
-                   INV_AMAX_MUL_RCP127, INV_MULTIPLIER, INV_RCP_OF_SCALE, Q_CLAMP, Q_EPS_ADD, Q_HAD128, Q_SCALE_BF16, Q_WS_PINGPONG, Q_WS_SECOND,
+                   INV_AMAX_MUL_RCP127, INV_MULTIPLIER, INV_RCP_OF_SCALE, Q_CLAMP, Q_EPS_ADD, Q_HAD128, Q_SCALE_BF16, Q_TORCH_BF16, Q_TORCH_ROUND,
+                   Q_WS_PINGPONG, Q_WS_SECOND,
                    SCALE_BLOCK128, SCALE_BLOCK_K256, SCALE_ROW, SCALE_ROW_K128)
 
 __all__ = ["quant_block", "quant_block_had128", "quant_row", "quant_col_t", "quant_row_col_t", "fwht", "gemm_i8_nt", "gemm_i8_nt_i32"]
@@ -42,12 +46,14 @@ def _check_bf16(x, name):
     _need(x.dtype == torch.bfloat16, f"{name} must be bfloat16, got {x.dtype}")
 
 
-def _qflags(clamp, eps_add, scale_bf16):
-    return (Q_CLAMP if clamp else 0) | (Q_EPS_ADD if eps_add else 0) | (Q_SCALE_BF16 if scale_bf16 else 0)
+def _qflags(clamp, eps_add, scale_bf16, torch_arith=None):
+    _need(torch_arith in (None, "f32", "bf16"), "torch_arith must be None, 'f32' or 'bf16'")
+    return ((Q_CLAMP if clamp else 0) | (Q_EPS_ADD if eps_add else 0) | (Q_SCALE_BF16 if scale_bf16 else 0) |
+            {None: 0, "f32": Q_TORCH_ROUND, "bf16": Q_TORCH_ROUND | Q_TORCH_BF16}[torch_arith])
 
 
 def quant_block(x, *, clamp=True, group_c=128, eps_add=False, scale_bf16=False, inv_mode=INV_RCP_OF_SCALE,
-                out="like", with_transpose=False):
+                out="like", with_transpose=False, torch_arith=None):
     """Per-128 x group_c-block absmax quantisation of ``x`` [B, M, N] (bf16).
 
     ``x`` may be row-major (last stride 1) or a transposed view of a row-major
@@ -56,6 +62,9 @@ def quant_block(x, *, clamp=True, group_c=128, eps_add=False, scale_bf16=False, 
       "contiguous"  q is contiguous in the logical [B, M, N] orientation
     ``with_transpose`` additionally returns ``qT`` = contiguous [B, N, M] int8 holding
     ``q`` transposed, written by the same kernel from the same registers.
+    ``torch_arith`` "f32" / "bf16": the arithmetic of the reference's pure-torch quantisers (reciprocal
+    times 127, round half to even, clamp +-127; "bf16" rounds every intermediate to bf16) instead of
+    its kernels'; row-major ``x``, ``q`` only.
     Returns ``(q, s)`` or ``(q, qT, s)``; ``s`` is fp32 [B, M/128, N/group_c]."""
     _check_bf16(x, "x")
     _need(x.dim() == 3, "x must be [B, M, N]")
@@ -72,6 +81,7 @@ def quant_block(x, *, clamp=True, group_c=128, eps_add=False, scale_bf16=False, 
     _need(group_c in (128, 256), "group_c must be 128 or 256")
     _need(out in ("like", "contiguous"), "out must be 'like' or 'contiguous'")
     _need(not (transposed or with_transpose) or group_c == 128, "transposed layouts need 128 x 128 blocks")
+    _need(torch_arith is None or not (transposed or with_transpose), "torch_arith needs a row-major x and no transposed output")
     _need(M % 128 == 0 and N % (group_c if not transposed else 128) == 0,
           f"block quantisation needs M % 128 == 0 and N % {group_c} == 0, got M={M} N={N}")
     R, C = xc.shape[1], xc.shape[2]          # canonical (row-major) view of the memory
@@ -93,7 +103,7 @@ def quant_block(x, *, clamp=True, group_c=128, eps_add=False, scale_bf16=False, 
               qc.data_ptr() if qc is not None else None, R * C, C,
               qct.data_ptr() if qct is not None else None, R * C, R,
               s.data_ptr(), s.stride(0), ssr, ssc, B, R, C, group_c,
-              _qflags(clamp, eps_add, scale_bf16), inv_mode, _stream())
+              _qflags(clamp, eps_add, scale_bf16, torch_arith), inv_mode, _stream())
     if not transposed:
         q = qc
         qT = qct
@@ -122,7 +132,8 @@ def quant_block_had128(x, *, along_rows=False, clamp=True, inv_mode=INV_RCP_OF_S
     return q, s
 
 
-def quant_row(x, *, clamp=True, group=0, eps_add=False, scale_bf16=False, inv_mode=INV_RCP_OF_SCALE, hadamard128=False):
+def quant_row(x, *, clamp=True, group=0, eps_add=False, scale_bf16=False, inv_mode=INV_RCP_OF_SCALE, hadamard128=False,
+              torch_arith=None):
     """Per-row (``group=0``) or per-(row, 128 columns) absmax quantisation of the last dim.
     ``x``: bf16 [..., cols].  Returns ``(q, s)`` with ``s`` fp32 [...] or [..., cols/128].
     ``hadamard128`` rotates every group of 128 columns by H_128 first (fused, one read)."""
@@ -137,7 +148,7 @@ def quant_row(x, *, clamp=True, group=0, eps_add=False, scale_bf16=False, inv_mo
     q = torch.empty((rows, cols), dtype=torch.int8, device=x.device)
     s = torch.empty((rows, cols // 128) if group else (rows,), dtype=torch.float32, device=x.device)
     _lib.call("ti8_quant_row", x2.data_ptr(), x2.stride(0), q.data_ptr(), cols, s.data_ptr(), rows, cols, group,
-              _qflags(clamp, eps_add, scale_bf16) | (Q_HAD128 if hadamard128 else 0), inv_mode, _stream())
+              _qflags(clamp, eps_add, scale_bf16, torch_arith) | (Q_HAD128 if hadamard128 else 0), inv_mode, _stream())
     lead = x.shape[:-1]
     return q.reshape(*lead, cols), s.reshape(*lead, cols // 128) if group else s.reshape(*lead)
 
@@ -177,32 +188,44 @@ def quant_row_col_t(x, *, clamp=True, inv_mode=INV_RCP_OF_SCALE):
     s_col = torch.empty((C,), dtype=torch.float32, device=x.device)
     flags = _qflags(clamp, False, False)
     stream = _stream()
+    args = (x.data_ptr(), x.stride(0), q.data_ptr(), C, s_row.data_ptr(), qT.data_ptr(), R, s_col.data_ptr())
     if torch.cuda.is_current_stream_capturing():
         # a replayed call cannot alternate: plain workspace, cleared by the library on every replay
         ws = torch.empty((R + C,), dtype=torch.float32, device=x.device)
+        _lib.call("ti8_quant_row_col_t", *args, ws.data_ptr(), R, C, flags, inv_mode, stream)
     else:
-        slot = _pingpong_workspace(x.device, stream, R, C)
-        ws = slot[0]
-        flags |= Q_WS_PINGPONG | (Q_WS_SECOND if slot[1] else 0)
-    _lib.call("ti8_quant_row_col_t", x.data_ptr(), x.stride(0), q.data_ptr(), C, s_row.data_ptr(), qT.data_ptr(), R,
-              s_col.data_ptr(), ws.data_ptr(), R, C, flags, inv_mode, stream)
-    if flags & Q_WS_PINGPONG:
-        slot[1] ^= 1   # only once the launches are queued: a rejected call leaves both parts as they were
+        with _PINGPONG_LOCK:
+            slot = _pingpong_workspace(x.device, stream, R, C)
+            _lib.call("ti8_quant_row_col_t", *args, slot[0].data_ptr(), R, C,
+                      flags | Q_WS_PINGPONG | (Q_WS_SECOND if slot[1] else 0), inv_mode, stream)
+            slot[1] ^= 1   # only once the launches are queued: a rejected call leaves both parts as they were
     return q, s_row, qT, s_col
 
 
 # Two-part workspaces of quant_row_col_t: a call collects its maxima in one part and clears the
-# other for the next call, so no call needs a launch that clears memory.  One buffer (and the
-# part to use next) per device, stream and shape: calls on one stream run in order and can share
-# it; calls on different streams may overlap and get different buffers.
-_PINGPONG_WS = {}
+# other for the next call, so no call needs a launch that clears memory.  One buffer (and the part
+# to use next) per device, stream and shape: calls on one stream run in order and can share it;
+# calls on different streams may overlap and get different buffers.  The cache holds the
+# _PINGPONG_SLOTS most recently used buffers (a training step alternates between a handful of
+# shapes); a buffer that drops out is released once the work queued on it has run (torch's
+# allocator keeps the memory of a freed tensor until the stream has passed the free), and a
+# shape that comes back starts again from a zero-filled buffer.  Lookup, launch and the flip of
+# the part happen under one lock, so that threads sharing a stream enqueue their calls in the
+# order in which they were handed the parts.
+_PINGPONG_SLOTS = 16
+_PINGPONG_WS = collections.OrderedDict()
+_PINGPONG_LOCK = threading.Lock()
 
 
 def _pingpong_workspace(device, stream, R, C):
+    """The slot [buffer of 2 * (R + C) floats, part the next call works in]; call with the lock held."""
     key = (device.index, stream, R, C)
-    slot = _PINGPONG_WS.get(key)
+    slot = _PINGPONG_WS.pop(key, None)
     if slot is None:
-        slot = _PINGPONG_WS[key] = [torch.zeros((2 * (R + C),), dtype=torch.float32, device=device), 0]
+        slot = [torch.zeros((2 * (R + C),), dtype=torch.float32, device=device), 0]
+        while len(_PINGPONG_WS) >= _PINGPONG_SLOTS:
+            _PINGPONG_WS.popitem(last=False)
+    _PINGPONG_WS[key] = slot          # most recently used last
     return slot
 
 

@@ -3,10 +3,13 @@ promotion multiplies by the scale PRODUCT (``acc += f32(dot) * (sA*sB)``)."""
 import torch
 
 from . import ops
-from ._common import StageTimer, calc_diff
+from typing import Tuple
+
+from ._common import StageTimer, bf16_reference_nt, calc_diff, ceildiv
 from ._lib import COMBINE_MUL_PROD, INV_RCP_OF_SCALE, SCALE_BLOCK128
 
-__all__ = ["tl_gemm", "triton_per_block_quant", "bwd_33", "calc_diff"]
+__all__ = ["tl_gemm", "triton_per_block_quant", "bwd_33", "per_block_cast_to_int8", "assert_tl_gemm_correctness", "ceildiv",
+           "calc_diff"]
 
 
 def triton_per_block_quant(x: torch.Tensor, out="like"):
@@ -43,3 +46,28 @@ def bwd_33(a, b, verbose=False):
     kernel(A_int8, B_int8, C, A_scale, B_scale)
     t.stop("kernel time")
     return C
+
+
+def per_block_cast_to_int8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """[B,M,N] bf16 -> (int8, fp32 [B,M/128,N/128]): the pure-torch block quantiser of
+    tilelang/block_channel_bwd.py:96-104 (unused at its call sites, :201-202) as a HIP kernel.  This
+    copy takes the absmax in fp32, so scale and product are fp32: reciprocal(amax) * 127, round half
+    to even, clamp +-127, returned scale reciprocal(scale)."""
+    assert x.dim() == 3
+    return ops.quant_block(x.contiguous(), torch_arith="f32")
+
+
+def assert_tl_gemm_correctness(B, M, N, K, block_N, in_dtype, out_dtype, accum_dtype):
+    """The reference's self-check (tilelang/block_channel_bwd.py:165-193): N(0,1) operands, both 3-D,
+    ``calc_diff`` against the bf16 product below 1e-3."""
+    kernel = tl_gemm(B, M, N, K, block_N, in_dtype, out_dtype, accum_dtype)
+    a = torch.randn(B, M, K).to(torch.bfloat16).cuda()
+    b = torch.randn(B, N, K).to(torch.bfloat16).cuda()
+    A_int8, A_scale = triton_per_block_quant(a.clone())
+    B_int8, B_scale = triton_per_block_quant(b.clone())
+    C = torch.zeros(B, M, N, device="cuda", dtype=torch.bfloat16)
+    kernel(A_int8, B_int8, C, A_scale, B_scale)
+    diff = calc_diff(C, bf16_reference_nt(a, b))
+    print(f"diff: {diff}")
+    assert diff < 1e-3
+    return float(diff)

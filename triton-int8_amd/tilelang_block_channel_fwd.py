@@ -7,11 +7,11 @@ from typing import Tuple
 import torch
 
 from . import ops
-from ._common import StageTimer, calc_diff
+from ._common import StageTimer, bf16_reference_nt, calc_diff
 from ._lib import COMBINE_MUL_PROD, INV_RCP_OF_SCALE, SCALE_BLOCK_K256, SCALE_ROW
 
 __all__ = ["tl_gemm", "triton_per_block_quant", "triton_per_token_quant", "fwd_32", "per_token_cast_to_int8",
-           "per_block_cast_to_int8", "calc_diff"]
+           "per_block_cast_to_int8", "assert_tl_gemm_correctness", "calc_diff"]
 
 
 def triton_per_block_quant(x: torch.Tensor):
@@ -61,22 +61,36 @@ def fwd_32(a, b, verbose=False):
 
 
 def per_token_cast_to_int8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
-    """The reference author's pure-torch quantiser (tilelang/block_channel_fwd.py:215-220),
-    unused at its call sites (:255-256); round-half-to-even and clamp +-127, so it is NOT
-    equal to the kernels on exact .5 ties.  Plain torch ops on whatever device ``x`` is on."""
+    """[M,N] bf16 -> (int8 [M,N], bf16 [M,1]): the reference author's pure-torch per-row quantiser
+    (tilelang/block_channel_fwd.py:215-220; commented out at its call sites, :255-256) as a HIP
+    kernel.  Evaluated as torch evaluates it on a bf16 tensor: every intermediate in bf16,
+    ``127.0 / amax`` as reciprocal times 127, round half to even, clamp +-127, so it is NOT equal to
+    the Triton kernels (exact .5 ties, and the bf16 rounding of ``x * scale``)."""
     m, n = x.shape
-    x_amax = x.abs().amax(dim=1, keepdim=True).clamp(min=1e-4)
-    scale = 127.0 / x_amax
-    x_int8 = (x * scale).round().clamp(-127, 127).to(torch.int8)
-    return x_int8.view(m, n), (1.0 / scale).view(m, -1)
+    q, s = ops.quant_row(x, torch_arith="bf16")
+    return q.view(m, n), s.to(x.dtype).view(m, -1)
 
 
 def per_block_cast_to_int8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
-    """tilelang/block_channel_fwd.py:222-230; see :func:`per_token_cast_to_int8`."""
+    """[B,M,N] bf16 -> (int8, bf16 [B,M/128,N/128]) (tilelang/block_channel_fwd.py:222-230);
+    see :func:`per_token_cast_to_int8`."""
     assert x.dim() == 3
-    b, m, n = x.shape
-    x_view = x.view(b, m // 128, 128, n // 128, 128)
-    x_amax = x_view.abs().amax(dim=(2, 4), keepdim=True).clamp(min=1e-4)
-    scale = 127.0 / x_amax
-    x_int8 = (x_view * scale).round().clamp(-127, 127).to(torch.int8)
-    return x_int8.view(b, m, n), (1.0 / scale).view(b, m // 128, n // 128)
+    q, s = ops.quant_block(x.contiguous(), torch_arith="bf16")
+    return q, s.to(x.dtype)
+
+
+def assert_tl_gemm_correctness(B, M, N, K, block_N, in_dtype, out_dtype, accum_dtype):
+    """The reference's self-check (tilelang/block_channel_fwd.py:242-268): N(0,1) operands through the
+    quantisers and the kernel ``tl_gemm`` returns, ``calc_diff`` against the bf16 product below 1e-3.
+    There is no generated source to look at here (the reference asserts that TileLang produced some)."""
+    kernel = tl_gemm(B, M, N, K, block_N, in_dtype, out_dtype, accum_dtype)
+    a = torch.randn(B, M, K).to(torch.bfloat16).cuda()
+    b = torch.randn(N, K).to(torch.bfloat16).cuda()
+    A_int8, A_scale = triton_per_block_quant(a)
+    B_int8, B_scale = triton_per_token_quant(b)
+    C = torch.zeros(B, M, N, device="cuda", dtype=torch.bfloat16)
+    kernel(A_int8, B_int8, C, A_scale, B_scale)
+    diff = calc_diff(C, bf16_reference_nt(a, b))
+    print(f"diff: {diff}")
+    assert diff < 1e-3
+    return float(diff)
