@@ -142,6 +142,50 @@ def event_time_ms(fn, reps):
     return sum(a.elapsed_time(b) for a, b in evs) / reps
 
 
+def probe_mfma(dev, iters=4096, reps=5):
+    """What the i8 matrix pipe sustains on a loop of nothing but MFMAs (ti8_probe_mfma): all-zero
+    operands, pseudo-random operands, and random operands with the block-channel promotion's vector
+    work beside them; the shader clock during each.  The random-operand rate is the practical ceiling
+    of a GEMM on real data (the clock falls under the power limit when the data toggles)."""
+    from triton_int8_amd import _lib
+    wgs = torch.cuda.get_device_properties(dev).multi_processor_count
+    sink = torch.empty(wgs * 512, dtype=torch.float32, device=dev)
+    clocks = torch.zeros(2, dtype=torch.int64, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    out = {}
+    for name, rnd, promo in (("zero_operands", 0, 0), ("random_operands", 1, 0), ("random_operands_with_promotion", 1, 1)):
+        call = lambda: _lib.call("ti8_probe_mfma", sink.data_ptr(), sink.numel(), clocks.data_ptr(), wgs, iters, rnd, promo, stream)
+        call()
+        ms = event_time_ms(call, reps)
+        ck = clocks.cpu().tolist()
+        ops = wgs * 8.0 * iters * 16 * 65536
+        out[name] = {"TOPS": round(ops / (ms * 1e-3) / 1e12, 1), "clock_MHz": round(ck[0] / max(ck[1], 1) * 100.0, 0),
+                     "frac_of_nominal": round(ops / (ms * 1e-3) / 1e12 / INT8_PEAK_TOPS, 4)}
+    return out
+
+
+def probe_gemm_data_dependence(T, dev, reps=20):
+    """The dominant GEMM kernels on random int8 operands and on all-zero operands of the same shape:
+    same instructions, same memory traffic, different switching activity."""
+    from triton_int8_amd import ops
+    from triton_int8_amd._lib import SCALE_BLOCK128, SCALE_ROW
+    g = torch.Generator().manual_seed(0)
+    A = torch.randint(-127, 128, (1, M, K), generator=g, dtype=torch.int8).to(dev)
+    B = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8).to(dev)
+    sa_blk = torch.full((1, M // 128, K // 128), 1e-2, device=dev)
+    sa_row, sb_row = torch.full((1, M), 1e-2, device=dev), torch.full((N,), 1e-2, device=dev)
+    res = {}
+    for data, (a, b) in (("random", (A, B)), ("zero", (torch.zeros_like(A), torch.zeros_like(B)))):
+        promo = lambda: ops.gemm_i8_nt(a, b, sa_blk, SCALE_BLOCK128, sb_row, SCALE_ROW)
+        i32 = lambda: ops.gemm_i8_nt(a, b, sa_row, SCALE_ROW, sb_row, SCALE_ROW, acc_i32_full=True)
+        for name, fn in (("promotion_kernel", promo), ("int32_kernel", i32)):
+            fn()
+            ms = event_time_ms(fn, reps)
+            res[f"{name}_{data}_us"] = round(ms * 1e3, 1)
+            res[f"{name}_{data}_TOPS"] = round(2.0 * M * N * K / (ms * 1e-3) / 1e12, 1)
+    return res
+
+
 def cpu_baseline(scheme):
     """The torch-CPU oracle of the same path on the host cores, bounded sample."""
     from oracle import linear as olin
@@ -161,11 +205,13 @@ def cpu_baseline(scheme):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=30)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200, help="timed steps (200 x 0.5 ms: box-to-box spread, not timer noise, is what is left)")
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--scheme", default="block_channel", choices=["block_channel", "row_block", "double_channel"])
     ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5], help="benchmark configuration (2 = headline)")
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU baseline leg (profiling runs)")
+    ap.add_argument("--probe", choices=["mfma"], help="print what the i8 matrix pipe sustains on pure MFMA loops (zero / random operands, "
+                    "clock) and the GEMM kernels on zero against random data, then exit")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build runs on ONE GPU only (the path has no collectives yet); use --gpus 1")
@@ -177,6 +223,10 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.probe == "mfma":
+        print(json.dumps({"probe": "mfma", "nominal_peak_TOPS": INT8_PEAK_TOPS, "pure_mfma_loop": probe_mfma(dev),
+                          "gemm_8192x4096x4096": probe_gemm_data_dependence(T, dev)}), flush=True)
+        return
     if args.config != 2:
         return other_config(args, T, dev)
     X, W, dY = (t.to(dev) for t in make_inputs())
@@ -198,36 +248,42 @@ def main():
     # events on the launch stream while whole steps run, in a second pass of K steps (so the events
     # do not sit in the region `value` is timed on)
     from triton_int8_amd import _lib
+    ev_steps = min(args.steps, 50)
     with _lib.timed_launches() as rec:
-        for _ in range(args.steps):
+        for _ in range(ev_steps):
             step()
     torch.cuda.synchronize()
-    per_entry_ms = {name: sum(a.elapsed_time(b) for a, b in ev) / args.steps for name, ev in rec.items()}
+    per_entry_ms = {name: sum(a.elapsed_time(b) for a, b in ev) / ev_steps for name, ev in rec.items()}
     g = [a.elapsed_time(b) for a, b in rec["ti8_gemm_i8_nt"]]
-    assert len(g) == 3 * args.steps
-    gemm_ms = [sum(g[i::3]) / args.steps for i in range(3)]
+    assert len(g) == 3 * ev_steps
+    gemm_ms = [sum(g[i::3]) / ev_steps for i in range(3)]
     kernel = "gemm_i8_kernel<256,256,2,4,EPI_ROWS>" if args.scheme == "double_channel" else "gemm_i8_kernel<256,256,2,4,EPI_PROMOTE_CHAIN>"
     avg_ms = sum(gemm_ms) / len(gemm_ms)
     achieved = 2.0 * M * N * K / (avg_ms * 1e-3) / 1e12
 
     # ---- secondary: the activation quantiser against HBM, and the bf16 GEMM the reference
     # times beside its int8 path (test.py:34-38)
-    q_ms = event_time_ms(lambda: ops.quant_block(X[None], clamp=True, with_transpose=True), args.steps)
+    side_reps = min(args.steps, 30)
+    q_ms = event_time_ms(lambda: ops.quant_block(X[None], clamp=True, with_transpose=True), side_reps)
     q_bytes = 4.0 * M * K  # 2 B read + 1 B int8 + 1 B transposed int8 per element
-    q1_ms = event_time_ms(lambda: ops.quant_block(X[None], clamp=True), args.steps)
+    q1_ms = event_time_ms(lambda: ops.quant_block(X[None], clamp=True), side_reps)
     # a plain device copy of X (64 MiB read + 64 MiB write): the reachable HBM rate on this box,
     # and the known-size kernel the rocprofv3 FETCH_SIZE / WRITE_SIZE counters are calibrated on
     X.clone()
-    copy_ms = event_time_ms(lambda: X.clone(), args.steps)
+    copy_ms = event_time_ms(lambda: X.clone(), side_reps)
     bf16_fns = (lambda: X @ W.t(), lambda: dY @ W, lambda: dY.t() @ X)
     for f in bf16_fns:
         f()
         f()
-    bf16_ms = sum(event_time_ms(f, args.steps) for f in bf16_fns)
+    bf16_ms = sum(event_time_ms(f, side_reps) for f in bf16_fns)
 
-    # HBM-side bytes per GEMM launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled on the device
-    # copy above (profiles/bench_config2_*_hbm_counters.md); measured for these two schemes
-    traffic = {"block_channel": 257610359, "double_channel": 257689548}.get(args.scheme)
+    # HBM-side bytes per GEMM launch: NOT measured by this run.  They come from two rocprofv3 --pmc runs of this
+    # command (FETCH_SIZE, WRITE_SIZE), scaled on the device copy above, whose summary is the file named in
+    # `traffic_source`; measured for these two schemes
+    traffic = {"block_channel": 257610249, "double_channel": 257628126}.get(args.scheme)
+    traffic_source = {"block_channel": "profiles/bench_config2_block_channel_counters.md (section 3)",
+                      "double_channel": "profiles/bench_config2_double_channel_counters.md (section 3)"}.get(args.scheme)
+    probe = probe_mfma(dev, iters=2048, reps=3)
 
     out = {
         "metric": METRIC, "value": round(tops, 2), "unit": "TOPS", "n_gpus": 1, "steps": args.steps,
@@ -238,18 +294,29 @@ def main():
                    "scheme": args.scheme, "M": M, "K": K, "N": N},
         "pct_int8_peak": round(100.0 * tops / INT8_PEAK_TOPS, 2),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": INT8_PEAK_TOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / INT8_PEAK_TOPS, 4), "traffic": traffic, "kernel": kernel,
+                     "frac": round(achieved / INT8_PEAK_TOPS, 4), "traffic": traffic, "traffic_source": traffic_source,
+                     "practical_peak": probe["random_operands"]["TOPS"],
+                     "frac_of_practical_peak": round(achieved / probe["random_operands"]["TOPS"], 4),
+                     "practical_peak_note": "pure v_mfma_i32_32x32x32_i8 loop on random operands in this run (bench.py --probe mfma): "
+                                            f"{probe['random_operands']['TOPS']} TOPS at {probe['random_operands']['clock_MHz']:.0f} MHz; "
+                                            f"on zero operands {probe['zero_operands']['TOPS']} TOPS at {probe['zero_operands']['clock_MHz']:.0f} MHz",
+                     "kernel": kernel,
                      "ops_per_launch": 2 * M * N * K, "launch_ms": [round(t, 4) for t in gemm_ms],
                      "note": "int8 multiply-adds counted as 2*M*N*K operations per launch; peak is the dense int8 MFMA rate"},
         "quant_roofline": {"bound": "hbm", "kernel": "quant_block_kernel<1,true,true>",
                            "achieved": round(q_bytes / (q_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                            "frac": round(q_bytes / (q_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "launch_ms": round(q_ms, 4),
                            "bytes_per_launch": int(q_bytes),
+                           "note": "launched back to back; `in_step` is the same kernel where it runs inside a step (X and dY each, behind a GEMM)",
+                           "in_step": ({"launch_ms": round(per_entry_ms["ti8_quant_block"] / 2, 4),
+                                        "frac": round(q_bytes / (per_entry_ms["ti8_quant_block"] / 2 * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+                                       if "ti8_quant_block" in per_entry_ms else None),
                            "single_output_GBs": round(3.0 * M * K / (q1_ms * 1e-3) / 1e9, 1)},
         "copy_GBs": round(2.0 * X.numel() * 2 / (copy_ms * 1e-3) / 1e9, 1),
         "bf16_matmul_ms_per_step": round(bf16_ms, 4),
         "bf16_matmul_tflops": round(6.0 * M * N * K / (bf16_ms * 1e-3) / 1e12, 1),
         "entry_point_ms_per_step": {k: round(v, 4) for k, v in sorted(per_entry_ms.items())},
+        "between_launches_ms_per_step": round(dt * 1e3 - sum(per_entry_ms.values()), 4),
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.scheme)

@@ -257,6 +257,18 @@ int ti8_gemm_i8_nt_i32(const int8_t* A, int64_t bsa, int64_t lda,
                        int32_t* C, int64_t bsc, int64_t ldc,
                        int64_t batch, int64_t M, int64_t N, int64_t K, ti8_stream_t stream);
 
+/* ---------------------------------------------------------------------------------
+ * Measurement aid (no counterpart in the reference; used by bench.py --probe mfma): a loop of nothing
+ * but v_mfma_i32_32x32x32_i8 on `workgroups` workgroups of 8 waves, `iters` x 16 MFMAs per wave,
+ * operands all zero or pseudo-random, optionally with the block-channel promotion's vector work
+ * (convert + fma per accumulator element per four MFMAs).  Operations = workgroups * 8 * iters * 16 *
+ * 65536; time it with events around the call.
+ *   sink   float [workgroups * 512]   scratch output that keeps the loop alive
+ *   clocks int64 [2]                  [0] shader-clock cycles, [1] ticks of the constant 100 MHz
+ *                                     counter, both across the loop of workgroup 0: [0] / [1] * 100 = MHz */
+int ti8_probe_mfma(float* sink, int64_t sink_elems, int64_t* clocks, int workgroups, int iters,
+                   int random_operands, int with_promotion, ti8_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -153,3 +153,39 @@ def test_linear_wiring_reduces_to_the_entry_points():
         assert float(calc_diff(Y, X.float() @ W.float().t())) < 1e-3
         assert float(calc_diff(dX, dY.float() @ W.float())) < 1e-3
         assert float(calc_diff(dW, dY.float().t() @ X.float())) < 1e-3
+
+
+def test_config1_plumbing_forward_as_worded():
+    """BASELINE config 1 as worded, on the CPU: block-channel INT8 linear forward, X 2048 x 4096 bf16
+    ~N(0,1) with 1 % of the input channels x20, W 4096 x 4096 ~N(0,0.02), per-token scale on X,
+    per-128x128-block scale on W, round to nearest, int32 matmul, bf16 out = acc * sx * sw, seed 0."""
+    import numpy as np
+    from oracle import linear as olin
+    g = torch.Generator().manual_seed(0)
+    M, K, N = 2048, 4096, 4096
+    X = torch.randn(M, K, generator=g)
+    X[:, torch.randperm(K, generator=g)[: K // 100 + 1]] *= 20.0
+    X = X.to(torch.bfloat16)
+    W = (torch.randn(N, K, generator=g) * 0.02).to(torch.bfloat16)
+    xq, xs = olin.quant2d(X, olin.ROW, clamp=True)
+    wq, ws = olin.quant2d(W, olin.BLOCK, clamp=True)
+    # quantiser invariants: every group reaches 127, codes reconstruct x within half a step
+    assert int(xq.abs().amax(dim=1).min()) == 127 and xs.shape == (M,)
+    assert int(wq.reshape(N // 128, 128, K // 128, 128).abs().amax(dim=(1, 3)).min()) == 127 and ws.shape == (N // 128, K // 128)
+    assert bool(((X.float() - xq.float() * xs[:, None]).abs() <= xs[:, None] * (0.5 + 1e-4)).all())
+    wsx = ws.repeat_interleave(128, 0).repeat_interleave(128, 1)
+    assert bool(((W.float() - wq.float() * wsx).abs() <= wsx * (0.5 + 1e-4)).all())
+    Y = olin.gemm_scaled(xq, xs, olin.ROW, wq, ws, olin.BLOCK)
+    assert Y.dtype == torch.bfloat16 and Y.shape == (M, N)
+    # the whole path equals the layer entry point of that scheme, and a sampled block of the integer
+    # GEMM equals an int64 evaluation
+    assert torch.equal(Y, olin.linear_fwd_bwd(X, W, torch.zeros(M, N, dtype=torch.bfloat16), "row_block")[0])
+    r, c = slice(1024, 1088), slice(512, 640)
+    acc = (xq[r, :128].long() @ wq[c, :128].long().t())
+    part = olin.gemm_scaled(xq[r, :128], xs[r], olin.ROW, wq[c, :128], ws[4:5, :1], olin.BLOCK, out_dtype=torch.float32)
+    want = (acc.double() * xs[r, None].double() * float(ws[4, 0])).float()
+    assert np.allclose(part.numpy(), want.numpy(), rtol=3e-7, atol=0)
+    # against the bf16 product: 1 % of the channels x20 costs int8 resolution, well inside 1e-2
+    ref = X.float() @ W.float().t()
+    from oracle._prims import calc_diff
+    assert float(calc_diff(Y, ref)) < 2e-3

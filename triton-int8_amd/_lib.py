@@ -26,6 +26,7 @@ PROTOTYPES = {
                        _vp, _int, _i64, _i64, _i64, _vp, _int, _i64, _i64, _i64,
                        _i64, _i64, _i64, _i64, _int, _int, _f32, _f32, _int, _vp],
     "ti8_gemm_i8_nt_i32": [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp],
+    "ti8_probe_mfma": [_vp, _i64, _vp, _int, _int, _int, _int, _vp],
 }
 EXPORTS = ["ti8_version", "ti8_last_error", "ti8_arch"] + list(PROTOTYPES)
 
