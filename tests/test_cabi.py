@@ -115,18 +115,21 @@ def test_python_surface_rejects_bad_inputs_without_gpu():
         T.block_channel_fwd32.triton_gemm(None, None, None, None, out_dtype=torch.float16)
 
 
-def test_latency_harness_refuses_shapes_it_has_not_completed():
-    """No GPU needed: the shape checks come before anything touches the device.  The bwd_33 half is
-    limited to small shapes (its bf16 baseline faulted the GPU at large ones), the fwd_32 half to
-    the reference's own shape."""
+def test_latency_harness_shape_rules():
+    """No GPU needed: the shape check comes before anything touches the device, and the bf16 product of
+    two large 3-D operands is never one batched matmul call (that call faulted the GPU twice)."""
+    import torch
     import triton_int8_amd as T
-    with pytest.raises(ValueError, match="bwd half"):
-        T.latency.main(["--batch", "4", "--m", "8192", "--n", "8192", "--k", "8192"])
-    with pytest.raises(ValueError, match="bwd half"):
-        T.latency.main(["--halves", "bwd", "--batch", "2", "--m", "8192", "--n", "4096", "--k", "4096"])
-    with pytest.raises(ValueError, match="fwd half"):
-        T.latency.main(["--halves", "fwd", "--batch", "8", "--m", "8192", "--n", "8192", "--k", "8192"])
+    lat = T.latency
+    with pytest.raises(ValueError, match="beyond the largest shape"):
+        lat.main(["--batch", "8", "--m", "8192", "--n", "8192", "--k", "8192"])
     with pytest.raises(ValueError, match="multiples of 128"):
-        T.latency.check_shape(1, 100, 128, 128)
-    T.latency.check_shape(4, 8192, 8192, 8192, "fwd")
-    T.latency.check_shape(2, 256, 512, 2048, "bwd")
+        lat.check_shape(1, 100, 128, 128)
+    lat.check_shape(4, 8192, 8192, 8192)
+    meta = lambda *shape: torch.empty(*shape, dtype=torch.bfloat16, device="meta")
+    assert lat.batched_matmul_allowed(meta(4, 8192, 8192), meta(8192, 8192))            # 3-D x 2-D: always one call
+    assert lat.batched_matmul_allowed(meta(2, 256, 2048), meta(2, 512, 2048))
+    assert not lat.batched_matmul_allowed(meta(2, 8192, 4096), meta(2, 4096, 4096))
+    assert not lat.batched_matmul_allowed(meta(4, 8192, 8192), meta(4, 8192, 8192))
+    a, b = torch.randn(3, 16, 8).to(torch.bfloat16), torch.randn(3, 4, 8).to(torch.bfloat16)
+    assert torch.equal(T._common.bf16_reference_nt(a, b), torch.matmul(a, b.transpose(-2, -1)))

@@ -310,3 +310,27 @@ def test_config5_down_proj_layer_sampled_tiles(T, dev):
     for (name, C, Aq, sA, oA, Bq, sB, oB, sc), got in zip(pieces, (y.detach().reshape(tokens, N), x.grad.reshape(tokens, K), lin.weight.grad)):
         assert torch.equal(C, got), name
         check_sampled_tiles(C, Aq, sA, oA, Bq, sB, oB, g, f"config 5 down_proj {name}", sc)
+
+
+def test_reference_acceptance_shape(T, dev):
+    """The reference's own self-check at its own shape (triton/block_channel_fwd32.py:257-272 and the
+    same block in every script; test.py:32-45): N(0,1) operands, B = 4, M = N = K = 8192,
+    calc_diff(C, bf16 product) < 1e-3, for fwd_32 (3-D x 2-D) and bwd_33 (3-D x 3-D) of every scheme.
+    The bf16 product of two 3-D operands is taken batch by batch as 2-D products."""
+    from triton_int8_amd._common import bf16_reference_nt
+    g = torch.Generator(device=dev).manual_seed(42)
+    B, S = 4, 8192
+    a = torch.randn(B, S, S, generator=g, device=dev, dtype=torch.bfloat16)
+    b2 = torch.randn(S, S, generator=g, device=dev, dtype=torch.bfloat16)
+    ref = bf16_reference_nt(a, b2)
+    for mod in ("block_channel_fwd32", "double_channel_fwd32", "fused_fwd32", "tilelang_block_channel_fwd"):
+        C = getattr(T, mod).fwd_32(a, b2)
+        assert C.shape == (B, S, S) and float(T.calc_diff(C, ref)) < 1e-3, mod
+        del C
+    del ref, b2
+    b3 = torch.randn(B, S, S, generator=g, device=dev, dtype=torch.bfloat16)
+    ref = bf16_reference_nt(a, b3)
+    for mod in ("block_channel_bwd33", "double_channel_bwd33", "fused_bwd33", "tilelang_block_channel_bwd"):
+        C = getattr(T, mod).bwd_33(a, b3)
+        assert C.shape == (B, S, S) and float(T.calc_diff(C, ref)) < 1e-3, mod
+        del C
