@@ -334,3 +334,37 @@ def test_reference_acceptance_shape(T, dev):
         C = getattr(T, mod).bwd_33(a, b3)
         assert C.shape == (B, S, S) and float(T.calc_diff(C, ref)) < 1e-3, mod
         del C
+
+
+def test_config5_decoder_layer_full_width(T, dev):
+    """Config 5 at its stated size: one training step of the decoder layer (hidden 4096, 32 heads, MLP
+    14336, 4 x 4096 tokens) with every linear in INT8 block-channel.  Each of the seven linears is
+    checked on the operands it actually received (captured by hooks): the module's Y, dX and dW equal
+    the launches of the same step on the captured tensors bit for bit, and those are compared with the
+    oracle element by element on sampled 256 x 256 tiles (contraction dims 4096, 14336 and 16384)."""
+    torch.manual_seed(4)
+    g = make_gen(44)
+    lay = T.decoder.DecoderLayer(4096, 32, 14336, int8=True, device=dev)
+    x = torch.randn(4, 4096, 4096, device=dev, dtype=torch.bfloat16)
+    seen = {}
+    names = ("q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj")
+    hooks = []
+    for name in names:
+        mod = getattr(lay, name)
+        hooks.append(mod.register_forward_hook(lambda m, inp, out, name=name: seen.setdefault(name, {}).update(x=inp[0].detach(), y=out.detach())))
+        hooks.append(mod.register_full_backward_hook(lambda m, gin, gout, name=name: seen[name].update(dx=gin[0].detach(), dy=gout[0].detach())))
+    xi = x.clone().requires_grad_(True)
+    y = lay(xi)
+    y.float().pow(2).mean().backward()
+    for h in hooks:
+        h.remove()
+    assert torch.isfinite(y).all() and torch.isfinite(xi.grad).all()
+    for name in names:
+        c, mod = seen[name], getattr(lay, name)
+        K, N = mod.in_features, mod.out_features
+        X2, dY2 = c["x"].reshape(-1, K), c["dy"].reshape(-1, N)
+        pieces = block_channel_step_pieces(T, X2, mod.weight.detach(), dY2)
+        for (what, C, Aq, sA, oA, Bq, sB, oB, sc), got in zip(pieces, (c["y"].reshape(-1, N), c["dx"].reshape(-1, K), mod.weight.grad)):
+            assert torch.equal(C, got), f"{name} {what}"
+            check_sampled_tiles(C, Aq, sA, oA, Bq, sB, oB, g, f"decoder {name} {what}", sc)
+        del pieces
