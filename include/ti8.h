@@ -124,6 +124,21 @@ int ti8_quant_block(const void* x, int64_t bsx, int64_t ldx,
                     int64_t B, int64_t R, int64_t C, int group_c,
                     int qflags, int inv_mode, ti8_stream_t stream);
 
+/* The same for up to 4 operands in ONE launch (128 x 128 tiles, every operand with the same set of
+ * outputs: q, qT or both): a training step quantises X and dY the same way (triton/block_channel_fwd32.py:221
+ * for X, the same call on dY for dX = fwd_32(dY, W^T)), and one launch instead of two saves a kernel
+ * boundary.  Each operand's fields mean what the arguments of ti8_quant_block mean; `operands` is a
+ * HOST array.  Bit-identical to separate ti8_quant_block calls. */
+typedef struct ti8_qblock_operand {
+    const void* x; int64_t bsx, ldx;
+    int8_t* q; int64_t bsq, ldq;
+    int8_t* qT; int64_t bsqt, ldqt;
+    float* s; int64_t ssb, ssr, ssc;
+    int64_t B, R, C;
+} ti8_qblock_operand;
+int ti8_quant_block_multi(const ti8_qblock_operand* operands, int count,
+                          int qflags, int inv_mode, ti8_stream_t stream);
+
 /* ---------------------------------------------------------------------------------
  * Block quantiser with the block-diagonal 128-point Walsh-Hadamard rotation fused in: what
  * BASELINE config 4 calls the "fused Hadamard + quantize path".  The reference has no such

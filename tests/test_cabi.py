@@ -133,3 +133,22 @@ def test_latency_harness_shape_rules():
     assert not lat.batched_matmul_allowed(meta(4, 8192, 8192), meta(4, 8192, 8192))
     a, b = torch.randn(3, 16, 8).to(torch.bfloat16), torch.randn(3, 4, 8).to(torch.bfloat16)
     assert torch.equal(T._common.bf16_reference_nt(a, b), torch.matmul(a, b.transpose(-2, -1)))
+
+
+def test_quant_block_multi_validation(lib):
+    """ti8_quant_block_multi takes a host array of operand descriptors; bad ones are rejected before any launch."""
+    import triton_int8_amd
+    L = triton_int8_amd._lib
+    good = dict(x=FAKE, bsx=0, ldx=128, q=FAKE, bsq=0, ldq=128, qT=None, bsqt=0, ldqt=0, s=FAKE, ssb=0, ssr=1, ssc=1, B=1, R=128, C=128)
+    arr = lambda *ds: (L.QBlockOperand * len(ds))(*[L.QBlockOperand(**d) for d in ds])
+    cases = [((None, 1), 1, "operands is required"),
+             ((arr(good), 0), 2, "between 1 and 4"),
+             ((arr(good, good, good, good, good), 5), 2, "between 1 and 4"),
+             ((arr({**good, "R": 100}), 1), 2, "R%128"),
+             ((arr({**good, "x": None}), 1), 1, "required"),
+             ((arr(good, {**good, "qT": FAKE, "ldqt": 128}), 2), 4, "same outputs"),
+             ((arr({**good, "q": FAKE + 4}), 1), 3, "aligned")]
+    for (ops_, n), code, msg in cases:
+        rc = lib.ti8_quant_block_multi(ops_, n, 1, 0, None)
+        assert rc == code and msg in lib.ti8_last_error().decode(), (lib.ti8_last_error(), msg)
+    assert lib.ti8_quant_block_multi(arr(good), 1, 8, 0, None) == 4      # TI8_Q_HAD128

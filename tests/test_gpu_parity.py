@@ -81,6 +81,30 @@ def test_block_quant(T, dev):
     assert bits_equal(q, qo) and bits_equal(s, so)
 
 
+def test_block_quant_of_several_operands_in_one_launch(T, dev):
+    """ti8_quant_block_multi = separate ti8_quant_block calls, bit for bit: operands of different shapes,
+    with and without the transposed copy, and the layer step that uses it for X and dY."""
+    xs = [planted(70, 2, 256, 384), planted(71, 1, 128, 1024), planted(72, 1, 384, 128), planted(73, 3, 128, 128)]
+    xd = [x.to(dev) for x in xs]
+    for n in (1, 2, 4):
+        for wt in (False, True):
+            got = T.ops.quant_block_multi(xd[:n], with_transpose=wt)
+            for x, g, xo in zip(xd, got, xs):
+                want = T.ops.quant_block(x, clamp=True, with_transpose=wt)
+                assert len(g) == len(want) and all(bits_equal(a, b) for a, b in zip(g, want))
+                qo, so = obf.block_quant(xo, True)
+                assert bits_equal(g[0], qo) and bits_equal(g[-1], so)
+    with pytest.raises(ValueError):
+        T.ops.quant_block_multi([])
+    # the layer step with both activations at hand takes this path: same bits as forward + backward called separately
+    g = make_gen(74)
+    X, W, dY = randn_bf16(g, 384, 512).to(dev), randn_bf16(g, 256, 512, std=0.02).to(dev), randn_bf16(g, 384, 256, std=1e-3).to(dev)
+    Y, dX, dW = T.linear_fwd_bwd(X, W, dY, "block_channel")
+    Y0, saved = T.linear.linear_forward(X, W, "block_channel")
+    dX0, dW0 = T.linear.linear_backward(dY, X, W, "block_channel", None, saved)
+    assert torch.equal(Y, Y0) and torch.equal(dX, dX0) and torch.equal(dW, dW0)
+
+
 @pytest.mark.parametrize("cols", [128, 512, 1024, 2048, 4096, 6144, 14336, 32768])
 def test_row_quant_every_width(T, dev, cols):
     x = randn_bf16(make_gen(cols), 37, cols)

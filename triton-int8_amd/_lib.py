@@ -12,10 +12,18 @@ LIB_PATH = os.path.join(_HERE, "libti8.so")
 
 _i64, _int, _f32, _vp = ctypes.c_int64, ctypes.c_int, ctypes.c_float, ctypes.c_void_p
 
+class QBlockOperand(ctypes.Structure):
+    """ti8_qblock_operand of include/ti8.h."""
+    _fields_ = [("x", _vp), ("bsx", _i64), ("ldx", _i64), ("q", _vp), ("bsq", _i64), ("ldq", _i64),
+                ("qT", _vp), ("bsqt", _i64), ("ldqt", _i64), ("s", _vp), ("ssb", _i64), ("ssr", _i64), ("ssc", _i64),
+                ("B", _i64), ("R", _i64), ("C", _i64)]
+
+
 # name -> argument types, in the order of include/ti8.h
 PROTOTYPES = {
     "ti8_quant_block": [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _i64,
                         _i64, _i64, _i64, _int, _int, _int, _vp],
+    "ti8_quant_block_multi": [ctypes.POINTER(QBlockOperand), _int, _int, _int, _vp],
     "ti8_quant_block_had128": [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _int, _vp],
     "ti8_quant_row": [_vp, _i64, _vp, _i64, _vp, _i64, _i64, _int, _int, _int, _vp],
     "ti8_quant_col_t": [_vp, _i64, _vp, _i64, _vp, _vp, _i64, _i64, _int, _int, _vp],

@@ -206,14 +206,11 @@ __device__ __forceinline__ void transpose4x4_bytes(uint32_t r0, uint32_t r1, uin
 // transpose in registers for the optional transposed output (staged through LDS so
 // that the global writes of qT are 128-byte rows too).
 template <int NSUB, bool WRITE_Q, bool WRITE_QT, int ARITH = ARITH_KERNEL>
-__global__ __launch_bounds__(256) void quant_block_kernel(
+__device__ __forceinline__ void quant_block_tile(
     const uint16_t* __restrict__ x, int64_t bsx, int64_t ldx, int8_t* __restrict__ q, int64_t bsq, int64_t ldq,
     int8_t* __restrict__ qT, int64_t bsqt, int64_t ldqt, float* __restrict__ s, int64_t ssb, int64_t ssr,
-    int64_t ssc, int nrb, int ncb, QMode mode) {
-    __shared__ float red4[4];
-    __shared__ uint32_t tileT[WRITE_QT ? 128 * 33 : 1];
-
-    const idx::TileId tl = idx::qblock_tile(blockIdx.x, nrb, ncb);
+    int64_t ssc, int nrb, int ncb, const QMode& mode, int tile_index, float* red4, uint32_t* tileT) {
+    const idx::TileId tl = idx::qblock_tile(tile_index, nrb, ncb);
     const int b = tl.b, rb = tl.rb, cb = tl.cb;
 
     const int tid = threadIdx.x;
@@ -285,6 +282,52 @@ __global__ __launch_bounds__(256) void quant_block_kernel(
             }
         }
     }
+}
+
+
+template <int NSUB, bool WRITE_Q, bool WRITE_QT, int ARITH = ARITH_KERNEL>
+__global__ __launch_bounds__(256) void quant_block_kernel(
+    const uint16_t* __restrict__ x, int64_t bsx, int64_t ldx, int8_t* __restrict__ q, int64_t bsq, int64_t ldq,
+    int8_t* __restrict__ qT, int64_t bsqt, int64_t ldqt, float* __restrict__ s, int64_t ssb, int64_t ssr,
+    int64_t ssc, int nrb, int ncb, QMode mode) {
+    __shared__ float red4[4];
+    __shared__ uint32_t tileT[WRITE_QT ? 128 * 33 : 1];
+    quant_block_tile<NSUB, WRITE_Q, WRITE_QT, ARITH>(x, bsx, ldx, q, bsq, ldq, qT, bsqt, ldqt, s, ssb, ssr, ssc, nrb, ncb, mode,
+                                                     blockIdx.x, red4, tileT);
+}
+
+// Several operands in one launch (a training step quantises X and dY the same way: one launch
+// instead of two saves a kernel boundary and fills the tail of one operand with tiles of the next).
+// Workgroup w works on tile w - first[i] of the operand i whose range holds w.
+constexpr int QBLOCK_MULTI_MAX = 4;
+struct QBlockOperand {
+    const uint16_t* x;
+    int64_t bsx, ldx;
+    int8_t* q;
+    int64_t bsq, ldq;
+    int8_t* qT;
+    int64_t bsqt, ldqt;
+    float* s;
+    int64_t ssb, ssr, ssc;
+    int nrb, ncb;
+};
+struct QBlockMulti {
+    QBlockOperand op[QBLOCK_MULTI_MAX];
+    int first[QBLOCK_MULTI_MAX + 1];   // first workgroup of operand i; first[count] = grid size
+    int count;
+};
+
+template <bool WRITE_Q, bool WRITE_QT>
+__global__ __launch_bounds__(256) void quant_block_multi_kernel(const QBlockMulti m, QMode mode) {
+    __shared__ float red4[4];
+    __shared__ uint32_t tileT[WRITE_QT ? 128 * 33 : 1];
+    int i = 0;
+#pragma unroll
+    for (int k = 1; k < QBLOCK_MULTI_MAX; ++k)
+        if (k < m.count && (int)blockIdx.x >= m.first[k]) i = k;
+    const QBlockOperand& o = m.op[i];
+    quant_block_tile<1, WRITE_Q, WRITE_QT, ARITH_KERNEL>(o.x, o.bsx, o.ldx, o.q, o.bsq, o.ldq, o.qT, o.bsqt, o.ldqt, o.s, o.ssb, o.ssr,
+                                                         o.ssc, o.nrb, o.ncb, mode, (int)blockIdx.x - m.first[i], red4, tileT);
 }
 
 
@@ -716,6 +759,23 @@ static int parse_mode(int qflags, int inv_mode, QMode* m) {
 
 using namespace ti8;
 
+// argument checks of one block-quantiser operand (shared by ti8_quant_block and ti8_quant_block_multi)
+static int check_qblock_operand(const char* fn, const void* x, int64_t bsx, int64_t ldx, const int8_t* q, int64_t bsq, int64_t ldq,
+                                const int8_t* qT, int64_t bsqt, int64_t ldqt, const float* s, int64_t B, int64_t R, int64_t C, int group_c) {
+    if (!x || !s || (!q && !qT)) return fail(TI8_ERR_NULL, "%s: x, s and one of q/qT are required", fn);
+    if (group_c != 128 && group_c != 256) return fail(TI8_ERR_MODE, "%s: group_c must be 128 or 256, got %d", fn, group_c);
+    if (qT && group_c != 128) return fail(TI8_ERR_MODE, "%s: the transposed output needs group_c = 128", fn);
+    if (B <= 0 || R <= 0 || C <= 0 || R % 128 || C % group_c)
+        return fail(TI8_ERR_SHAPE, "%s: need B>0, R%%128==0, C%%%d==0; got B=%lld R=%lld C=%lld", fn, group_c,
+                    (long long)B, (long long)R, (long long)C);
+    if (ldx < C || (q && ldq < C) || (qT && ldqt < R)) return fail(TI8_ERR_SHAPE, "%s: leading dimension smaller than the row length", fn);
+    if (!aligned16(x) || (ldx % 8) || (bsx % 8) || (q && (!aligned16(q) || (ldq % 16) || (bsq % 16))) ||
+        (qT && (!aligned16(qT) || (ldqt % 16) || (bsqt % 16))))
+        return fail(TI8_ERR_ALIGN, "%s: pointers must be 16-byte aligned and strides multiples of 16 bytes", fn);
+    if (B * (R / 128) * (C / group_c) > 0x7fffffffLL) return fail(TI8_ERR_SHAPE, "%s: too many tiles", fn);
+    return TI8_OK;
+}
+
 extern "C" int ti8_quant_block(const void* x, int64_t bsx, int64_t ldx, int8_t* q, int64_t bsq, int64_t ldq,
                                int8_t* qT, int64_t bsqt, int64_t ldqt, float* s, int64_t ssb, int64_t ssr,
                                int64_t ssc, int64_t B, int64_t R, int64_t C, int group_c, int qflags,
@@ -727,18 +787,8 @@ extern "C" int ti8_quant_block(const void* x, int64_t bsx, int64_t ldx, int8_t* 
     if (arith != ARITH_KERNEL && (group_c != 128 || qT || (qflags & (TI8_Q_EPS_ADD | TI8_Q_SCALE_BF16)) || inv_mode != TI8_INV_RCP_OF_SCALE))
         return fail(TI8_ERR_MODE, "ti8_quant_block: the torch arithmetic goes with group_c = 128, q only, no other flag and TI8_INV_RCP_OF_SCALE");
     if (qflags & TI8_Q_HAD128) return fail(TI8_ERR_MODE, "ti8_quant_block: use ti8_quant_block_had128 for the Hadamard rotation");
-    if (!x || !s || (!q && !qT)) return fail(TI8_ERR_NULL, "ti8_quant_block: x, s and one of q/qT are required");
-    if (group_c != 128 && group_c != 256) return fail(TI8_ERR_MODE, "ti8_quant_block: group_c must be 128 or 256, got %d", group_c);
-    if (qT && group_c != 128) return fail(TI8_ERR_MODE, "ti8_quant_block: the transposed output needs group_c = 128");
-    if (B <= 0 || R <= 0 || C <= 0 || R % 128 || C % group_c)
-        return fail(TI8_ERR_SHAPE, "ti8_quant_block: need B>0, R%%128==0, C%%%d==0; got B=%lld R=%lld C=%lld", group_c,
-                    (long long)B, (long long)R, (long long)C);
-    if (ldx < C || (q && ldq < C) || (qT && ldqt < R)) return fail(TI8_ERR_SHAPE, "ti8_quant_block: leading dimension smaller than the row length");
-    if (!aligned16(x) || (ldx % 8) || (bsx % 8) || (q && (!aligned16(q) || (ldq % 16) || (bsq % 16))) ||
-        (qT && (!aligned16(qT) || (ldqt % 16) || (bsqt % 16))))
-        return fail(TI8_ERR_ALIGN, "ti8_quant_block: pointers must be 16-byte aligned and strides multiples of 16 bytes");
+    if (int e = check_qblock_operand("ti8_quant_block", x, bsx, ldx, q, bsq, ldq, qT, bsqt, ldqt, s, B, R, C, group_c)) return e;
     const int64_t ntiles = B * (R / 128) * (C / group_c);
-    if (ntiles > 0x7fffffffLL) return fail(TI8_ERR_SHAPE, "ti8_quant_block: too many tiles");
     hipStream_t st = static_cast<hipStream_t>(stream);
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     const int nrb = (int)(R / 128), ncb = (int)(C / group_c);
@@ -756,6 +806,38 @@ extern "C" int ti8_quant_block(const void* x, int64_t bsx, int64_t ldx, int8_t* 
     else TI8_LAUNCH_QB(1, false, true);
 #undef TI8_LAUNCH_QB
     return check_launch("ti8_quant_block");
+}
+
+extern "C" int ti8_quant_block_multi(const ti8_qblock_operand* operands, int count, int qflags, int inv_mode, ti8_stream_t stream) {
+    const char* fn = "ti8_quant_block_multi";
+    QMode mode;
+    if (int e = parse_mode(qflags, inv_mode, &mode)) return e;
+    if (qflags & TI8_Q_HAD128) return fail(TI8_ERR_MODE, "%s: the Hadamard rotation is not offered here", fn);
+    if (!operands) return fail(TI8_ERR_NULL, "%s: operands is required", fn);
+    if (count < 1 || count > QBLOCK_MULTI_MAX) return fail(TI8_ERR_SHAPE, "%s: between 1 and %d operands, got %d", fn, QBLOCK_MULTI_MAX, count);
+    QBlockMulti m;
+    int64_t total = 0;
+    for (int i = 0; i < count; ++i) {
+        const ti8_qblock_operand& o = operands[i];
+        if (int e = check_qblock_operand(fn, o.x, o.bsx, o.ldx, o.q, o.bsq, o.ldq, o.qT, o.bsqt, o.ldqt, o.s, o.B, o.R, o.C, 128)) return e;
+        if ((o.q != nullptr) != (operands[0].q != nullptr) || (o.qT != nullptr) != (operands[0].qT != nullptr))
+            return fail(TI8_ERR_MODE, "%s: every operand must ask for the same outputs (q, qT or both)", fn);
+        m.op[i] = QBlockOperand{static_cast<const uint16_t*>(o.x), o.bsx, o.ldx, o.q, o.bsq, o.ldq, o.qT, o.bsqt, o.ldqt, o.s,
+                                o.ssb, o.ssr, o.ssc, (int)(o.R / 128), (int)(o.C / 128)};
+        m.first[i] = (int)total;
+        total += o.B * (o.R / 128) * (o.C / 128);
+        if (total > 0x7fffffffLL) return fail(TI8_ERR_SHAPE, "%s: too many tiles", fn);
+    }
+    for (int i = count; i < QBLOCK_MULTI_MAX; ++i) { m.op[i] = m.op[0]; m.first[i] = (int)total; }
+    m.first[QBLOCK_MULTI_MAX] = (int)total;
+    m.count = count;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    dim3 grid((unsigned)total), block(256);
+    const bool wq = operands[0].q != nullptr, wqt = operands[0].qT != nullptr;
+    if (wq && wqt) hipLaunchKernelGGL((quant_block_multi_kernel<true, true>), grid, block, 0, st, m, mode);
+    else if (wq) hipLaunchKernelGGL((quant_block_multi_kernel<true, false>), grid, block, 0, st, m, mode);
+    else hipLaunchKernelGGL((quant_block_multi_kernel<false, true>), grid, block, 0, st, m, mode);
+    return check_launch(fn);
 }
 
 extern "C" int ti8_quant_row(const void* x, int64_t ldx, int8_t* q, int64_t ldq, float* s, int64_t rows,

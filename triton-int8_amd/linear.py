@@ -100,13 +100,14 @@ def quantize_weight(W, scheme="block_channel", hadamard=None):
     return ops.quant_row(ops.fwht(W) if hadamard == "full" else W, clamp=True, inv_mode=INV_AMAX_DIV_127)
 
 
-def linear_forward(X2, W, scheme="block_channel", hadamard=None, need_backward=True, wq=None, tokens=None):
+def linear_forward(X2, W, scheme="block_channel", hadamard=None, need_backward=True, wq=None, tokens=None, xq=None):
     """X2 bf16 [T, K] (tokens flattened), W bf16 [N, K] -> (Y bf16 [T, N], saved) where
     ``saved`` holds what the backward can reuse: operands the forward quantises anyway are
     quantised for the backward GEMMs in the same pass (transposed copies, column-wise scales)
     unless ``need_backward`` is false.  ``wq`` = :func:`quantize_weight` of W computed earlier
     (forward-only use; W itself is then not read).  ``tokens`` = number of real rows of X2 when the
-    caller has zero-padded it: with few tokens the GEMM skips the padding rows."""
+    caller has zero-padded it: with few tokens the GEMM skips the padding rows.  ``xq`` = ``(q, qT, s)`` of
+    ``ops.quant_block(X2[None], with_transpose=True)`` computed earlier ("block_channel" without rotation only)."""
     _check(scheme, hadamard)
     saved = {}
     if wq is not None and need_backward:
@@ -120,7 +121,7 @@ def linear_forward(X2, W, scheme="block_channel", hadamard=None, need_backward=T
             q, s = ops.quant_block(X2[None], clamp=True)
             wq, ws = wq if wq is not None else quantize_weight(W, scheme, hadamard)
             return _gemm_bc(q[0], s[0], SCALE_BLOCK128, wq, ws, SCALE_ROW, tokens=tokens), saved
-        q, qT, s = ops.quant_block(X2[None], clamp=True, with_transpose=True)
+        q, qT, s = xq if xq is not None else ops.quant_block(X2[None], clamp=True, with_transpose=True)
         saved["XqT"], saved["Xs"] = qT[0], s[0]
         wq, ws, saved["WtQ"], saved["Wts"] = _row_col(W, clamp=True)   # rows for Y, columns for dX
         return _gemm_bc(q[0], s[0], SCALE_BLOCK128, wq, ws, SCALE_ROW, tokens=tokens), saved
@@ -161,7 +162,7 @@ def linear_backward(dY2, X2, W, scheme="block_channel", hadamard=None, saved=Non
             dW = ops.gemm_i8_nt(dyt, xt, dyts.transpose(1, 2), SCALE_BLOCK128, xts.transpose(1, 2), SCALE_BLOCK128,
                                 out_scale=2.0 ** -7)[0]
             return dX, dW
-        dq, dqT, ds = ops.quant_block(dY2[None], clamp=True, with_transpose=True)
+        dq, dqT, ds = saved["dYq"] if "dYq" in saved else ops.quant_block(dY2[None], clamp=True, with_transpose=True)
         if "WtQ" in saved:
             wtq, wts = saved["WtQ"], saved["Wts"]
         else:
@@ -240,7 +241,14 @@ def linear_fwd_bwd(X, W, dY, scheme="block_channel", hadamard=None):
     X2, dY2 = X.reshape(-1, K), dY.reshape(-1, N)
     T = X2.shape[0]
     X2, dY2 = pad_tokens(X2), pad_tokens(dY2)
-    Y, saved = linear_forward(X2, W, scheme, hadamard, tokens=T)
+    pre = None
+    if scheme == "block_channel" and hadamard is None:
+        # both activations are at hand: one quantiser launch for X and dY (the forward alone would quantise X, the
+        # backward dY, with the same kernel and the same bits)
+        pre = ops.quant_block_multi([X2[None], dY2[None]], clamp=True, with_transpose=True)
+    Y, saved = linear_forward(X2, W, scheme, hadamard, tokens=T, xq=pre[0] if pre else None)
+    if pre:
+        saved["dYq"] = pre[1]
     dX, dW = linear_backward(dY2, X2, W, scheme, hadamard, saved, tokens=T)
     return Y[:T].reshape(*lead, N), dX[:T].reshape(*lead, K), dW
 

@@ -16,7 +16,7 @@ from ._lib import (COMBINE_DIV_PROD, COMBINE_MUL_MUL, COMBINE_MUL_PROD, GEMM_LAR
                    Q_WS_PINGPONG, Q_WS_SECOND,
                    SCALE_BLOCK128, SCALE_BLOCK_K256, SCALE_ROW, SCALE_ROW_K128)
 
-__all__ = ["quant_block", "quant_block_had128", "quant_row", "quant_col_t", "quant_row_col_t", "fwht", "gemm_i8_nt", "gemm_i8_nt_i32"]
+__all__ = ["quant_block", "quant_block_multi", "quant_block_had128", "quant_row", "quant_col_t", "quant_row_col_t", "fwht", "gemm_i8_nt", "gemm_i8_nt_i32"]
 
 
 # Which GEMM kernel `gemm_i8_nt` asks for: "auto" (the few-rows kernel for M <= 256, else an
@@ -111,6 +111,32 @@ def quant_block(x, *, clamp=True, group_c=128, eps_add=False, scale_bf16=False, 
         q = qct if out == "contiguous" else qc.transpose(1, 2)
         qT = qc  # canonical orientation IS the logical transpose
     return (q, qT, s) if with_transpose else (q, s)
+
+
+def quant_block_multi(xs, *, clamp=True, with_transpose=False, inv_mode=INV_RCP_OF_SCALE):
+    """``quant_block`` of several row-major operands [B, M, N] (up to 4) in ONE launch: a list of
+    ``(q, s)`` or ``(q, qT, s)``, bit-identical to separate calls.  A training step that has X and dY
+    at hand quantises both this way."""
+    _need(1 <= len(xs) <= 4, "between 1 and 4 operands")
+    descs, outs = (_lib.QBlockOperand * len(xs))(), []
+    for i, x in enumerate(xs):
+        _check_bf16(x, "x")
+        _need(x.dim() == 3 and x.numel() > 0, "every operand must be a non-empty [B, M, N] tensor")
+        B, M, N = x.shape
+        _need(M % 128 == 0 and N % 128 == 0, f"block quantisation needs M % 128 == 0 and N % 128 == 0, got M={M} N={N}")
+        if x.stride(2) != 1 or (B > 1 and x.stride(0) % 8) or x.stride(1) % 8 or x.data_ptr() % 16:
+            x = x.contiguous()
+        q = torch.empty((B, M, N), dtype=torch.int8, device=x.device)
+        qT = torch.empty((B, N, M), dtype=torch.int8, device=x.device) if with_transpose else None
+        s = torch.empty((B, M // 128, N // 128), dtype=torch.float32, device=x.device)
+        descs[i] = _lib.QBlockOperand(x.data_ptr(), x.stride(0), x.stride(1), q.data_ptr(), M * N, N,
+                                      qT.data_ptr() if with_transpose else None, M * N, M,
+                                      s.data_ptr(), s.stride(0), s.stride(1), s.stride(2), B, M, N)
+        outs.append((q, qT, s) if with_transpose else (q, s))
+        xs = list(xs)
+        xs[i] = x     # keep a contiguous copy alive until the launch is queued
+    _lib.call("ti8_quant_block_multi", descs, len(xs), _qflags(clamp, False, False), inv_mode, _stream())
+    return outs
 
 
 def quant_block_had128(x, *, along_rows=False, clamp=True, inv_mode=INV_RCP_OF_SCALE):
