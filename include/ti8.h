@@ -235,6 +235,15 @@ int ti8_quant_row_col_t_noalloc(const void* x, int64_t ldx, int8_t* q, int64_t l
 int ti8_fwht(const void* x, int64_t ldx, void* y, int64_t ldy,
              int64_t rows, int64_t cols, int64_t n, float scale, ti8_stream_t stream);
 
+/* The same transform of x^T along its rows, without materialising x^T: x bf16 [R][C] (ldx) ->
+ * y bf16 [C][R] (ldy), y[c][:] = FWHT_R(x[:, c]) * scale, bit-identical to ti8_fwht on the
+ * transposed copy.  Serves the transposed operands of the backward GEMMs (dX = fwd_32(dY, W^T),
+ * dW = bwd_33(dY^T, X^T)) when the scheme rotates along the full contraction dim
+ * (triton/double-channle_fwd32.py:299-300 applied to W^T, dY^T, X^T).
+ * R a power of two, 128 <= R <= 32768; C % 8 == 0; not in place. */
+int ti8_fwht_t(const void* x, int64_t ldx, void* y, int64_t ldy,
+               int64_t R, int64_t C, float scale, ti8_stream_t stream);
+
 /* ---------------------------------------------------------------------------------
  * INT8 NT GEMM with fused dequantising epilogue, C[b] = dequant(A[b] * B[b]^T):
  * replaces triton_gemm + int8_gemm_kernel of every scheme

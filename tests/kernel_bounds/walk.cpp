@@ -98,6 +98,78 @@ int walk_fwht(int64_t ldx, int64_t ldy, int64_t rows, int64_t cols, int64_t n, i
     return r.bad;
 }
 
+// ti8_fwht_t -> fwht_t_kernel<NT, W> (fwht.hip): x bf16 [R][C] (ldx) -> y bf16 [C][R] (ldy)
+int walk_fwht_t(int64_t ldx, int64_t ldy, int64_t R, int64_t C, int64_t x_elems, int64_t y_elems, int64_t lds_bytes_limit,
+                int64_t* n_checked, char* msg, int msglen) {
+    Report r{msg, msglen};
+    if (!fwht_t_direct(R, C)) {
+        // transpose_bf16_kernel: 64 x 64 tiles, thread t reads 8 columns of rows t/8 and t/8 + 32 and writes 8 rows
+        // of columns t/8 and t/8 + 32; then fwht_kernel in place on y [C][R]
+        const int tiles_c = (int)(C / 64);
+        for (int64_t block = 0; block < (R / 64) * (C / 64) && !r.bad; ++block) {
+            const int64_t tc = block % tiles_c, tr = block / tiles_c;
+            for (int tid = 0; tid < 256; ++tid)
+                for (int h = 0; h < 2; ++h) {
+                    const int a = (tid >> 3) + 32 * h, b = (tid & 7) * 8;
+                    r.access("fwht_t transpose x", (tr * 64 + a) * ldx + tc * 64 + b, 8, x_elems, block, tid, h);
+                    r.access("fwht_t transpose y", (tc * 64 + a) * ldy + tr * 64 + b, 8, y_elems, block, tid, h);
+                }
+        }
+        int64_t n2 = 0;
+        const int bad = r.bad ? 1 : walk_fwht(ldy, ldy, C, R, R, y_elems, y_elems, lds_bytes_limit, &n2, msg, msglen);
+        *n_checked = r.checked + n2;
+        return bad;
+    }
+    const int W = fwht_t_cols_per_wg(R);
+    const int NT = (int64_t)W * R >= 16384 ? 1024 : 256;
+    const int64_t nblocks = C / W;
+    const int64_t Lp = fwht_lds_words(R), lds_words = (int64_t)W * Lp;
+    if (C % W) r.fail("fwht_t: %lld columns are not a multiple of %d per workgroup", (long long)C, W);
+    if (lds_words * 4 > lds_bytes_limit) r.fail("fwht_t: %lld bytes of LDS requested, limit %lld", (long long)(lds_words * 4), (long long)lds_bytes_limit);
+    int logn = 0;
+    while ((1LL << logn) < R) ++logn;
+    // LDS indices (the same for every workgroup)
+    for (int tid = 0; tid < NT && !r.bad; ++tid) {
+        for (int row = tid; row < R; row += NT)
+            for (int w = 0; w < W; ++w) r.access("fwht_t lds fill", w * Lp + fwht_padded(row), 1, lds_words, tid, row, w);
+        auto pass = [&](int p, int rb) {   // pass_in_lds_segments<RB, NT>
+            const int per_seg = (int)(R >> rb);
+            for (int vt = tid; vt < W * per_seg; vt += NT) {
+                const int base = fwht_group_base(vt % per_seg, p, rb);
+                for (int e = 0; e < (1 << rb); ++e)
+                    r.access("fwht_t lds pass", (vt / per_seg) * Lp + fwht_padded(base + (e << p)), 1, lds_words, tid, vt, e, p);
+            }
+        };
+        pass(0, 4);
+        pass(4, imin(4, logn - 4));
+        int rem = logn - 8;
+        if (rem > 0) {
+            const int rb2 = rem <= 5 ? rem : (rem + 1) / 2;
+            pass(8, rb2);
+            rem -= rb2;
+            if (rem > 0) pass(8 + rb2, rem);
+        }
+        const int per_seg = (int)(R >> 3);
+        for (int i = tid; i < W * per_seg; i += NT) r.access("fwht_t lds read-back", (i / per_seg) * Lp + fwht_padded((i % per_seg) * 8), 8, lds_words, tid, i);
+    }
+    std::vector<uint8_t> seen((size_t)nblocks, 0);
+    for (int64_t block = 0; block < nblocks && !r.bad; ++block) {
+        const int64_t cb = fwht_t_colblock(block, nblocks, W);
+        if (cb < 0 || cb >= nblocks) { r.fail("fwht_t: workgroup %lld maps to column block %lld of %lld", (long long)block, (long long)cb, (long long)nblocks); break; }
+        ++seen[(size_t)cb];
+        const int64_t c0 = cb * W;
+        for (int tid = 0; tid < NT; ++tid) {
+            for (int row = tid; row < R; row += NT) r.access("fwht_t x", (int64_t)row * ldx + c0, W, x_elems, block, tid, row);
+            const int per_seg = (int)(R >> 3);
+            for (int i = tid; i < W * per_seg; i += NT) r.access("fwht_t y", (c0 + i / per_seg) * ldy + (int64_t)(i % per_seg) * 8, 8, y_elems, block, tid, i);
+        }
+    }
+    for (int64_t cb = 0; cb < nblocks && !r.bad; ++cb)
+        if (seen[(size_t)cb] != 1) r.fail("fwht_t: column block %lld is transformed %d times", (long long)cb, (int)seen[(size_t)cb]);
+    *n_checked = r.checked;
+    return r.bad;
+}
+
 // ti8_quant_row -> quant_row_kernel<NLOAD, WG_ROW, GROUP16, HAD> (quant.hip)
 int walk_quant_row(int64_t ldx, int64_t ldq, int64_t rows, int64_t cols, int group, int64_t x_elems, int64_t q_elems,
                    int64_t s_elems, int64_t* n_checked, char* msg, int msglen) {

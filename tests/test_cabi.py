@@ -81,6 +81,10 @@ FAKE = 0x10000  # a 16-byte aligned non-null "device pointer"; validation never 
     (("ti8_quant_row_col_t_noalloc", FAKE, 256, FAKE, 256, FAKE, FAKE, 128, FAKE, 128, 256, 16, 0, None), 4, "workspace flags"),
     (("ti8_fwht", FAKE, 384, FAKE, 384, 4, 384, 384, 1.0, None), 2, "power of two"),
     (("ti8_fwht", FAKE, 256, FAKE, 256, 4, 256, 64, 1.0, None), 2, "power of two"),
+    (("ti8_fwht_t", FAKE, 256, FAKE + 0x100000, 384, 384, 256, 1.0, None), 2, "power of two"),
+    (("ti8_fwht_t", FAKE, 260, FAKE + 0x100000, 256, 256, 260, 1.0, None), 2, "C % 8"),
+    (("ti8_fwht_t", FAKE, 256, FAKE, 256, 256, 256, 1.0, None), 4, "in place"),
+    (("ti8_fwht_t", FAKE, 256, FAKE + 0x100000, 128, 256, 256, 1.0, None), 2, "leading dimension"),
     (("ti8_gemm_i8_nt", FAKE, 0, 128, FAKE, 0, 128, FAKE, 0, 128, FAKE, 0, 0, 1, 0, FAKE, 0, 0, 1, 0,
       1, 128, 128, 100, 0, 0, 1.0, 0.0, 0, None), 2, "multiples of 128"),
     (("ti8_gemm_i8_nt", FAKE, 0, 128, FAKE, 0, 128, FAKE, 0, 128, None, 0, 0, 1, 0, FAKE, 0, 0, 1, 0,

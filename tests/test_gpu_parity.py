@@ -246,6 +246,24 @@ def test_fwht(T, dev, n, cols):
         assert bits_equal(T.double_channel_fwd32.hadamard_transform(x.to(dev)), ohad.hadamard_transform(x))
 
 
+@pytest.mark.parametrize("R,C", [(128, 8), (128, 520), (256, 512), (1024, 1024), (2048, 72), (4096, 512), (8192, 1024),
+                                 (16384, 96), (32768, 64), (512, 4096)])
+def test_fwht_of_the_transpose(T, dev, R, C):
+    """ti8_fwht_t: the transform along the ROWS of x with transposed output = ti8_fwht of the transposed
+    copy, bit for bit, and equal to the oracle's butterflies on x^T; with and without the sibling
+    workgroups' XCD grouping (column counts that are and are not multiples of 8 x 64)."""
+    x = randn_bf16(make_gen(R * 7 + C), R, C)
+    xd = x.to(dev)
+    y = T.ops.fwht_t(xd)
+    assert y.shape == (C, R) and torch.equal(y, T.ops.fwht(xd.t().contiguous()))
+    assert bits_equal(y, ohad.fwht_f32(x.t().contiguous().float(), R).to(torch.bfloat16))
+    ys = T.ops.fwht_t(xd, scale=1.0 / R)
+    assert torch.equal(ys, T.ops.fwht(xd.t().contiguous(), None, 1.0 / R))
+    wide = torch.zeros(R, C + 24, dtype=torch.bfloat16, device=dev)      # a strided view: leading dimension > C
+    wide[:, 8:8 + C] = xd
+    assert torch.equal(T.ops.fwht_t(wide[:, 8:8 + C]), y)
+
+
 def test_fused_hadamard_quantisers(T, dev):
     """H_128 fused into the quantisers equals the un-fused oracle (rotate, round to bf16, quantise)."""
     x = planted(20, 2, 256, 384)

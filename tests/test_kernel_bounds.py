@@ -37,6 +37,7 @@ def walker(tmp_path_factory):
     i64, ci, cp = ctypes.c_int64, ctypes.c_int, ctypes.c_char_p
     p64 = ctypes.POINTER(ctypes.c_int64)
     lib.walk_fwht.argtypes = [i64] * 8 + [p64, cp, ci]
+    lib.walk_fwht_t.argtypes = [i64] * 7 + [p64, cp, ci]
     lib.walk_quant_row.argtypes = [i64] * 4 + [ci] + [i64] * 3 + [p64, cp, ci]
     lib.walk_quant_block.argtypes = [i64, i64, ci, i64, i64, ci, i64, i64, i64, i64, i64, i64, i64, i64, ci, i64, i64, i64, i64, p64, cp, ci]
     lib.walk_gemm.argtypes = [i64] * 6 + [ctypes.POINTER(ScaleArg)] * 2 + [i64] * 4 + [ci] * 5 + [i64] * 3 + [ctypes.POINTER(ci), p64, cp, ci]
@@ -88,6 +89,9 @@ def walk(lib, allocs, name, a):
     if name == "ti8_fwht":
         x, ldx, y, ldy, rows, cols, nn = a[:7]
         rc = lib.walk_fwht(ldx, ldy, rows, cols, nn, allocs.room(x, 2), allocs.room(y, 2), LDS_LIMIT, ctypes.byref(n), msg, 512)
+    elif name == "ti8_fwht_t":
+        x, ldx, y, ldy, R, C = a[:6]
+        rc = lib.walk_fwht_t(ldx, ldy, R, C, allocs.room(x, 2), allocs.room(y, 2), LDS_LIMIT, ctypes.byref(n), msg, 512)
     elif name == "ti8_quant_row":
         x, ldx, q, ldq, s, rows, cols, group = a[:8]
         rc = lib.walk_quant_row(ldx, ldq, rows, cols, group, allocs.room(x, 2), allocs.room(q, 1), allocs.room(s, 4), ctypes.byref(n), msg, 512)
@@ -187,3 +191,18 @@ def test_gemm_launch_geometries(walker, M, N, K, batch, mA, mB, acc, flags):
     rc = walker.walk_gemm(M * K, K, 0, K, M * N, N, ctypes.byref(sa), ctypes.byref(sb), batch, M, N, K, acc, flags & 1, (flags >> 3) & 1, 0,
                           NUM_CU, batch * M * K, N * K, batch * M * N, picked, ctypes.byref(n), msg, 512)
     assert rc == 0, msg.value.decode()
+
+
+@pytest.mark.parametrize("R,C", [(128, 8), (128, 520), (2048, 72), (4096, 512), (8192, 1024), (16384, 2048), (32768, 4096), (32768, 64),
+                                 (16384, 96)])
+def test_transposed_hadamard_launches(walker, recorded, R, C):
+    """ti8_fwht_t as ops.fwht_t launches it: every read of x, every LDS index and every write of y in
+    bounds, and the XCD-aware column-block map a bijection (with and without the sibling grouping)."""
+    T, allocs, calls = recorded
+    y = T.ops.fwht_t(torch.empty(R, C, dtype=torch.bfloat16))
+    assert tuple(y.shape) == (C, R) and [c[0] for c in calls] == ["ti8_fwht_t"]
+    assert walk(walker, allocs, *calls[0]) > R * C // 8
+    msg = ctypes.create_string_buffer(512)
+    n = ctypes.c_int64(0)
+    assert walker.walk_fwht_t(C, R, R, C, R * C - 1, R * C, LDS_LIMIT, ctypes.byref(n), msg, 512) == 1 and msg.value.split(b":")[0].endswith(b" x")
+    assert walker.walk_fwht_t(C, R, R, C, R * C, R * C - 8, LDS_LIMIT, ctypes.byref(n), msg, 512) == 1 and msg.value.split(b":")[0].endswith(b" y")

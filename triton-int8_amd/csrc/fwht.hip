@@ -120,9 +120,181 @@ __global__ __launch_bounds__(NT) void fwht_kernel(const uint16_t* __restrict__ x
     }
 }
 
+// ---- transposed input: y[c][r] = sum_r' H[r][r'] x[r'][c], i.e. the transform of x^T along its
+// rows without materialising x^T.  A workgroup owns W columns of x (W = 8, 4, 2, 1 as the length R
+// grows: W * R fp32 elements must fit in LDS), reads them row by row -- W bf16 = 2 W bytes per row;
+// the other columns of the same 128-byte lines belong to the sibling workgroups that the block map
+// keeps together on one XCD -- and lays them out in LDS as W segments of R elements in the padded
+// layout of the kernel above, after which the butterfly passes are those of the kernel above
+// applied to every segment (bits 0..3 first, from LDS here), and each segment leaves as one
+// contiguous row of y.  Same butterfly order, same single rounding: bit-identical to
+// ti8_fwht(transpose(x)).
+template <int RB, int NT>
+__device__ __forceinline__ void pass_in_lds_segments(float* lds, int L, int Lp, int W, int p, int tid) {
+    constexpr int RAD = 1 << RB;
+    const int per_seg = L >> RB;
+    for (int vt = tid; vt < W * per_seg; vt += NT) {
+        float* seg = lds + (vt / per_seg) * Lp;
+        const int base = idx::fwht_group_base(vt % per_seg, p, RB);
+        float a[RAD];
+#pragma unroll
+        for (int e = 0; e < RAD; ++e) a[e] = seg[padded(base + (e << p))];
+        butterflies<RB>(a);
+#pragma unroll
+        for (int e = 0; e < RAD; ++e) seg[padded(base + (e << p))] = a[e];
+    }
+}
+
+template <int NT>
+__device__ __forceinline__ void pass_dispatch_segments(float* lds, int L, int Lp, int W, int p, int rb, int tid) {
+    switch (rb) {
+        case 5: pass_in_lds_segments<5, NT>(lds, L, Lp, W, p, tid); break;
+        case 4: pass_in_lds_segments<4, NT>(lds, L, Lp, W, p, tid); break;
+        case 3: pass_in_lds_segments<3, NT>(lds, L, Lp, W, p, tid); break;
+        case 2: pass_in_lds_segments<2, NT>(lds, L, Lp, W, p, tid); break;
+        default: pass_in_lds_segments<1, NT>(lds, L, Lp, W, p, tid); break;
+    }
+}
+
+template <int W> struct ColumnLoad;
+template <> struct ColumnLoad<8> { typedef uint4 type; };
+template <> struct ColumnLoad<4> { typedef uint2 type; };
+template <> struct ColumnLoad<2> { typedef uint32_t type; };
+template <> struct ColumnLoad<1> { typedef uint16_t type; };
+
+template <int NT, int W>
+__global__ __launch_bounds__(NT) void fwht_t_kernel(const uint16_t* __restrict__ x, int64_t ldx, uint16_t* __restrict__ y,
+                                                     int64_t ldy, int R, int logn, int64_t nblocks, float scale) {
+    extern __shared__ float lds[];
+    const int tid = threadIdx.x;
+    const int L = R, Lp = (int)idx::fwht_lds_words(R);
+    const int64_t c0 = idx::fwht_t_colblock(blockIdx.x, nblocks, W) * W;
+    typedef typename ColumnLoad<W>::type load_t;
+    for (int r = tid; r < R; r += NT) {
+        const load_t v = *reinterpret_cast<const load_t*>(x + (int64_t)r * ldx + c0);
+        uint16_t h[W];
+        __builtin_memcpy(h, &v, sizeof(v));
+#pragma unroll
+        for (int w = 0; w < W; ++w) lds[w * Lp + padded(r)] = __uint_as_float((uint32_t)h[w] << 16);
+    }
+    __syncthreads();
+    pass_in_lds_segments<4, NT>(lds, L, Lp, W, 0, tid);   // bits 0..3 (R >= 128)
+    __syncthreads();
+    const int rb1 = min(4, logn - 4);
+    pass_dispatch_segments<NT>(lds, L, Lp, W, 4, rb1, tid);
+    __syncthreads();
+    int rem = logn - 8;
+    if (rem > 0) {
+        const int rb2 = rem <= 5 ? rem : (rem + 1) / 2;
+        pass_dispatch_segments<NT>(lds, L, Lp, W, 8, rb2, tid);
+        __syncthreads();
+        rem -= rb2;
+        if (rem > 0) {
+            pass_dispatch_segments<NT>(lds, L, Lp, W, 8 + rb2, rem, tid);
+            __syncthreads();
+        }
+    }
+    const int per_seg = L >> 3;
+    for (int i = tid; i < W * per_seg; i += NT) {
+        const int w = i / per_seg, c = i % per_seg;
+        const float* src = lds + w * Lp + padded(c * 8);   // 8 words of one 16-word run: contiguous
+        float f[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) f[e] = src[e];
+        if (scale != 1.0f) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) f[e] = f[e] * scale;
+        }
+        uint4 o;
+        o.x = pack_bf16x2(f[0], f[1]);
+        o.y = pack_bf16x2(f[2], f[3]);
+        o.z = pack_bf16x2(f[4], f[5]);
+        o.w = pack_bf16x2(f[6], f[7]);
+        *reinterpret_cast<uint4*>(y + (c0 + w) * ldy + c * 8) = o;
+    }
+}
+
+// bf16 transpose, 64 x 64 tiles through LDS: x [R][C] -> y [C][R], 16-byte loads and stores.
+// Thread t reads 8 consecutive columns of row (t / 8) + 32 h; the tile is kept as 32-bit words of
+// two ROWS' elements so that a thread later picks up 8 consecutive rows of one column with 4 reads.
+__global__ __launch_bounds__(256) void transpose_bf16_kernel(const uint16_t* __restrict__ x, int64_t ldx, uint16_t* __restrict__ y,
+                                                             int64_t ldy, int tiles_c) {
+    __shared__ uint16_t tile[64][64 + 2];   // +2: rows 4 bytes apart modulo the banks
+    const int tc = blockIdx.x % tiles_c, tr = blockIdx.x / tiles_c;
+    const int tid = threadIdx.x;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int r = (tid >> 3) + 32 * h, c = (tid & 7) * 8;
+        const uint4 v = *reinterpret_cast<const uint4*>(x + ((int64_t)tr * 64 + r) * ldx + (int64_t)tc * 64 + c);
+        uint16_t e[8];
+        __builtin_memcpy(e, &v, 16);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) tile[c + k][r] = e[k];   // transposed in LDS: tile[column][row]
+    }
+    __syncthreads();
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int c = (tid >> 3) + 32 * h, r = (tid & 7) * 8;   // row c of y's tile = column c of x's tile
+        uint16_t e[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) e[k] = tile[c][r + k];
+        uint4 v;
+        __builtin_memcpy(&v, e, 16);
+        *reinterpret_cast<uint4*>(y + ((int64_t)tc * 64 + c) * ldy + (int64_t)tr * 64 + r) = v;
+    }
+}
+
 }  // namespace ti8
 
 using namespace ti8;
+
+template <int NT, int W>
+static int launch_fwht_t(const void* x, int64_t ldx, void* y, int64_t ldy, int64_t R, int64_t C, int logn, float scale, hipStream_t st) {
+    const size_t shmem = (size_t)W * idx::fwht_lds_words(R) * sizeof(float);
+    auto kern = fwht_t_kernel<NT, W>;
+    if (shmem > 64 * 1024) {
+        static thread_local int attr_dev = -1;
+        int dev = 0;
+        (void)hipGetDevice(&dev);
+        if (attr_dev != dev) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 136 * 1024);
+            if (e != hipSuccess) return fail(TI8_ERR_HIP, "ti8_fwht_t: cannot raise the LDS limit: %s", hipGetErrorString(e));
+            attr_dev = dev;
+        }
+    }
+    const int64_t nblocks = C / W;
+    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(NT), shmem, st, static_cast<const uint16_t*>(x), ldx,
+                       static_cast<uint16_t*>(y), ldy, (int)R, logn, nblocks, scale);
+    return check_launch("ti8_fwht_t");
+}
+
+extern "C" int ti8_fwht_t(const void* x, int64_t ldx, void* y, int64_t ldy, int64_t R, int64_t C, float scale, ti8_stream_t stream) {
+    if (!x || !y) return fail(TI8_ERR_NULL, "ti8_fwht_t: x and y are required");
+    if (R < 128 || R > 32768 || (R & (R - 1))) return fail(TI8_ERR_SHAPE, "ti8_fwht_t: R must be a power of two in [128, 32768], got %lld", (long long)R);
+    if (C <= 0 || C % 8) return fail(TI8_ERR_SHAPE, "ti8_fwht_t: need C > 0 and C %% 8 == 0; got C=%lld", (long long)C);
+    if (x == y) return fail(TI8_ERR_MODE, "ti8_fwht_t: the transform cannot run in place");
+    if (ldx < C || ldy < R) return fail(TI8_ERR_SHAPE, "ti8_fwht_t: leading dimension smaller than the row length");
+    if (!aligned16(x) || !aligned16(y) || (ldx % 8) || (ldy % 8)) return fail(TI8_ERR_ALIGN, "ti8_fwht_t: pointers must be 16-byte aligned and strides multiples of 16 bytes");
+    if (C / 1 > 0x7fffffffLL) return fail(TI8_ERR_SHAPE, "ti8_fwht_t: too many columns");
+    int logn = 0;
+    while ((1LL << logn) < R) ++logn;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (idx::fwht_t_direct(R, C)) {
+        switch (idx::fwht_t_cols_per_wg(R)) {
+            case 8: return R * 8 >= 16384 ? launch_fwht_t<1024, 8>(x, ldx, y, ldy, R, C, logn, scale, st)
+                                          : launch_fwht_t<256, 8>(x, ldx, y, ldy, R, C, logn, scale, st);
+            case 4: return launch_fwht_t<1024, 4>(x, ldx, y, ldy, R, C, logn, scale, st);
+            case 2: return launch_fwht_t<1024, 2>(x, ldx, y, ldy, R, C, logn, scale, st);
+            default: return launch_fwht_t<1024, 1>(x, ldx, y, ldy, R, C, logn, scale, st);
+        }
+    }
+    // long columns: one or two columns per workgroup would be read 2 or 4 bytes per row and lane; transpose
+    // into y with 16-byte accesses instead and transform y in place (the output is the only scratch)
+    hipLaunchKernelGGL(transpose_bf16_kernel, dim3((unsigned)((R / 64) * (C / 64))), dim3(256), 0, st, static_cast<const uint16_t*>(x), ldx,
+                       static_cast<uint16_t*>(y), ldy, (int)(C / 64));
+    if (int e = check_launch("ti8_fwht_t")) return e;
+    return ti8_fwht(y, ldy, y, ldy, C, R, R, scale, stream);
+}
 
 extern "C" int ti8_fwht(const void* x, int64_t ldx, void* y, int64_t ldy, int64_t rows, int64_t cols, int64_t n,
                         float scale, ti8_stream_t stream) {

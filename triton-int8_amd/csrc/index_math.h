@@ -133,6 +133,24 @@ TI8_HD int fwht_group_base(int vt, int p, int rb) {
     return (hi << (p + rb)) | lo;
 }
 
+// transposed-input transform (y = FWHT of x^T along its rows = along the ROWS of x, length R):
+// columns of x per workgroup (as many as fit the LDS budget of 32768 fp32 elements, at most the 8
+// that one 16-byte load brings) and the column block of workgroup `id`: the G = 64 / W workgroups
+// whose columns share one 128-byte line of every row get consecutive places on ONE XCD (workgroup
+// ids 8 apart share an XCD), so that the line is fetched from HBM once; identity when the number of
+// such groups is not a multiple of 8
+TI8_HD int fwht_t_cols_per_wg(int64_t R) { return R <= 4096 ? 8 : (int)(32768 / R); }
+// whether the one-kernel transposed transform is used: up to 8192 rows (4 columns per workgroup and
+// more); longer columns go through a transposing copy into the output and an in-place transform
+// there, which needs whole 64 x 64 tiles
+TI8_HD bool fwht_t_direct(int64_t R, int64_t C) { return R <= 8192 || (C % 64) != 0; }
+TI8_HD int64_t fwht_t_colblock(int64_t id, int64_t nblocks, int W) {
+    const int G = 64 / W;
+    if (nblocks % (8 * (int64_t)G) != 0) return id;
+    const int64_t xcd = id & 7, j = id >> 3;
+    return ((j / G) * 8 + xcd) * G + (j % G);
+}
+
 // ---- per-row quantiser (quant.hip) -----------------------------------------------------------
 // row handled by (workgroup, wave): one workgroup per row, or one wave per row (4 rows per workgroup)
 TI8_HD int64_t qrow_row(int64_t block, int wave, bool wg_row) { return wg_row ? block : block * 4 + wave; }

@@ -197,11 +197,14 @@ def linear_backward(dY2, X2, W, scheme="block_channel", hadamard=None, saved=Non
         return dX, dW
     # double_channel
     if hadamard == "full":
+        # the transposed operands are rotated along the rows of the tensors as they lie in memory (ops.fwht_t):
+        # no bf16 transpose of W, dY or X.  A token count that is not a power of two in [128, 32768] has no
+        # full-length rotation along the tokens (as in the reference, whose transform needs a power of two)
         dq, ds = ops.quant_row(ops.fwht(dY2), clamp=True, inv_mode=INV_AMAX_DIV_127)
-        wtq, wts = ops.quant_row(ops.fwht(W.t().contiguous()), clamp=True, inv_mode=INV_AMAX_DIV_127)
+        wtq, wts = ops.quant_row(ops.fwht_t(W), clamp=True, inv_mode=INV_AMAX_DIV_127)
         dX = _gemm_dc(dq, ds, wtq, wts, 1.0 / N, tokens=tokens)
-        dytq, dyts = ops.quant_row(ops.fwht(dY2.t().contiguous()), clamp=True, inv_mode=INV_AMAX_DIV_127)
-        xtq, xts = ops.quant_row(ops.fwht(X2.t().contiguous()), clamp=True, inv_mode=INV_AMAX_DIV_127)
+        dytq, dyts = ops.quant_row(ops.fwht_t(dY2), clamp=True, inv_mode=INV_AMAX_DIV_127)
+        xtq, xts = ops.quant_row(ops.fwht_t(X2), clamp=True, inv_mode=INV_AMAX_DIV_127)
         dW = _gemm_dc(dytq, dyts, xtq, xts, 1.0 / T)
         return dX, dW
     dq, ds, dytq, dyts = _row_col(dY2, clamp=True, inv_mode=INV_AMAX_DIV_127)

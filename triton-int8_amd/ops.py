@@ -16,7 +16,7 @@ from ._lib import (COMBINE_DIV_PROD, COMBINE_MUL_MUL, COMBINE_MUL_PROD, GEMM_LAR
                    Q_WS_PINGPONG, Q_WS_SECOND,
                    SCALE_BLOCK128, SCALE_BLOCK_K256, SCALE_ROW, SCALE_ROW_K128)
 
-__all__ = ["quant_block", "quant_block_multi", "quant_block_had128", "quant_row", "quant_col_t", "quant_row_col_t", "fwht", "gemm_i8_nt", "gemm_i8_nt_i32"]
+__all__ = ["quant_block", "quant_block_multi", "quant_block_had128", "quant_row", "quant_col_t", "quant_row_col_t", "fwht", "fwht_t", "gemm_i8_nt", "gemm_i8_nt_i32"]
 
 
 # Which GEMM kernel `gemm_i8_nt` asks for: "auto" (the few-rows kernel for M <= 256, else an
@@ -268,6 +268,21 @@ def fwht(x, n=None, scale=1.0):
     y = torch.empty((x2.shape[0], cols), dtype=torch.bfloat16, device=x.device)
     _lib.call("ti8_fwht", x2.data_ptr(), x2.stride(0), y.data_ptr(), cols, x2.shape[0], cols, n, float(scale), _stream())
     return y.reshape(x.shape)
+
+
+def fwht_t(x, scale=1.0):
+    """Walsh-Hadamard transform of ``x.T`` along its rows, i.e. along the ROWS of ``x`` [R, C], without
+    the bf16 transpose: returns y [C, R] = ``fwht(x.T.contiguous())``, bit for bit."""
+    _check_bf16(x, "x")
+    _need(x.dim() == 2, "x must be [R, C]")
+    R, C = x.shape
+    _need(R >= 128 and R <= 32768 and (R & (R - 1)) == 0, f"R must be a power of two in [128, 32768], got {R}")
+    _need(C > 0 and C % 8 == 0, f"C must be a positive multiple of 8, got {C}")
+    if x.stride(1) != 1 or x.stride(0) % 8 or x.data_ptr() % 16:
+        x = x.contiguous()
+    y = torch.empty((C, R), dtype=torch.bfloat16, device=x.device)
+    _lib.call("ti8_fwht_t", x.data_ptr(), x.stride(0), y.data_ptr(), R, R, C, float(scale), _stream())
+    return y
 
 
 def _k_contig(t):
