@@ -273,6 +273,27 @@ int ti8_gemm_i8_nt(const int8_t* A, int64_t bsa, int64_t lda,
                    int acc_i32_full, int combine, float out_scale, float post_scale,
                    int gemm_flags, ti8_stream_t stream);
 
+/* Up to 3 such GEMMs, each with batch = 1 and M % 128 == 0, in ONE launch: the three GEMMs of a
+ * training step (Y = fwd_32(X, W), dX = fwd_32(dY, W^T), dW = bwd_33(dY^T, X^T); the reference
+ * launches int8_gemm_kernel once for each, triton/block_channel_fwd32.py:83,
+ * triton/block_channel_bwd33.py:72) when all their operands are at hand.  Every field means what the
+ * argument of that name means in ti8_gemm_i8_nt; `problems` is a HOST array, read before the call
+ * returns.  Each GEMM runs the kernel that ti8_gemm_i8_nt with TI8_GEMM_TILED selects for its shape
+ * and scale modes, so results are bit-identical to such separate calls; one launch serves them when
+ * they all select the same kernel (not TI8_GEMM_STRICT, not TI8_SCALE_ROW_K128), otherwise they are
+ * launched one after the other.  TI8_GEMM_SKINNY is refused. */
+typedef struct ti8_gemm_problem {
+    const int8_t* A; int64_t bsa, lda;
+    const int8_t* B; int64_t bsb, ldb;
+    void* C; int64_t bsc, ldc;
+    const float* sA; int modeA; int64_t sa_bs, sa_rs, sa_ks;
+    const float* sB; int modeB; int64_t sb_bs, sb_rs, sb_ks;
+    int64_t batch, M, N, K;
+    int acc_i32_full, combine;
+    float out_scale, post_scale;
+} ti8_gemm_problem;
+int ti8_gemm_i8_nt_multi(const ti8_gemm_problem* problems, int count, int gemm_flags, ti8_stream_t stream);
+
 /* Raw int32 accumulators of the same GEMM over the whole K, C int32 [batch][M][N]:
  * the accumulator of int8_gemm_kernel in triton/double-channle_fwd32.py:44,56.
  * Exists so that tests can compare accumulators bit for bit. */

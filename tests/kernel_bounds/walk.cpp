@@ -385,4 +385,38 @@ int walk_gemm(int64_t bsa, int64_t lda, int64_t bsb, int64_t ldb, int64_t bsc, i
     return r.bad;
 }
 
+// Workgroup -> (GEMM, tile) map of a several-GEMM launch (gemm.hip: gemm_i8_multi_kernel, launch_multi):
+// tiles[i] = workgroups of GEMM i.  Every workgroup of the grid must land in a GEMM i < count with
+// a tile index in [0, tiles[i]), and every (GEMM, tile) must be taken exactly once.
+int walk_gemm_multi_map(const int* tiles, int count, int64_t* n_checked, char* msg, int msglen) {
+    Report r{msg, msglen};
+    int first[4] = {0, 0, 0, 0};
+    int total = 0;
+    for (int i = 0; i < count; ++i) {
+        first[i] = total;
+        total += tiles[i];
+    }
+    for (int i = count; i < 4; ++i) first[i] = total;
+    std::vector<std::vector<int>> seen(count);
+    for (int i = 0; i < count; ++i) seen[i].assign(tiles[i], 0);
+    for (int w = 0; w < total && !r.bad; ++w) {
+        const int i = gemm_multi_pick(w, first[1], first[2], count);
+        const int t = w - first[i];
+        if (i < 0 || i >= count || t < 0 || t >= tiles[i]) {
+            r.fail("gemm multi: workgroup %d maps to GEMM %d tile %d (of %d GEMMs, %d tiles)", w, i, t, count, i >= 0 && i < count ? tiles[i] : -1);
+            break;
+        }
+        ++seen[i][t];
+        ++r.checked;
+    }
+    for (int i = 0; i < count && !r.bad; ++i)
+        for (int t = 0; t < tiles[i]; ++t)
+            if (seen[i][t] != 1) {
+                r.fail("gemm multi: tile %d of GEMM %d is computed %d times", t, i, seen[i][t]);
+                break;
+            }
+    *n_checked = r.checked;
+    return r.bad ? 1 : 0;
+}
+
 }  // extern "C"

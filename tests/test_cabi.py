@@ -156,3 +156,29 @@ def test_quant_block_multi_validation(lib):
         rc = lib.ti8_quant_block_multi(ops_, n, 1, 0, None)
         assert rc == code and msg in lib.ti8_last_error().decode(), (lib.ti8_last_error(), msg)
     assert lib.ti8_quant_block_multi(arr(good), 1, 8, 0, None) == 4      # TI8_Q_HAD128
+
+
+def test_gemm_multi_validation(lib):
+    """ti8_gemm_i8_nt_multi takes a host array of GEMM descriptors; a bad one is rejected before any launch, with
+    the checks of ti8_gemm_i8_nt."""
+    import triton_int8_amd
+    L = triton_int8_amd._lib
+    good = dict(A=FAKE, bsa=0, lda=128, B=FAKE, bsb=0, ldb=128, C=FAKE, bsc=0, ldc=512, sA=FAKE, modeA=1, sa_bs=0, sa_rs=1, sa_ks=1,
+                sB=FAKE, modeB=0, sb_bs=0, sb_rs=1, sb_ks=0, batch=1, M=512, N=512, K=128, acc_i32_full=0, combine=0,
+                out_scale=1.0, post_scale=0.0)
+    arr = lambda *ds: (L.GemmProblem * len(ds))(*[L.GemmProblem(**d) for d in ds])
+    cases = [((None, 1, 0), 1, "problems is required"),
+             ((arr(good), 0, 0), 2, "between 1 and 3"),
+             ((arr(good, good, good, good), 4, 0), 2, "between 1 and 3"),
+             ((arr(good), 1, 4), 4, "few-rows kernel"),                      # TI8_GEMM_SKINNY
+             ((arr(good), 1, 256), 4, "unknown flag"),
+             ((arr(good, {**good, "batch": 2}), 2, 0), 2, "batch = 1, GEMM 1"),
+             ((arr({**good, "M": 64}), 1, 0), 2, "multiple of 128"),
+             ((arr({**good, "K": 100}), 1, 0), 2, "multiples of 128"),
+             ((arr(good, {**good, "sB": None}), 2, 0), 1, "scale pointer of B"),
+             ((arr({**good, "acc_i32_full": 1}), 1, 0), 4, "per-row scales on both"),
+             ((arr({**good, "A": FAKE + 4}), 1, 0), 3, "aligned"),
+             ((arr({**good, "ldc": 64}), 1, 0), 2, "leading dimension")]
+    for (p, n, flags), code, msg in cases:
+        rc = lib.ti8_gemm_i8_nt_multi(p, n, flags, None)
+        assert rc == code and msg in lib.ti8_last_error().decode(), (rc, lib.ti8_last_error(), msg)

@@ -81,6 +81,58 @@ def test_block_quant(T, dev):
     assert bits_equal(q, qo) and bits_equal(s, so)
 
 
+def test_gemms_of_a_step_in_one_launch(T, dev):
+    """ti8_gemm_i8_nt_multi = separate tiled ti8_gemm_i8_nt calls, bit for bit: GEMMs that share a kernel (one launch), GEMMs
+    that do not (launched one after the other inside the call), both scale layouts, and the layer step built on it."""
+    from triton_int8_amd import ops
+    g = make_gen(75)
+
+    def operands(M, N, K, rows):
+        A = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8).to(dev)
+        B = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8).to(dev)
+        if rows:
+            sA, sB = torch.rand(M, generator=g).add(0.5).mul(1e-2).to(dev), torch.rand(N, generator=g).add(0.5).mul(1e-2).to(dev)
+            return dict(A=A, B=B, sA=sA, modeA=0, sB=sB, modeB=0, acc_i32_full=True)
+        sA, sB = torch.rand(M // 128, K // 128, generator=g).add(0.5).mul(1e-2).to(dev), torch.rand(N, generator=g).add(0.5).mul(1e-2).to(dev)
+        return dict(A=A, B=B, sA=sA, modeA=1, sB=sB, modeB=0)
+
+    def separate(p):
+        kw = {k: v for k, v in p.items() if k in ("acc_i32_full", "combine", "out_scale", "post_scale")}
+        return ops.gemm_i8_nt(p["A"][None], p["B"], p["sA"][None], p["modeA"], p["sB"], p["modeB"], **kw)[0]
+
+    ops.GEMM_PATH = "tiled"
+    try:
+        for rows in (False, True):
+            # 128 x 128 tiles for all three: one launch; the ragged one has tile counts that are no multiple of 8
+            same = [operands(384, 256, 512, rows), operands(128, 640, 256, rows), operands(256, 128, 1024, rows)]
+            # 4096 x 4096 fills the machine with 256 x 256 tiles, the others take 128 x 128: separate launches inside the call
+            mixed = [operands(256, 256, 256, rows), operands(4096, 4096, 256, rows)]
+            for ps in (same, same[:1], same[:2], mixed):
+                for got, p in zip(ops.gemm_i8_nt_multi(ps), ps):
+                    assert torch.equal(got, separate(p))
+        # caller-provided outputs, out_scale
+        ps = [dict(operands(256, 256, 256, False), out_scale=0.5, out=torch.empty(256, 256, dtype=torch.bfloat16, device=dev))]
+        out, = ops.gemm_i8_nt_multi(ps)
+        assert out.data_ptr() == ps[0]["out"].data_ptr() and torch.equal(out, separate(ps[0]))
+    finally:
+        ops.GEMM_PATH = "auto"
+    with pytest.raises(ValueError):
+        ops.gemm_i8_nt_multi([])
+    # the layer step above 256 tokens runs Y, dX and dW in one launch: same bits as forward + backward called separately
+    X, W, dY = randn_bf16(g, 640, 512).to(dev), randn_bf16(g, 384, 512, std=0.02).to(dev), randn_bf16(g, 640, 384, std=1e-3).to(dev)
+    with T._lib.timed_launches() as rec:
+        Y, dX, dW = T.linear_fwd_bwd(X, W, dY, "block_channel")
+    assert len(rec["ti8_gemm_i8_nt_multi"]) == 1 and "ti8_gemm_i8_nt" not in rec
+    Y0, saved = T.linear.linear_forward(X, W, "block_channel")
+    dX0, dW0 = T.linear.linear_backward(dY, X, W, "block_channel", None, saved)
+    assert torch.equal(Y, Y0) and torch.equal(dX, dX0) and torch.equal(dW, dW0)
+    # a ragged token count is padded to the tile before the launch
+    Yr, dXr, dWr = T.linear_fwd_bwd(X[:300], W, dY[:300], "block_channel")
+    Y1, saved = T.linear.linear_forward(T.linear.pad_tokens(X[:300]), W, "block_channel")
+    dX1, dW1 = T.linear.linear_backward(T.linear.pad_tokens(dY[:300]), T.linear.pad_tokens(X[:300]), W, "block_channel", None, saved)
+    assert torch.equal(Yr, Y1[:300]) and torch.equal(dXr, dX1[:300]) and torch.equal(dWr, dW1)
+
+
 def test_block_quant_of_several_operands_in_one_launch(T, dev):
     """ti8_quant_block_multi = separate ti8_quant_block calls, bit for bit: operands of different shapes,
     with and without the transposed copy, and the layer step that uses it for X and dY."""

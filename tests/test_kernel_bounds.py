@@ -41,6 +41,7 @@ def walker(tmp_path_factory):
     lib.walk_quant_row.argtypes = [i64] * 4 + [ci] + [i64] * 3 + [p64, cp, ci]
     lib.walk_quant_block.argtypes = [i64, i64, ci, i64, i64, ci, i64, i64, i64, i64, i64, i64, i64, i64, ci, i64, i64, i64, i64, p64, cp, ci]
     lib.walk_gemm.argtypes = [i64] * 6 + [ctypes.POINTER(ScaleArg)] * 2 + [i64] * 4 + [ci] * 5 + [i64] * 3 + [ctypes.POINTER(ci), p64, cp, ci]
+    lib.walk_gemm_multi_map.argtypes = [ctypes.POINTER(ci), ci, p64, cp, ci]
     return lib
 
 
@@ -77,6 +78,7 @@ def recorded(monkeypatch):
     monkeypatch.setattr(T.ops, "_on_gpu", lambda t: True)
     monkeypatch.setattr(T.ops, "_stream", lambda: None)
     monkeypatch.setattr(torch.cuda, "set_device", lambda d: None)
+    monkeypatch.setattr(torch.cuda, "is_current_stream_capturing", lambda: False)
     monkeypatch.setattr(torch.Tensor, "cuda", lambda self, *a, **k: self)
     monkeypatch.setattr(T._lib, "call", lambda name, *args: calls.append((name, args)))
     yield T, allocs, calls
@@ -112,6 +114,23 @@ def walk(lib, allocs, name, a):
             A, bsa, lda, B, bsb, ldb, C, bsc, ldc, batch, M, N, K = a[:13]
             rc = lib.walk_gemm(bsa, lda, bsb, ldb, bsc, ldc, None, None, batch, M, N, K, 0, 0, 0, 1,
                                NUM_CU, allocs.room(A, 1), allocs.room(B, 1), allocs.room(C, 4), picked, ctypes.byref(n), msg, 512)
+    elif name == "ti8_gemm_i8_nt_multi":
+        # every GEMM of the launch as the tiled kernel walks it alone, then the workgroup -> (GEMM, tile) map
+        problems, count, flags = a[:3]
+        total, tiles = 0, (ctypes.c_int * count)()
+        for i in range(count):
+            p = problems[i]
+            picked = (ctypes.c_int * 3)()
+            sa = ScaleArg(p.modeA, p.sa_bs, p.sa_rs, p.sa_ks, allocs.room(p.sA, 4))
+            sb = ScaleArg(p.modeB, p.sb_bs, p.sb_rs, p.sb_ks, allocs.room(p.sB, 4))
+            rc = lib.walk_gemm(p.bsa, p.lda, p.bsb, p.ldb, p.bsc, p.ldc, ctypes.byref(sa), ctypes.byref(sb), 1, p.M, p.N, p.K, p.acc_i32_full,
+                               flags & 1, (flags >> 3) & 1, 0, NUM_CU, allocs.room(p.A, 1), allocs.room(p.B, 1), allocs.room(p.C, 2),
+                               picked, ctypes.byref(n), msg, 512)
+            assert rc == 0, f"{name}, GEMM {i}: {msg.value.decode()}"
+            total += n.value
+            tiles[i] = -(-p.M // picked[0]) * -(-p.N // picked[1])
+        rc = lib.walk_gemm_multi_map(tiles, count, ctypes.byref(n), msg, 512)
+        n.value += total
     else:
         raise AssertionError(f"no walker for {name}")
     assert rc == 0, f"{name}: {msg.value.decode()}"
@@ -206,3 +225,24 @@ def test_transposed_hadamard_launches(walker, recorded, R, C):
     n = ctypes.c_int64(0)
     assert walker.walk_fwht_t(C, R, R, C, R * C - 1, R * C, LDS_LIMIT, ctypes.byref(n), msg, 512) == 1 and msg.value.split(b":")[0].endswith(b" x")
     assert walker.walk_fwht_t(C, R, R, C, R * C, R * C - 8, LDS_LIMIT, ctypes.byref(n), msg, 512) == 1 and msg.value.split(b":")[0].endswith(b" y")
+
+
+@pytest.mark.parametrize("M,K,N", [(1024, 512, 768), (8192, 4096, 4096)])
+def test_one_launch_step_is_in_bounds(walker, recorded, M, K, N):
+    """The three GEMMs of a block-channel step in one launch: each GEMM's accesses stay inside its operands, and the
+    launch's workgroups cover every tile of every GEMM exactly once."""
+    T, allocs, calls = recorded
+    X, W, dY = (allocs.add(torch.empty(s, dtype=torch.bfloat16)) for s in ((M, K), (N, K), (M, N)))
+    T.linear_fwd_bwd(X, W, dY, "block_channel")
+    names = [c[0] for c in calls]
+    assert names.count("ti8_gemm_i8_nt_multi") == 1 and "ti8_gemm_i8_nt" not in names
+    name, a = next(c for c in calls if c[0] == "ti8_gemm_i8_nt_multi")
+    assert a[1] == 3 and walk(walker, allocs, name, a) > 3
+
+
+@pytest.mark.parametrize("tiles", [[512, 512, 512], [1, 1, 1], [7, 300, 2], [5], [9, 4]])
+def test_multi_launch_map(walker, tiles):
+    msg, n = ctypes.create_string_buffer(512), ctypes.c_int64(0)
+    arr = (ctypes.c_int * len(tiles))(*tiles)
+    assert walker.walk_gemm_multi_map(arr, len(tiles), ctypes.byref(n), msg, 512) == 0, msg.value.decode()
+    assert n.value == sum(tiles)

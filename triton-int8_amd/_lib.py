@@ -18,6 +18,15 @@ class QBlockOperand(ctypes.Structure):
                 ("qT", _vp), ("bsqt", _i64), ("ldqt", _i64), ("s", _vp), ("ssb", _i64), ("ssr", _i64), ("ssc", _i64),
                 ("B", _i64), ("R", _i64), ("C", _i64)]
 
+class GemmProblem(ctypes.Structure):
+    """ti8_gemm_problem of include/ti8.h."""
+    _fields_ = [("A", _vp), ("bsa", _i64), ("lda", _i64), ("B", _vp), ("bsb", _i64), ("ldb", _i64),
+                ("C", _vp), ("bsc", _i64), ("ldc", _i64),
+                ("sA", _vp), ("modeA", _int), ("sa_bs", _i64), ("sa_rs", _i64), ("sa_ks", _i64),
+                ("sB", _vp), ("modeB", _int), ("sb_bs", _i64), ("sb_rs", _i64), ("sb_ks", _i64),
+                ("batch", _i64), ("M", _i64), ("N", _i64), ("K", _i64), ("acc_i32_full", _int), ("combine", _int),
+                ("out_scale", _f32), ("post_scale", _f32)]
+
 
 # name -> argument types, in the order of include/ti8.h
 PROTOTYPES = {
@@ -34,6 +43,7 @@ PROTOTYPES = {
     "ti8_gemm_i8_nt": [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64,
                        _vp, _int, _i64, _i64, _i64, _vp, _int, _i64, _i64, _i64,
                        _i64, _i64, _i64, _i64, _int, _int, _f32, _f32, _int, _vp],
+    "ti8_gemm_i8_nt_multi": [ctypes.POINTER(GemmProblem), _int, _int, _vp],
     "ti8_gemm_i8_nt_i32": [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp],
     "ti8_probe_mfma": [_vp, _i64, _vp, _int, _int, _int, _int, _vp],
 }

@@ -45,8 +45,10 @@ __device__ __forceinline__ void interleave_hint() {
 //             into buffer cur (every wave is past its last read of it)
 // so there is one barrier per K tile, it sits where the next fragments are already in
 // registers, and a tile's loads have a full K tile of MFMA time to land.
+// One output tile of one GEMM: the whole kernel body.  `block_x` = index of the workgroup among the
+// tiles of this GEMM, `batch` = batch index.
 template <int BM, int BN, int WM, int WN, int EPI>
-__global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g) {
+__device__ __forceinline__ void gemm_i8_tile(const GemmArgs& g, const int block_x, const int batch) {
     constexpr int NW = WM * WN;
     constexpr int TM = BM / WM / 32;  // 32x32 blocks per wave along M
     constexpr int TN = BN / WN / 32;
@@ -74,8 +76,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
     // share are about the same size (256-row tiles: 4 measured 0.4 % faster than 8 and 1 % faster
     // than 16 on 8192 x 4096 x 4096)
     constexpr int GROUP = idx::gemm_group_rows(BM);
-    const idx::TileCoord tc = idx::gemm_tile_of(blockIdx.x, g.tiles_m, g.tiles_n, GROUP);
-    const int batch = blockIdx.y;
+    const idx::TileCoord tc = idx::gemm_tile_of(block_x, g.tiles_m, g.tiles_n, GROUP);
     const int m0 = tc.tile_m * BM, n0 = tc.tile_n * BN;
 
     const int8_t* Ab = g.A + (int64_t)batch * g.bsa;
@@ -520,6 +521,54 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
 }
 
 template <int BM, int BN, int WM, int WN, int EPI>
+__global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g) {
+    gemm_i8_tile<BM, BN, WM, WN, EPI>(g, blockIdx.x, blockIdx.y);
+}
+
+// Several GEMMs (batch of one each) in ONE launch: workgroup w computes tile w - first[i] of the
+// GEMM i whose range holds w.  The three GEMMs of a training step (Y, dX, dW) run this way when all
+// their operands are at hand: no kernel boundary between them, and the last tiles of one GEMM run
+// beside the first tiles of the next instead of beside idle CUs.
+constexpr int GEMM_MULTI_MAX = 3;
+struct GemmMulti {
+    GemmArgs g[GEMM_MULTI_MAX];
+    int first[GEMM_MULTI_MAX + 1];
+    int count;
+};
+
+template <int BM, int BN, int WM, int WN, int EPI>
+__global__ __launch_bounds__(64 * WM * WN) void gemm_i8_multi_kernel(const GemmMulti m) {
+    static_assert(GEMM_MULTI_MAX == 3, "gemm_multi_pick knows three ranges");
+    const int i = idx::gemm_multi_pick((int)blockIdx.x, m.first[1], m.first[2], m.count);
+    gemm_i8_tile<BM, BN, WM, WN, EPI>(m.g[i], (int)blockIdx.x - m.first[i], 0);
+}
+
+template <int BM, int BN, int WM, int WN, int EPI>
+static int launch_multi(GemmMulti& m, hipStream_t st) {
+    int total = 0;
+    for (int i = 0; i < m.count; ++i) {
+        m.g[i].tiles_m = (m.g[i].M + BM - 1) / BM;
+        m.g[i].tiles_n = (m.g[i].N + BN - 1) / BN;
+        m.first[i] = total;
+        total += m.g[i].tiles_m * m.g[i].tiles_n;
+    }
+    for (int i = m.count; i <= GEMM_MULTI_MAX; ++i) m.first[i] = total;
+    for (int i = m.count; i < GEMM_MULTI_MAX; ++i) m.g[i] = m.g[0];
+    const size_t shmem = 2 * (size_t)(BM + BN) * 128;
+    static thread_local int attr_dev = -1;
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    auto kern = gemm_i8_multi_kernel<BM, BN, WM, WN, EPI>;
+    if (shmem > 64 * 1024 && attr_dev != dev) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+        if (e != hipSuccess) return fail(TI8_ERR_HIP, "gemm: cannot raise the LDS limit to %zu: %s", shmem, hipGetErrorString(e));
+        attr_dev = dev;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(64 * WM * WN), shmem, st, m);
+    return check_launch("ti8_gemm_i8_nt_multi");
+}
+
+template <int BM, int BN, int WM, int WN, int EPI>
 static int launch(const GemmArgs& a0, int64_t batch, hipStream_t st) {
     GemmArgs a = a0;
     a.tiles_m = (a.M + BM - 1) / BM;
@@ -561,52 +610,40 @@ static int check_scale(const char* fn, const char* which, const float* p, int mo
     return TI8_OK;
 }
 
-}  // namespace ti8
-
-using namespace ti8;
-
-extern "C" int ti8_gemm_i8_nt(const int8_t* A, int64_t bsa, int64_t lda, const int8_t* B, int64_t bsb, int64_t ldb,
-                              void* C, int64_t bsc, int64_t ldc, const float* sA, int modeA, int64_t sa_bs,
-                              int64_t sa_rs, int64_t sa_ks, const float* sB, int modeB, int64_t sb_bs, int64_t sb_rs,
-                              int64_t sb_ks, int64_t batch, int64_t M, int64_t N, int64_t K, int acc_i32_full,
-                              int combine, float out_scale, float post_scale, int gemm_flags, ti8_stream_t stream) {
-    const char* fn = "ti8_gemm_i8_nt";
+// Argument checks of one dequantising GEMM and its argument block (shared by ti8_gemm_i8_nt and
+// ti8_gemm_i8_nt_multi)
+static int prepare_gemm(const char* fn, const ti8_gemm_problem& p, int gemm_flags, GemmArgs* out) {
     // up to 256 rows M may be any multiple of 32 (decode shapes): only the few-rows kernel takes those
-    if (int e = check_operands(fn, A, bsa, lda, B, bsb, ldb, C, ldc, batch, M, N, K, M <= 256 ? 32 : 128)) return e;
-    if (int e = check_scale(fn, "A", sA, modeA)) return e;
-    if (int e = check_scale(fn, "B", sB, modeB)) return e;
+    if (int e = check_operands(fn, p.A, p.bsa, p.lda, p.B, p.bsb, p.ldb, p.C, p.ldc, p.batch, p.M, p.N, p.K, p.M <= 256 ? 32 : 128)) return e;
+    if (int e = check_scale(fn, "A", p.sA, p.modeA)) return e;
+    if (int e = check_scale(fn, "B", p.sB, p.modeB)) return e;
     // the epilogue keeps (row within a tile) * (row stride of A's scales) in 32 bits
-    if (modeA == TI8_SCALE_ROW && (sa_rs < 0 || sa_rs > 0x00ffffff))
+    if (p.modeA == TI8_SCALE_ROW && (p.sa_rs < 0 || p.sa_rs > 0x00ffffff))
         return fail(TI8_ERR_SHAPE, "%s: row stride of A's scales must be in [0, 2^24)", fn);
-    if (combine < 0 || combine > 2) return fail(TI8_ERR_MODE, "%s: unknown combine %d", fn, combine);
+    if (p.combine < 0 || p.combine > 2) return fail(TI8_ERR_MODE, "%s: unknown combine %d", fn, p.combine);
     if (gemm_flags & ~(TI8_GEMM_STRICT | TI8_GEMM_TILED | TI8_GEMM_SKINNY | TI8_GEMM_LARGE_TILES)) return fail(TI8_ERR_MODE, "%s: unknown flag 0x%x", fn, gemm_flags);
     if ((gemm_flags & TI8_GEMM_SKINNY) && (gemm_flags & (TI8_GEMM_TILED | TI8_GEMM_LARGE_TILES)))
         return fail(TI8_ERR_MODE, "%s: TI8_GEMM_SKINNY excludes TI8_GEMM_TILED and TI8_GEMM_LARGE_TILES", fn);
-    if (acc_i32_full && (modeA != TI8_SCALE_ROW || modeB != TI8_SCALE_ROW))
+    if (p.acc_i32_full && (p.modeA != TI8_SCALE_ROW || p.modeB != TI8_SCALE_ROW))
         return fail(TI8_ERR_MODE, "%s: int32 accumulation over the whole K needs per-row scales on both operands", fn);
-    if ((modeA == TI8_SCALE_BLOCK_K256 || modeB == TI8_SCALE_BLOCK_K256) && (K % 256))
+    if ((p.modeA == TI8_SCALE_BLOCK_K256 || p.modeB == TI8_SCALE_BLOCK_K256) && (p.K % 256))
         return fail(TI8_ERR_SHAPE, "%s: 256-wide scale groups need K %% 256 == 0", fn);
-    if ((reinterpret_cast<uintptr_t>(C) & 7) || (ldc % 4) || (bsc % 4)) return fail(TI8_ERR_ALIGN, "%s: C must be 8-byte aligned with strides multiples of 4", fn);
+    if ((reinterpret_cast<uintptr_t>(p.C) & 7) || (p.ldc % 4) || (p.bsc % 4)) return fail(TI8_ERR_ALIGN, "%s: C must be 8-byte aligned with strides multiples of 4", fn);
     GemmArgs a;
-    a.A = A; a.B = B; a.C = C;
-    a.bsa = bsa; a.lda = lda; a.bsb = bsb; a.ldb = ldb; a.bsc = bsc; a.ldc = ldc;
-    a.sa = ScaleDesc{sA, modeA, sa_bs, sa_rs, sa_ks};
-    a.sb = ScaleDesc{sB, modeB, sb_bs, sb_rs, sb_ks};
-    a.M = (int)M; a.N = (int)N; a.K = (int)K;
+    a.A = p.A; a.B = p.B; a.C = p.C;
+    a.bsa = p.bsa; a.lda = p.lda; a.bsb = p.bsb; a.ldb = p.ldb; a.bsc = p.bsc; a.ldc = p.ldc;
+    a.sa = ScaleDesc{p.sA, p.modeA, p.sa_bs, p.sa_rs, p.sa_ks};
+    a.sb = ScaleDesc{p.sB, p.modeB, p.sb_bs, p.sb_rs, p.sb_ks};
+    a.M = (int)p.M; a.N = (int)p.N; a.K = (int)p.K;
     a.tiles_m = a.tiles_n = 0;
-    a.combine = combine;
+    a.combine = p.combine;
     a.strict = (gemm_flags & TI8_GEMM_STRICT) ? 1 : 0;
-    a.out_scale = out_scale; a.post_scale = post_scale;
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    // few rows: too few 256-row tiles to fill the machine, take the kernel that splits N and K finer
-    const bool large = (gemm_flags & TI8_GEMM_LARGE_TILES) != 0;
-    const bool want_skinny = (gemm_flags & TI8_GEMM_SKINNY) || (!(gemm_flags & (TI8_GEMM_TILED | TI8_GEMM_LARGE_TILES)) && M <= 256);
-    if (want_skinny && !a.strict && skinny_supported(a)) return launch_skinny(a, batch, acc_i32_full != 0, st);
-    if (M % 128)
-        return fail(TI8_ERR_SHAPE, "%s: M = %lld is not a multiple of 128, which only the few-rows kernel accepts "
-                    "(not with TI8_GEMM_STRICT / TI8_GEMM_TILED, per-(row, K tile) scales or K > 32768)", fn, (long long)M);
-    // Medium sizes: when the large tiles would leave CUs without a workgroup, use 128 x 128 tiles
-    // (4 waves of 64 x 64, two workgroups per CU): four (two) times as many workgroups.
+    a.out_scale = p.out_scale; a.post_scale = p.post_scale;
+    *out = a;
+    return TI8_OK;
+}
+
+static int device_cu_count() {
     static int num_cu = 0;
     if (num_cu == 0) {
         int dev = 0;
@@ -614,7 +651,11 @@ extern "C" int ti8_gemm_i8_nt(const int8_t* A, int64_t bsa, int64_t lda, const i
         (void)hipGetDevice(&dev);
         num_cu = (hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
     }
-    const idx::GemmConfig c = idx::gemm_config(M, N, K, batch, acc_i32_full != 0, a.strict != 0, modeA, modeB, large, num_cu);
+    return num_cu;
+}
+
+// One GEMM on the LDS-tiled kernel that `c` names
+static int launch_tiled(const char* fn, const GemmArgs& a, int64_t batch, const idx::GemmConfig& c, hipStream_t st) {
 #define TI8_GEMM_CASE(BM, BN, WM, WN, EPI) \
     if (c.bm == BM && c.bn == BN && c.epi == EPI) return launch<BM, BN, WM, WN, EPI>(a, batch, st)
     TI8_GEMM_CASE(128, 128, 2, 2, EPI_ROWS);
@@ -626,6 +667,67 @@ extern "C" int ti8_gemm_i8_nt(const int8_t* A, int64_t bsa, int64_t lda, const i
     TI8_GEMM_CASE(128, 128, 2, 2, EPI_PROMOTE);
 #undef TI8_GEMM_CASE
     return fail(TI8_ERR_MODE, "%s: no kernel for tile %d x %d, epilogue %d", fn, c.bm, c.bn, c.epi);
+}
+
+}  // namespace ti8
+
+using namespace ti8;
+
+extern "C" int ti8_gemm_i8_nt(const int8_t* A, int64_t bsa, int64_t lda, const int8_t* B, int64_t bsb, int64_t ldb,
+                              void* C, int64_t bsc, int64_t ldc, const float* sA, int modeA, int64_t sa_bs,
+                              int64_t sa_rs, int64_t sa_ks, const float* sB, int modeB, int64_t sb_bs, int64_t sb_rs,
+                              int64_t sb_ks, int64_t batch, int64_t M, int64_t N, int64_t K, int acc_i32_full,
+                              int combine, float out_scale, float post_scale, int gemm_flags, ti8_stream_t stream) {
+    const char* fn = "ti8_gemm_i8_nt";
+    const ti8_gemm_problem p = {A, bsa, lda, B, bsb, ldb, C, bsc, ldc, sA, modeA, sa_bs, sa_rs, sa_ks, sB, modeB, sb_bs, sb_rs, sb_ks,
+                                batch, M, N, K, acc_i32_full, combine, out_scale, post_scale};
+    GemmArgs a;
+    if (int e = prepare_gemm(fn, p, gemm_flags, &a)) return e;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    // few rows: too few 256-row tiles to fill the machine, take the kernel that splits N and K finer
+    const bool large = (gemm_flags & TI8_GEMM_LARGE_TILES) != 0;
+    const bool want_skinny = (gemm_flags & TI8_GEMM_SKINNY) || (!(gemm_flags & (TI8_GEMM_TILED | TI8_GEMM_LARGE_TILES)) && M <= 256);
+    if (want_skinny && !a.strict && skinny_supported(a)) return launch_skinny(a, batch, acc_i32_full != 0, st);
+    if (M % 128)
+        return fail(TI8_ERR_SHAPE, "%s: M = %lld is not a multiple of 128, which only the few-rows kernel accepts "
+                    "(not with TI8_GEMM_STRICT / TI8_GEMM_TILED, per-(row, K tile) scales or K > 32768)", fn, (long long)M);
+    return launch_tiled(fn, a, batch, idx::gemm_config(M, N, K, batch, acc_i32_full != 0, a.strict != 0, modeA, modeB, large, device_cu_count()), st);
+}
+
+extern "C" int ti8_gemm_i8_nt_multi(const ti8_gemm_problem* problems, int count, int gemm_flags, ti8_stream_t stream) {
+    const char* fn = "ti8_gemm_i8_nt_multi";
+    if (!problems) return fail(TI8_ERR_NULL, "%s: problems is required", fn);
+    if (count < 1 || count > GEMM_MULTI_MAX) return fail(TI8_ERR_SHAPE, "%s: between 1 and %d GEMMs, got %d", fn, GEMM_MULTI_MAX, count);
+    if (gemm_flags & TI8_GEMM_SKINNY) return fail(TI8_ERR_MODE, "%s: the few-rows kernel is not offered here", fn);
+    GemmMulti m;
+    m.count = count;
+    idx::GemmConfig c[GEMM_MULTI_MAX];
+    // every GEMM runs the kernel its own shape selects; one launch serves them when they all agree on it
+    bool one_launch = true;
+    for (int i = 0; i < count; ++i) {
+        const ti8_gemm_problem& p = problems[i];
+        if (int e = prepare_gemm(fn, p, gemm_flags, &m.g[i])) return e;
+        if (p.batch != 1) return fail(TI8_ERR_SHAPE, "%s: every GEMM must have batch = 1, GEMM %d has %lld", fn, i, (long long)p.batch);
+        if (p.M % 128) return fail(TI8_ERR_SHAPE, "%s: M must be a multiple of 128, GEMM %d has %lld", fn, i, (long long)p.M);
+        c[i] = idx::gemm_config(p.M, p.N, p.K, 1, p.acc_i32_full != 0, m.g[i].strict != 0, p.modeA, p.modeB,
+                                (gemm_flags & TI8_GEMM_LARGE_TILES) != 0, device_cu_count());
+        one_launch = one_launch && c[i].bm == c[0].bm && c[i].bn == c[0].bn && c[i].epi == c[0].epi;
+    }
+    one_launch = one_launch && c[0].epi != EPI_STRICT && c[0].epi != EPI_PROMOTE_LANE;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (one_launch) {
+#define TI8_GEMM_CASE(BM, BN, WM, WN, EPI) \
+        if (c[0].bm == BM && c[0].bn == BN && c[0].epi == EPI) return launch_multi<BM, BN, WM, WN, EPI>(m, st)
+        TI8_GEMM_CASE(128, 128, 2, 2, EPI_ROWS);
+        TI8_GEMM_CASE(256, 256, 2, 4, EPI_ROWS);
+        TI8_GEMM_CASE(256, 256, 2, 4, EPI_PROMOTE_CHAIN);
+        TI8_GEMM_CASE(256, 128, 4, 2, EPI_PROMOTE);
+        TI8_GEMM_CASE(128, 128, 2, 2, EPI_PROMOTE);
+#undef TI8_GEMM_CASE
+    }
+    for (int i = 0; i < count; ++i)
+        if (int e = launch_tiled(fn, m.g[i], 1, c[i], st)) return e;
+    return TI8_OK;
 }
 
 extern "C" int ti8_gemm_i8_nt_i32(const int8_t* A, int64_t bsa, int64_t lda, const int8_t* B, int64_t bsb, int64_t ldb,

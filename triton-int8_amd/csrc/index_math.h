@@ -42,6 +42,15 @@ TI8_HD TileCoord gemm_tile_of(int block_id, int tiles_m, int tiles_n, int group)
     return t;
 }
 
+// GEMM of a several-GEMM launch that workgroup `block` works for: GEMM i owns the workgroups
+// [first[i], first[i + 1]), first[0] = 0; only first[1] and first[2] are needed for up to 3 GEMMs
+TI8_HD int gemm_multi_pick(int block, int first1, int first2, int count) {
+    int i = 0;
+    if (count > 1 && block >= first1) i = 1;
+    if (count > 2 && block >= first2) i = 2;
+    return i;
+}
+
 // tile rows per group of the map above for tiles of bm rows
 constexpr int gemm_group_rows(int bm) { return bm >= 256 ? 4 : 8; }
 

@@ -235,6 +235,35 @@ def pad_tokens(x2, multiple=128):
     return out
 
 
+# Schemes whose whole step (linear_fwd_bwd, no rotation, more than 256 tokens and output features) runs its three GEMMs as one
+# launch (ops.gemm_i8_nt_multi; same kernels on the same operands, so the same bits as linear_forward +
+# linear_backward).  Measured at 8192 tokens, K = N = 4096: block_channel 0.497 -> 0.482 ms per step;
+# double_channel, which the function also serves, gains nothing (0.445 -> 0.448) and stays on three launches.
+ONE_LAUNCH_SCHEMES = ("block_channel",)
+
+
+def _step_one_launch(X2, W, dY2, scheme):
+    """(Y, dX, dW) of padded 2-D operands with more than 256 tokens, without rotation: the quantisers of
+    linear_forward / linear_backward, then Y, dX and dW in one GEMM launch."""
+    if scheme == "block_channel":
+        (xq, xqT, xs), (dq, dqT, ds) = ops.quant_block_multi([X2[None], dY2[None]], clamp=True, with_transpose=True)
+        wq, ws, wtq, wts = _row_col(W, clamp=True)
+        blk, row = dict(modeA=SCALE_BLOCK128), dict(modeB=SCALE_ROW)
+        return ops.gemm_i8_nt_multi([
+            dict(A=xq[0], B=wq, sA=xs[0], sB=ws, **blk, **row),
+            dict(A=dq[0], B=wtq, sA=ds[0], sB=wts, **blk, **row),
+            # scales of the transposed operands are the transposed scale grids
+            dict(A=dqT[0], B=xqT[0], sA=ds[0].t(), sB=xs[0].t(), **blk, modeB=SCALE_BLOCK128)])
+    kw = dict(clamp=True, inv_mode=INV_AMAX_DIV_127)
+    xq, xs, xtq, xts = _row_col(X2, **kw)
+    wq, ws, wtq, wts = _row_col(W, **kw)
+    dq, ds, dytq, dyts = _row_col(dY2, **kw)
+    rows = dict(modeA=SCALE_ROW, modeB=SCALE_ROW, acc_i32_full=True)
+    return ops.gemm_i8_nt_multi([dict(A=xq, B=wq, sA=xs, sB=ws, **rows),
+                                 dict(A=dq, B=wtq, sA=ds, sB=wts, **rows),
+                                 dict(A=dytq, B=xtq, sA=dyts, sB=xts, **rows)])
+
+
 def linear_fwd_bwd(X, W, dY, scheme="block_channel", hadamard=None):
     """One forward + backward of the layer: returns (Y, dX, dW) for X [B,M,K] or [M,K].
     Any number of tokens is accepted (zero-padded to a multiple of 128, see :func:`pad_tokens`);
@@ -244,6 +273,10 @@ def linear_fwd_bwd(X, W, dY, scheme="block_channel", hadamard=None):
     X2, dY2 = X.reshape(-1, K), dY.reshape(-1, N)
     T = X2.shape[0]
     X2, dY2 = pad_tokens(X2), pad_tokens(dY2)
+    # (with up to 256 rows - tokens for Y and dX, output features for dW - a GEMM launched alone takes the few-rows kernel)
+    if hadamard is None and scheme in ONE_LAUNCH_SCHEMES and min(X2.shape[0], N) > 256 and ops.GEMM_PATH in ("auto", "tiled", "large"):
+        Y, dX, dW = _step_one_launch(X2, W, dY2, scheme)
+        return Y[:T].reshape(*lead, N), dX[:T].reshape(*lead, K), dW
     pre = None
     if scheme == "block_channel" and hadamard is None:
         # both activations are at hand: one quantiser launch for X and dY (the forward alone would quantise X, the

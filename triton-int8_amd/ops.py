@@ -342,6 +342,40 @@ def gemm_i8_nt(A, B, sA, modeA, sB, modeB, *, acc_i32_full=False, combine=COMBIN
     return out
 
 
+def gemm_i8_nt_multi(problems):
+    """Up to 3 GEMMs ``dequant(A @ B^T)`` with A int8 [M, K] and B int8 [N, K] in ONE launch; `problems`
+    is a list of dicts with the keys A, B, sA, modeA, sB, modeB and optionally acc_i32_full, combine,
+    out_scale, post_scale, out (meaning as in ``gemm_i8_nt``).  Returns the bf16 outputs [M, N],
+    bit-identical to separate calls.  The GEMMs must select the same kernel (else RuntimeError)."""
+    _need(1 <= len(problems) <= 3, "between 1 and 3 GEMMs")
+    descs, outs, keep = (_lib.GemmProblem * len(problems))(), [], []
+    for i, p in enumerate(problems):
+        A, B = p["A"], p["B"]
+        _need(A.dtype == torch.int8 and B.dtype == torch.int8 and _on_gpu(A) and _on_gpu(B), "A and B must be int8 GPU tensors")
+        _need(A.dim() == 2 and B.dim() == 2, "A must be [M, K] and B [N, K]")
+        M, K = A.shape
+        N = B.shape[0]
+        _need(B.shape[1] == K, f"K mismatch: A has {K}, B has {B.shape[1]}")
+        _need(M % 128 == 0 and N % 128 == 0 and K % 128 == 0 and M > 0 and N > 0 and K > 0,
+              f"M, N, K must be positive multiples of 128, got M={M} N={N} K={K}")
+        A, B = _k_contig(A), _k_contig(B)
+        sAv, _, sa_rs, sa_ks = _scale_desc(p["sA"], p["modeA"], M, K // 128, 1, False, "A")
+        sBv, _, sb_rs, sb_ks = _scale_desc(p["sB"], p["modeB"], N, K // 128, 1, False, "B")
+        out = p.get("out")
+        if out is None:
+            out = torch.empty((M, N), dtype=torch.bfloat16, device=A.device)
+        else:
+            _need(out.shape == (M, N) and out.dtype == torch.bfloat16 and out.stride(1) == 1, "bad `out` tensor")
+        descs[i] = _lib.GemmProblem(A.data_ptr(), 0, A.stride(0), B.data_ptr(), 0, B.stride(0), out.data_ptr(), 0, out.stride(0),
+                                    sAv.data_ptr(), p["modeA"], 0, sa_rs, sa_ks, sBv.data_ptr(), p["modeB"], 0, sb_rs, sb_ks,
+                                    1, M, N, K, 1 if p.get("acc_i32_full") else 0, p.get("combine", COMBINE_MUL_MUL),
+                                    float(p.get("out_scale", 1.0)), float(p.get("post_scale", 0.0)))
+        outs.append(out)
+        keep.append((A, B, sAv, sBv))     # contiguous copies stay alive until the launch is queued
+    _lib.call("ti8_gemm_i8_nt_multi", descs, len(problems), {"auto": 0, "tiled": GEMM_TILED, "large": GEMM_LARGE_TILES}.get(GEMM_PATH, 0), _stream())
+    return outs
+
+
 def gemm_i8_nt_i32(A, B):
     """Raw int32 accumulators of A[b] @ B[b]^T over the whole K."""
     _need(A.dtype == torch.int8 and B.dtype == torch.int8 and _on_gpu(A) and _on_gpu(B), "A and B must be int8 GPU tensors")
