@@ -532,13 +532,15 @@ def test_skinny_and_ragged_token_counts(T, dev, tokens, gemm_path):
                 assert bits_equal(a, b)
 
 
-@pytest.mark.parametrize("tokens,scheme", [(256, "block_channel"), (16, "block_channel"), (384, "double_channel"), (128, "row_block")])
-def test_graphed_step_replays_match_eager(T, dev, tokens, scheme):
+@pytest.mark.parametrize("tokens,scheme,n_out", [(256, "block_channel", 256), (16, "block_channel", 256), (384, "double_channel", 256),
+                                                 (128, "row_block", 256), (640, "block_channel", 384)])
+def test_graphed_step_replays_match_eager(T, dev, tokens, scheme, n_out):
     """A whole fwd+bwd step captured into a HIP graph: every replay, with eager work and device
-    synchronisations in between and with new inputs, must equal the eager result bit for bit."""
+    synchronisations in between and with new inputs, must equal the eager result bit for bit.  (The last case has more
+    than 256 tokens and output features: its Y, dX and dW GEMMs are one launch.)"""
     g = make_gen(40 + tokens)
-    W = randn_bf16(g, 256, 512, std=0.02).to(dev)
-    mk = lambda: (randn_bf16(g, tokens, 512).to(dev), randn_bf16(g, tokens, 256, std=1e-3).to(dev))
+    W = randn_bf16(g, n_out, 512, std=0.02).to(dev)
+    mk = lambda: (randn_bf16(g, tokens, 512).to(dev), randn_bf16(g, tokens, n_out, std=1e-3).to(dev))
     X0, dY0 = mk()
     step = T.GraphedStep(lambda x, w, dy: T.linear_fwd_bwd(x, w, dy, scheme), X0, W, dY0)
     for it in range(4):
