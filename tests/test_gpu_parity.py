@@ -126,6 +126,14 @@ def test_gemms_of_a_step_in_one_launch(T, dev):
     Y0, saved = T.linear.linear_forward(X, W, "block_channel")
     dX0, dW0 = T.linear.linear_backward(dY, X, W, "block_channel", None, saved)
     assert torch.equal(Y, Y0) and torch.equal(dX, dX0) and torch.equal(dW, dW0)
+    # the other modes that run a step's GEMMs as one launch
+    for scheme, had in (("block_channel", 128), ("row_block", None), ("row_block", 128)):
+        with T._lib.timed_launches() as rec:
+            Y, dX, dW = T.linear_fwd_bwd(X, W, dY, scheme, had)
+        assert len(rec["ti8_gemm_i8_nt_multi"]) == 1 and "ti8_gemm_i8_nt" not in rec, (scheme, had)
+        Y0, saved = T.linear.linear_forward(X, W, scheme, had)
+        dX0, dW0 = T.linear.linear_backward(dY, X, W, scheme, had, saved)
+        assert torch.equal(Y, Y0) and torch.equal(dX, dX0) and torch.equal(dW, dW0), (scheme, had)
     # a ragged token count is padded to the tile before the launch
     Yr, dXr, dWr = T.linear_fwd_bwd(X[:300], W, dY[:300], "block_channel")
     Y1, saved = T.linear.linear_forward(T.linear.pad_tokens(X[:300]), W, "block_channel")

@@ -58,8 +58,21 @@ def _live_rows(a_q, tokens):
     return min(rows, -(-tokens // 32) * 32)
 
 
-def _gemm_bc(a_q, a_s, a_mode, b_q, b_s, b_mode, out_scale=1.0, tokens=None):
-    """2-D operands through the batched block-channel GEMM (batch of one)."""
+def _deferred(gemms, problem):
+    """Queue one 2-D GEMM for the launch that ends a whole step (``linear_fwd_bwd``); returns its output tensor,
+    which holds the result once that launch has run."""
+    M, N = problem["A"].shape[0], problem["B"].shape[0]
+    problem["out"] = torch.empty((M, N), dtype=torch.bfloat16, device=problem["A"].device)
+    gemms.append(problem)
+    return problem["out"]
+
+
+def _gemm_bc(a_q, a_s, a_mode, b_q, b_s, b_mode, out_scale=1.0, tokens=None, gemms=None):
+    """2-D operands through the batched block-channel GEMM (batch of one); with ``gemms`` (a list) the GEMM is
+    queued there instead of launched."""
+    if gemms is not None:
+        return _deferred(gemms, dict(A=a_q, B=b_q, sA=a_s.reshape(-1) if a_mode == SCALE_ROW else a_s, modeA=a_mode,
+                                     sB=b_s.reshape(-1) if b_mode == SCALE_ROW else b_s, modeB=b_mode, out_scale=out_scale))
     rows = _live_rows(a_q, tokens)
     a_q = a_q[:rows]
     a_s3 = a_s[:rows].reshape(1, -1) if a_mode == SCALE_ROW else a_s[None]
@@ -67,7 +80,10 @@ def _gemm_bc(a_q, a_s, a_mode, b_q, b_s, b_mode, out_scale=1.0, tokens=None):
                           out_scale=out_scale)[0]
 
 
-def _gemm_dc(a_q, a_s, b_q, b_s, post_scale=0.0, tokens=None):
+def _gemm_dc(a_q, a_s, b_q, b_s, post_scale=0.0, tokens=None, gemms=None):
+    if gemms is not None:
+        return _deferred(gemms, dict(A=a_q, B=b_q, sA=a_s.reshape(-1), modeA=SCALE_ROW, sB=b_s.reshape(-1), modeB=SCALE_ROW,
+                                     acc_i32_full=True, post_scale=post_scale))
     rows = _live_rows(a_q, tokens)
     return ops.gemm_i8_nt(a_q[:rows][None], b_q, a_s[:rows].reshape(1, -1), SCALE_ROW, b_s, SCALE_ROW, acc_i32_full=True,
                           post_scale=post_scale)[0]
@@ -100,14 +116,15 @@ def quantize_weight(W, scheme="block_channel", hadamard=None):
     return ops.quant_row(ops.fwht(W) if hadamard == "full" else W, clamp=True, inv_mode=INV_AMAX_DIV_127)
 
 
-def linear_forward(X2, W, scheme="block_channel", hadamard=None, need_backward=True, wq=None, tokens=None, xq=None):
+def linear_forward(X2, W, scheme="block_channel", hadamard=None, need_backward=True, wq=None, tokens=None, xq=None, gemms=None):
     """X2 bf16 [T, K] (tokens flattened), W bf16 [N, K] -> (Y bf16 [T, N], saved) where
     ``saved`` holds what the backward can reuse: operands the forward quantises anyway are
     quantised for the backward GEMMs in the same pass (transposed copies, column-wise scales)
     unless ``need_backward`` is false.  ``wq`` = :func:`quantize_weight` of W computed earlier
     (forward-only use; W itself is then not read).  ``tokens`` = number of real rows of X2 when the
     caller has zero-padded it: with few tokens the GEMM skips the padding rows.  ``xq`` = ``(q, qT, s)`` of
-    ``ops.quant_block(X2[None], with_transpose=True)`` computed earlier ("block_channel" without rotation only)."""
+    ``ops.quant_block(X2[None], with_transpose=True)`` computed earlier ("block_channel" without rotation only).
+    ``gemms`` = a list: the GEMM is queued there instead of launched (see :func:`linear_fwd_bwd`)."""
     _check(scheme, hadamard)
     saved = {}
     if wq is not None and need_backward:
@@ -116,35 +133,35 @@ def linear_forward(X2, W, scheme="block_channel", hadamard=None, need_backward=T
         if hadamard == 128:
             q, s = ops.quant_block_had128(X2[None], clamp=True)
             wq, ws = wq if wq is not None else quantize_weight(W, scheme, hadamard)
-            return _gemm_bc(q[0], s[0], SCALE_BLOCK128, wq, ws, SCALE_ROW, 2.0 ** -7, tokens=tokens), saved
+            return _gemm_bc(q[0], s[0], SCALE_BLOCK128, wq, ws, SCALE_ROW, 2.0 ** -7, tokens=tokens, gemms=gemms), saved
         if not need_backward:
             q, s = ops.quant_block(X2[None], clamp=True)
             wq, ws = wq if wq is not None else quantize_weight(W, scheme, hadamard)
-            return _gemm_bc(q[0], s[0], SCALE_BLOCK128, wq, ws, SCALE_ROW, tokens=tokens), saved
+            return _gemm_bc(q[0], s[0], SCALE_BLOCK128, wq, ws, SCALE_ROW, tokens=tokens, gemms=gemms), saved
         q, qT, s = xq if xq is not None else ops.quant_block(X2[None], clamp=True, with_transpose=True)
         saved["XqT"], saved["Xs"] = qT[0], s[0]
         wq, ws, saved["WtQ"], saved["Wts"] = _row_col(W, clamp=True)   # rows for Y, columns for dX
-        return _gemm_bc(q[0], s[0], SCALE_BLOCK128, wq, ws, SCALE_ROW, tokens=tokens), saved
+        return _gemm_bc(q[0], s[0], SCALE_BLOCK128, wq, ws, SCALE_ROW, tokens=tokens, gemms=gemms), saved
     if scheme == "row_block":
         q, s = ops.quant_row(X2, clamp=True, hadamard128=(hadamard == 128))
         if hadamard == 128 or not need_backward:
             wq, ws = wq if wq is not None else quantize_weight(W, scheme, hadamard)
-            return _gemm_bc(q, s, SCALE_ROW, wq, ws, SCALE_BLOCK128, 2.0 ** -7 if hadamard == 128 else 1.0, tokens=tokens), saved
+            return _gemm_bc(q, s, SCALE_ROW, wq, ws, SCALE_BLOCK128, 2.0 ** -7 if hadamard == 128 else 1.0, tokens=tokens, gemms=gemms), saved
         wq, wqT, ws = ops.quant_block(W[None], clamp=True, with_transpose=True)
         saved["WqT"], saved["Ws"] = wqT[0], ws[0]
-        return _gemm_bc(q, s, SCALE_ROW, wq[0], ws[0], SCALE_BLOCK128, tokens=tokens), saved
+        return _gemm_bc(q, s, SCALE_ROW, wq[0], ws[0], SCALE_BLOCK128, tokens=tokens, gemms=gemms), saved
     # double_channel
     K = X2.shape[1]
     if hadamard == "full" or not need_backward:
         q, s = ops.quant_row(ops.fwht(X2) if hadamard == "full" else X2, clamp=True, inv_mode=INV_AMAX_DIV_127)
         wq, ws = wq if wq is not None else quantize_weight(W, scheme, hadamard)
-        return _gemm_dc(q, s, wq, ws, 1.0 / K if hadamard == "full" else 0.0, tokens=tokens), saved
+        return _gemm_dc(q, s, wq, ws, 1.0 / K if hadamard == "full" else 0.0, tokens=tokens, gemms=gemms), saved
     q, s, saved["XtQ"], saved["Xts"] = _row_col(X2, clamp=True, inv_mode=INV_AMAX_DIV_127)
     wq, ws, saved["WtQ"], saved["Wts"] = _row_col(W, clamp=True, inv_mode=INV_AMAX_DIV_127)
-    return _gemm_dc(q, s, wq, ws, tokens=tokens), saved
+    return _gemm_dc(q, s, wq, ws, tokens=tokens, gemms=gemms), saved
 
 
-def linear_backward(dY2, X2, W, scheme="block_channel", hadamard=None, saved=None, tokens=None):
+def linear_backward(dY2, X2, W, scheme="block_channel", hadamard=None, saved=None, tokens=None, gemms=None):
     """dY2 bf16 [T, N], X2 bf16 [T, K], W bf16 [N, K] -> (dX bf16 [T, K], dW bf16 [N, K])."""
     _check(scheme, hadamard)
     saved = saved or {}
@@ -155,35 +172,34 @@ def linear_backward(dY2, X2, W, scheme="block_channel", hadamard=None, saved=Non
             # H_128 along N for dX, along the tokens for dW: two differently rotated copies
             dq, ds = ops.quant_block_had128(dY2[None], clamp=True)
             wtq, wts = ops.quant_col_t(W, clamp=True, hadamard128=True)   # W^T [K,N] per row, rotated along N
-            dX = _gemm_bc(dq[0], ds[0], SCALE_BLOCK128, wtq, wts, SCALE_ROW, 2.0 ** -7, tokens=tokens)
+            dX = _gemm_bc(dq[0], ds[0], SCALE_BLOCK128, wtq, wts, SCALE_ROW, 2.0 ** -7, tokens=tokens, gemms=gemms)
             # the token-dim rotation is fused too: one read of dY / X, transposed int8 out
             dyt, dyts = ops.quant_block_had128(dY2[None], along_rows=True, clamp=False)
             xt, xts = ops.quant_block_had128(X2[None], along_rows=True, clamp=False)
-            dW = ops.gemm_i8_nt(dyt, xt, dyts.transpose(1, 2), SCALE_BLOCK128, xts.transpose(1, 2), SCALE_BLOCK128,
-                                out_scale=2.0 ** -7)[0]
+            dW = _gemm_bc(dyt[0], dyts[0].t(), SCALE_BLOCK128, xt[0], xts[0].t(), SCALE_BLOCK128, 2.0 ** -7, gemms=gemms)
             return dX, dW
         dq, dqT, ds = saved["dYq"] if "dYq" in saved else ops.quant_block(dY2[None], clamp=True, with_transpose=True)
         if "WtQ" in saved:
             wtq, wts = saved["WtQ"], saved["Wts"]
         else:
             wtq, wts = ops.quant_col_t(W, clamp=True)                # W^T [K,N] per row
-        dX = _gemm_bc(dq[0], ds[0], SCALE_BLOCK128, wtq, wts, SCALE_ROW, tokens=tokens)
+        dX = _gemm_bc(dq[0], ds[0], SCALE_BLOCK128, wtq, wts, SCALE_ROW, tokens=tokens, gemms=gemms)
         if "XqT" in saved:
             xqT, xs = saved["XqT"], saved["Xs"]
         else:
             _, xqT3, xs3 = ops.quant_block(X2[None], clamp=True, with_transpose=True)
             xqT, xs = xqT3[0], xs3[0]
         # scales of the transposed operands are the transposed scale grids
-        dW = ops.gemm_i8_nt(dqT, xqT[None], ds.transpose(1, 2), SCALE_BLOCK128, xs.t()[None], SCALE_BLOCK128)[0]
+        dW = _gemm_bc(dqT[0], ds[0].t(), SCALE_BLOCK128, xqT, xs.t(), SCALE_BLOCK128, gemms=gemms)
         return dX, dW
     if scheme == "row_block":
         if hadamard == 128:
             dq, ds = ops.quant_row(dY2, clamp=True, hadamard128=True)
             wtq, wts = ops.quant_block_had128(W[None], along_rows=True, clamp=True)      # W^T [K,N], groups along N
-            dX = _gemm_bc(dq, ds, SCALE_ROW, wtq[0], wts[0].t(), SCALE_BLOCK128, 2.0 ** -7, tokens=tokens)
+            dX = _gemm_bc(dq, ds, SCALE_ROW, wtq[0], wts[0].t(), SCALE_BLOCK128, 2.0 ** -7, tokens=tokens, gemms=gemms)
             dytq, dyts = ops.quant_col_t(dY2, clamp=True, hadamard128=True)   # dY^T [N,T] per row, rotated along the tokens
             xtq, xts = ops.quant_block_had128(X2[None], along_rows=True, clamp=True)
-            dW = _gemm_bc(dytq, dyts, SCALE_ROW, xtq[0], xts[0].t(), SCALE_BLOCK128, 2.0 ** -7)
+            dW = _gemm_bc(dytq, dyts, SCALE_ROW, xtq[0], xts[0].t(), SCALE_BLOCK128, 2.0 ** -7, gemms=gemms)
             return dX, dW
         dq, ds, dytq, dyts = _row_col(dY2, clamp=True)    # rows for dX, columns (dY^T [N,T] per row) for dW
         if "WqT" in saved:
@@ -191,9 +207,9 @@ def linear_backward(dY2, X2, W, scheme="block_channel", hadamard=None, saved=Non
         else:
             _, wqT3, ws3 = ops.quant_block(W[None], clamp=True, with_transpose=True)
             wqT, ws = wqT3[0], ws3[0]
-        dX = _gemm_bc(dq, ds, SCALE_ROW, wqT, ws.t(), SCALE_BLOCK128, tokens=tokens)
+        dX = _gemm_bc(dq, ds, SCALE_ROW, wqT, ws.t(), SCALE_BLOCK128, tokens=tokens, gemms=gemms)
         _, xqT, xs = ops.quant_block(X2[None], clamp=True, with_transpose=True)
-        dW = _gemm_bc(dytq, dyts, SCALE_ROW, xqT[0], xs[0].t(), SCALE_BLOCK128)
+        dW = _gemm_bc(dytq, dyts, SCALE_ROW, xqT[0], xs[0].t(), SCALE_BLOCK128, gemms=gemms)
         return dX, dW
     # double_channel
     if hadamard == "full":
@@ -202,22 +218,22 @@ def linear_backward(dY2, X2, W, scheme="block_channel", hadamard=None, saved=Non
         # full-length rotation along the tokens (as in the reference, whose transform needs a power of two)
         dq, ds = ops.quant_row(ops.fwht(dY2), clamp=True, inv_mode=INV_AMAX_DIV_127)
         wtq, wts = ops.quant_row(ops.fwht_t(W), clamp=True, inv_mode=INV_AMAX_DIV_127)
-        dX = _gemm_dc(dq, ds, wtq, wts, 1.0 / N, tokens=tokens)
+        dX = _gemm_dc(dq, ds, wtq, wts, 1.0 / N, tokens=tokens, gemms=gemms)
         dytq, dyts = ops.quant_row(ops.fwht_t(dY2), clamp=True, inv_mode=INV_AMAX_DIV_127)
         xtq, xts = ops.quant_row(ops.fwht_t(X2), clamp=True, inv_mode=INV_AMAX_DIV_127)
-        dW = _gemm_dc(dytq, dyts, xtq, xts, 1.0 / T)
+        dW = _gemm_dc(dytq, dyts, xtq, xts, 1.0 / T, gemms=gemms)
         return dX, dW
     dq, ds, dytq, dyts = _row_col(dY2, clamp=True, inv_mode=INV_AMAX_DIV_127)
     if "WtQ" in saved:
         wtq, wts = saved["WtQ"], saved["Wts"]
     else:
         wtq, wts = ops.quant_col_t(W, clamp=True, inv_mode=INV_AMAX_DIV_127)
-    dX = _gemm_dc(dq, ds, wtq, wts, tokens=tokens)
+    dX = _gemm_dc(dq, ds, wtq, wts, tokens=tokens, gemms=gemms)
     if "XtQ" in saved:
         xtq, xts = saved["XtQ"], saved["Xts"]
     else:
         xtq, xts = ops.quant_col_t(X2, clamp=True, inv_mode=INV_AMAX_DIV_127)
-    dW = _gemm_dc(dytq, dyts, xtq, xts)
+    dW = _gemm_dc(dytq, dyts, xtq, xts, gemms=gemms)
     return dX, dW
 
 
@@ -235,33 +251,11 @@ def pad_tokens(x2, multiple=128):
     return out
 
 
-# Schemes whose whole step (linear_fwd_bwd, no rotation, more than 256 tokens and output features) runs its three GEMMs as one
-# launch (ops.gemm_i8_nt_multi; same kernels on the same operands, so the same bits as linear_forward +
-# linear_backward).  Measured at 8192 tokens, K = N = 4096: block_channel 0.497 -> 0.482 ms per step;
-# double_channel, which the function also serves, gains nothing (0.445 -> 0.448) and stays on three launches.
-ONE_LAUNCH_SCHEMES = ("block_channel",)
-
-
-def _step_one_launch(X2, W, dY2, scheme):
-    """(Y, dX, dW) of padded 2-D operands with more than 256 tokens, without rotation: the quantisers of
-    linear_forward / linear_backward, then Y, dX and dW in one GEMM launch."""
-    if scheme == "block_channel":
-        (xq, xqT, xs), (dq, dqT, ds) = ops.quant_block_multi([X2[None], dY2[None]], clamp=True, with_transpose=True)
-        wq, ws, wtq, wts = _row_col(W, clamp=True)
-        blk, row = dict(modeA=SCALE_BLOCK128), dict(modeB=SCALE_ROW)
-        return ops.gemm_i8_nt_multi([
-            dict(A=xq[0], B=wq, sA=xs[0], sB=ws, **blk, **row),
-            dict(A=dq[0], B=wtq, sA=ds[0], sB=wts, **blk, **row),
-            # scales of the transposed operands are the transposed scale grids
-            dict(A=dqT[0], B=xqT[0], sA=ds[0].t(), sB=xs[0].t(), **blk, modeB=SCALE_BLOCK128)])
-    kw = dict(clamp=True, inv_mode=INV_AMAX_DIV_127)
-    xq, xs, xtq, xts = _row_col(X2, **kw)
-    wq, ws, wtq, wts = _row_col(W, **kw)
-    dq, ds, dytq, dyts = _row_col(dY2, **kw)
-    rows = dict(modeA=SCALE_ROW, modeB=SCALE_ROW, acc_i32_full=True)
-    return ops.gemm_i8_nt_multi([dict(A=xq, B=wq, sA=xs, sB=ws, **rows),
-                                 dict(A=dq, B=wtq, sA=ds, sB=wts, **rows),
-                                 dict(A=dytq, B=xtq, sA=dyts, sB=xts, **rows)])
+# Schemes whose whole step (linear_fwd_bwd with more than 256 tokens and output features) runs its three GEMMs as
+# one launch (ops.gemm_i8_nt_multi; same kernels on the same operands, so the same bits as linear_forward +
+# linear_backward).  Measured at 8192 tokens, K = N = 4096: block_channel 0.497 -> 0.482 ms per step; double_channel,
+# which the launch also serves, gains nothing (0.445 -> 0.448) and stays on three launches.
+ONE_LAUNCH_SCHEMES = ("block_channel", "row_block")
 
 
 def linear_fwd_bwd(X, W, dY, scheme="block_channel", hadamard=None):
@@ -273,19 +267,22 @@ def linear_fwd_bwd(X, W, dY, scheme="block_channel", hadamard=None):
     X2, dY2 = X.reshape(-1, K), dY.reshape(-1, N)
     T = X2.shape[0]
     X2, dY2 = pad_tokens(X2), pad_tokens(dY2)
-    # (with up to 256 rows - tokens for Y and dX, output features for dW - a GEMM launched alone takes the few-rows kernel)
-    if hadamard is None and scheme in ONE_LAUNCH_SCHEMES and min(X2.shape[0], N) > 256 and ops.GEMM_PATH in ("auto", "tiled", "large"):
-        Y, dX, dW = _step_one_launch(X2, W, dY2, scheme)
-        return Y[:T].reshape(*lead, N), dX[:T].reshape(*lead, K), dW
+    # with up to 256 rows (tokens for Y and dX, output features for dW) a GEMM launched alone takes the few-rows kernel,
+    # which the one launch does not offer; the full-length rotation's GEMMs are left as they are
+    gemms = None
+    if scheme in ONE_LAUNCH_SCHEMES and hadamard != "full" and min(X2.shape[0], N) > 256 and ops.GEMM_PATH in ("auto", "tiled", "large"):
+        gemms = []
     pre = None
     if scheme == "block_channel" and hadamard is None:
         # both activations are at hand: one quantiser launch for X and dY (the forward alone would quantise X, the
         # backward dY, with the same kernel and the same bits)
         pre = ops.quant_block_multi([X2[None], dY2[None]], clamp=True, with_transpose=True)
-    Y, saved = linear_forward(X2, W, scheme, hadamard, tokens=T, xq=pre[0] if pre else None)
+    Y, saved = linear_forward(X2, W, scheme, hadamard, tokens=T, xq=pre[0] if pre else None, gemms=gemms)
     if pre:
         saved["dYq"] = pre[1]
-    dX, dW = linear_backward(dY2, X2, W, scheme, hadamard, saved, tokens=T)
+    dX, dW = linear_backward(dY2, X2, W, scheme, hadamard, saved, tokens=T, gemms=gemms)
+    if gemms:
+        ops.gemm_i8_nt_multi(gemms)   # Y, dX and dW, into the tensors handed out above
     return Y[:T].reshape(*lead, N), dX[:T].reshape(*lead, K), dW
 
 
