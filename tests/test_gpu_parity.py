@@ -134,6 +134,18 @@ def test_gemms_of_a_step_in_one_launch(T, dev):
         Y0, saved = T.linear.linear_forward(X, W, scheme, had)
         dX0, dW0 = T.linear.linear_backward(dY, X, W, scheme, had, saved)
         assert torch.equal(Y, Y0) and torch.equal(dX, dX0) and torch.equal(dW, dW0), (scheme, had)
+    # the autograd backward runs dX and dW as one launch
+    lin = T.Int8Linear(512, 384, device=dev)
+    with torch.no_grad():
+        lin.weight.copy_(W)
+    xg = X.clone().requires_grad_(True)
+    y = lin(xg)
+    with T._lib.timed_launches() as rec:
+        y.backward(dY)
+    assert len(rec["ti8_gemm_i8_nt_multi"]) == 1 and "ti8_gemm_i8_nt" not in rec
+    Y0, saved = T.linear.linear_forward(X, W, "block_channel")
+    dX0, dW0 = T.linear.linear_backward(dY, X, W, "block_channel", None, saved)
+    assert torch.equal(y.detach(), Y0) and torch.equal(xg.grad, dX0) and torch.equal(lin.weight.grad, dW0)
     # a ragged token count is padded to the tile before the launch
     Yr, dXr, dWr = T.linear_fwd_bwd(X[:300], W, dY[:300], "block_channel")
     Y1, saved = T.linear.linear_forward(T.linear.pad_tokens(X[:300]), W, "block_channel")

@@ -258,6 +258,12 @@ def pad_tokens(x2, multiple=128):
 ONE_LAUNCH_SCHEMES = ("block_channel", "row_block")
 
 
+def _one_launch(scheme, hadamard, padded_tokens, out_features):
+    """Whether the GEMMs of a step (or of its backward half) go into one launch.  With up to 256 rows (tokens for Y
+    and dX, output features for dW) a GEMM launched alone takes the few-rows kernel, which the one launch does not offer."""
+    return scheme in ONE_LAUNCH_SCHEMES and min(padded_tokens, out_features) > 256 and ops.GEMM_PATH in ("auto", "tiled", "large")
+
+
 def linear_fwd_bwd(X, W, dY, scheme="block_channel", hadamard=None):
     """One forward + backward of the layer: returns (Y, dX, dW) for X [B,M,K] or [M,K].
     Any number of tokens is accepted (zero-padded to a multiple of 128, see :func:`pad_tokens`);
@@ -267,11 +273,7 @@ def linear_fwd_bwd(X, W, dY, scheme="block_channel", hadamard=None):
     X2, dY2 = X.reshape(-1, K), dY.reshape(-1, N)
     T = X2.shape[0]
     X2, dY2 = pad_tokens(X2), pad_tokens(dY2)
-    # with up to 256 rows (tokens for Y and dX, output features for dW) a GEMM launched alone takes the few-rows kernel,
-    # which the one launch does not offer; the full-length rotation's GEMMs are left as they are
-    gemms = None
-    if scheme in ONE_LAUNCH_SCHEMES and hadamard != "full" and min(X2.shape[0], N) > 256 and ops.GEMM_PATH in ("auto", "tiled", "large"):
-        gemms = []
+    gemms = [] if _one_launch(scheme, hadamard, X2.shape[0], N) else None
     pre = None
     if scheme == "block_channel" and hadamard is None:
         # both activations are at hand: one quantiser launch for X and dY (the forward alone would quantise X, the
@@ -310,7 +312,10 @@ class Int8LinearFunction(torch.autograd.Function):
         x2, weight = ctx.saved_tensors
         N = weight.shape[0]
         dy2 = pad_tokens(dy.reshape(-1, N).contiguous())
-        dx, dw = linear_backward(dy2, x2, weight, ctx.scheme, ctx.hadamard, ctx.saved_q, tokens=ctx.tokens)
+        gemms = [] if _one_launch(ctx.scheme, ctx.hadamard, x2.shape[0], N) else None
+        dx, dw = linear_backward(dy2, x2, weight, ctx.scheme, ctx.hadamard, ctx.saved_q, tokens=ctx.tokens, gemms=gemms)
+        if gemms:
+            ops.gemm_i8_nt_multi(gemms)   # dX and dW in one launch
         db = dy2.sum(dim=0).to(dy.dtype) if ctx.has_bias else None
         return dx[:ctx.tokens].reshape(*dy.shape[:-1], x2.shape[1]), dw, db, None, None
 
