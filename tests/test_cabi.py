@@ -182,3 +182,23 @@ def test_gemm_multi_validation(lib):
     for (p, n, flags), code, msg in cases:
         rc = lib.ti8_gemm_i8_nt_multi(p, n, flags, None)
         assert rc == code and msg in lib.ti8_last_error().decode(), (rc, lib.ti8_last_error(), msg)
+
+
+def test_empty_batch_needs_no_kernel():
+    """Zero tokens: empty Y and dX, a zero weight gradient, as torch.nn.functional.linear gives; no launch, so it runs here."""
+    import torch
+    import triton_int8_amd as T
+    W = torch.randn(256, 128).to(torch.bfloat16)
+    for lead in ((0,), (3, 0), (0, 5)):
+        X, dY = torch.empty(*lead, 128, dtype=torch.bfloat16), torch.empty(*lead, 256, dtype=torch.bfloat16)
+        for scheme in T.linear.SCHEMES:
+            Y, dX, dW = T.linear_fwd_bwd(X, W, dY, scheme)
+            assert Y.shape == (*lead, 256) and dX.shape == (*lead, 128) and dW.shape == W.shape and not dW.any()
+    lin = T.Int8Linear(128, 256, bias=True, device="cpu")
+    x = torch.empty(2, 0, 128, dtype=torch.bfloat16, requires_grad=True)
+    y = lin(x)
+    assert y.shape == (2, 0, 256)
+    y.sum().backward()
+    assert x.grad.shape == x.shape and not lin.weight.grad.any() and not lin.bias.grad.any()
+    with torch.no_grad():
+        assert lin(x.detach()).shape == (2, 0, 256)

@@ -272,6 +272,8 @@ def linear_fwd_bwd(X, W, dY, scheme="block_channel", hadamard=None):
     K, N = X.shape[-1], W.shape[0]
     X2, dY2 = X.reshape(-1, K), dY.reshape(-1, N)
     T = X2.shape[0]
+    if T == 0:   # nothing to multiply: empty Y and dX, a zero weight gradient (as torch.nn.functional.linear gives)
+        return X.new_empty((*lead, N)), X.new_empty((*lead, K)), W.new_zeros((N, K))
     X2, dY2 = pad_tokens(X2), pad_tokens(dY2)
     gemms = [] if _one_launch(scheme, hadamard, X2.shape[0], N) else None
     pre = None
@@ -296,6 +298,10 @@ class Int8LinearFunction(torch.autograd.Function):
         K, N = x.shape[-1], weight.shape[0]
         x2 = x.reshape(-1, K)
         ctx.tokens = x2.shape[0]
+        ctx.has_bias = bias is not None
+        if ctx.tokens == 0:   # an empty batch: empty output, zero gradients
+            ctx.save_for_backward(x2, weight)
+            return x.new_empty((*x.shape[:-1], N))
         x2 = pad_tokens(x2)
         need_bwd = any(ctx.needs_input_grad[:2])
         y, saved = linear_forward(x2, weight, scheme, hadamard, need_backward=need_bwd, tokens=ctx.tokens)
@@ -311,6 +317,8 @@ class Int8LinearFunction(torch.autograd.Function):
     def backward(ctx, dy):
         x2, weight = ctx.saved_tensors
         N = weight.shape[0]
+        if ctx.tokens == 0:
+            return dy.new_empty((*dy.shape[:-1], x2.shape[1])), torch.zeros_like(weight), (dy.new_zeros((N,)) if ctx.has_bias else None), None, None
         dy2 = pad_tokens(dy.reshape(-1, N).contiguous())
         gemms = [] if _one_launch(ctx.scheme, ctx.hadamard, x2.shape[0], N) else None
         dx, dw = linear_backward(dy2, x2, weight, ctx.scheme, ctx.hadamard, ctx.saved_q, tokens=ctx.tokens, gemms=gemms)
@@ -341,6 +349,8 @@ class Int8Linear(torch.nn.Module):
     def forward(self, x):
         if torch.is_grad_enabled() and (x.requires_grad or self.weight.requires_grad):
             return Int8LinearFunction.apply(x, self.weight, self.bias, self.scheme, self.hadamard)
+        if x.numel() == 0:
+            return x.new_empty((*x.shape[:-1], self.out_features))
         # forward only (inference): the weight is quantised once per weight update, not per call
         key = (self.weight._version, self.weight.data_ptr(), self.scheme, self.hadamard)
         if self._wq_key != key:
