@@ -259,7 +259,7 @@ int walk_gemm(int64_t bsa, int64_t lda, int64_t bsb, int64_t ldb, int64_t bsc, i
     const bool CHAIN = EPI == 5, LANEB = EPI == 4, FAST = EPI == 2 || EPI == 4 || EPI == 5;
     const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
     const int nk = (int)(K >> 7), klast = (nk - 1) * 128;
-    const int WCOLS = TN * 32, LPR = WCOLS / 4, RPI = 64 / LPR, NRR = 32 / RPI;
+    const int WCOLS = TN * 32, LPR = WCOLS / 8, RPI = 64 / LPR, NRR = 32 / RPI;
     const int GROUP = gemm_group_rows(BM);
     (void)CHAIN;
     std::vector<uint8_t> stored(c_elems <= (int64_t)1 << 30 ? (size_t)c_elems : 0, 0);
@@ -330,33 +330,45 @@ int walk_gemm(int64_t bsa, int64_t lda, int64_t bsb, int64_t ldb, int64_t bsc, i
                                     }
                                 }
                     }
-                    // ---- epilogue (gemm.hip: coln, prow0 / rm_all, store_tile)
-                    const int rb_col = epi_col_of_lane(lane, WCOLS), rb_row = epi_row_of_lane(lane, WCOLS);
-                    const int ncol0 = n0 + wn * WCOLS + rb_col;
+                    // ---- epilogue (gemm.hip: coln, cm, prow0 / rm_all, store_tile)
                     const bool col_part = EPI == 1 || (FAST && sb.mode == 0), row_part = EPI == 1 || (FAST && sa.mode == 0);
-                    if (EPI == 1 || FAST) {
+                    if (EPI == 1 || FAST) {   // column scales, fetched before the main loop by every wave
                         const int64_t cs = col_part ? sb.rs : 0;
+                        const int ncol0 = n0 + wn * WCOLS + epi_scale_col_of_lane(lane);
                         for (int c = 0; c < 4; ++c) r.access("gemm column scale", epi_col_scale_index(by, sb.bs, ncol0 + c, (int)N, cs), 1, sb.elems, bx, wave, lane, c);
                     }
-                    const int64_t rstride = row_part ? sa.rs : 0;
+                    // a wave whose tile lies outside the output stops here
+                    if (m0 + wm * TM * 32 >= M || n0 + wn * WCOLS >= N) continue;
+                    const int rb_col = epi_col_of_lane(lane, WCOLS), rb_row = epi_row_of_lane(lane, WCOLS);
+                    for (int c = 0; c < 8; ++c) {   // the lane that holds this lane's column scale c, and the column it fetched
+                        const int src = epi_scale_lane(lane, c);
+                        if (src < 0 || src >= 64 || epi_scale_col_of_lane(src) + (c & 3) != rb_col + c)
+                            r.fail("gemm: lane %d takes column scale %d from lane %d, which holds column %d, not %d", lane, c, src,
+                                   epi_scale_col_of_lane(src) + (c & 3), rb_col + c);
+                    }
                     const int row0 = m0 + wm * TM * 32 + rb_row;
-                    const bool col_ok = ncol0 < N;
-                    const uint32_t rs32 = (uint32_t)rstride;
-                    const uint32_t r_lim = epi_row_scale_limit(row0, (int)M, rs32);
-                    const bool mult = FAST && (row_part || col_part);
-                    if (EPI == 1 || (FAST && mult)) {
-                        const int64_t base = epi_row_scale_base(by, sa.bs, row0, (int)M, rstride);
+                    if (row_part) {
+                        const int64_t base = epi_row_scale_base(by, sa.bs, row0, sa.rs);
                         for (int i = 0; i < TM; ++i)
                             for (int k = 0; k < NRR; ++k)
-                                r.access("gemm row scale", base + epi_row_scale_rel(i * 32 + k * RPI, rs32, r_lim), 1, sa.elems, bx, wave, lane, i * NRR + k);
+                                r.access("gemm row scale", base + (int64_t)(i * 32 + k * RPI) * sa.rs, 1, sa.elems, bx, wave, lane, i * NRR + k);
                     }
-                    int64_t off = epi_out_offset(by, bsc, row0, ldc, ncol0);
+                    // slab: 32 rows of EPI_SLAB_LD words per wave, inside the operand buffers
+                    for (int e = 0; e < 16; ++e)
+                        for (int j = 0; j < TN; ++j) {
+                            const int rr = 8 * (e >> 2) + 4 * fr_half + (e & 3);
+                            r.access("gemm slab write", (int64_t)wave * 32 * EPI_SLAB_LD(WCOLS) + rr * EPI_SLAB_LD(WCOLS) + j * 32 + fr_row, 1,
+                                     (2 * (A_BYTES + B_BYTES)) / 4, bx, wave, lane, e);
+                        }
+                    for (int k = 0; k < NRR; ++k)
+                        r.access("gemm slab read", (int64_t)wave * 32 * EPI_SLAB_LD(WCOLS) + (rb_row + k * RPI) * EPI_SLAB_LD(WCOLS) + rb_col, 8,
+                                 (2 * (A_BYTES + B_BYTES)) / 4, bx, wave, lane, k);
+                    int64_t off = epi_out_offset(by, bsc, row0, ldc, n0 + wn * WCOLS + rb_col);
                     const int64_t c_step = (int64_t)RPI * ldc;
                     for (int i = 0; i < TM; ++i)
                         for (int k = 0; k < NRR; ++k, off += c_step) {
-                            if (row0 + i * 32 + k * RPI >= M || !col_ok) continue;
-                            if (r.access("gemm C", off, 4, c_elems, bx, wave, lane, i * NRR + k) && !stored.empty())
-                                for (int c = 0; c < 4; ++c) ++stored[(size_t)(off + c)];
+                            if (r.access("gemm C", off, 8, c_elems, bx, wave, lane, i * NRR + k) && !stored.empty())
+                                for (int c = 0; c < 8; ++c) ++stored[(size_t)(off + c)];
                         }
                 }
             }

@@ -102,23 +102,24 @@ TI8_HD int64_t gemm_factor_index(int64_t batch, int64_t bs, int block, int64_t r
     return batch * bs + (int64_t)block * rs + (int64_t)(kt >> shift) * ks;
 }
 
-// epilogue: a wave stores its tile 32 rows at a time; with wcols columns per wave tile a row of
-// the tile takes lpr = wcols / 4 lanes (4 columns each) and one instruction covers rpi = 64 / lpr rows
-TI8_HD int epi_col_of_lane(int lane, int wcols) { return (lane % (wcols / 4)) * 4; }
-TI8_HD int epi_row_of_lane(int lane, int wcols) { return lane / (wcols / 4); }
+// epilogue: a wave stores its tile 32 rows at a time through an LDS slab; with wcols columns per
+// wave tile a row of the tile takes lpr = wcols / 8 lanes (8 columns each) and one instruction
+// covers rpi = 64 / lpr rows.  Slab rows are padded by 4 words.
+constexpr int EPI_SLAB_LD(int wcols) { return wcols + 4; }
+TI8_HD int epi_col_of_lane(int lane, int wcols) { return (lane % (wcols / 8)) * 8; }
+TI8_HD int epi_row_of_lane(int lane, int wcols) { return lane / (wcols / 8); }
+// the column scales are fetched before the main loop, 4 per lane: lane l those of the wave tile's
+// columns 4 (l % 16) .. + 3; in the epilogue the lane that stores columns 8 q .. 8 q + 7 (q = lane % 8)
+// takes scale c of them from lane 2 q + c / 4 (register c % 4 there)
+TI8_HD int epi_scale_col_of_lane(int lane) { return (lane % 16) * 4; }
+TI8_HD int epi_scale_lane(int lane, int c) { return 2 * (lane % 8) + (c >> 2); }
 // index of the column scale of column `col` (clamped to the last column; stride 0 when absent)
 TI8_HD int64_t epi_col_scale_index(int64_t batch, int64_t bs, int col, int ncols, int64_t cs) {
     return batch * bs + (int64_t)imin(col, ncols - 1) * cs;
 }
-// row-scale offsets are kept in 32 bits relative to the lane's first row: d * stride clamped to
-// the distance to the last row
-TI8_HD int64_t epi_row_scale_base(int64_t batch, int64_t bs, int row0, int rows, int64_t rs) {
-    return batch * bs + (int64_t)imin(row0, rows - 1) * rs;
-}
-TI8_HD uint32_t epi_row_scale_limit(int row0, int rows, uint32_t rs32) { return (uint32_t)imax(rows - 1 - row0, 0) * rs32; }
-TI8_HD uint32_t epi_row_scale_rel(int d, uint32_t rs32, uint32_t limit) {
-    const uint32_t o = (uint32_t)d * rs32;
-    return o < limit ? o : limit;
+// per-row scale of A of this lane's first output row (only waves whose tile lies inside the output get here)
+TI8_HD int64_t epi_row_scale_base(int64_t batch, int64_t bs, int row0, int64_t rs) {
+    return batch * bs + (int64_t)row0 * rs;
 }
 // output element offset of (batch, row0, col0) and the step between the rows one lane stores
 TI8_HD int64_t epi_out_offset(int64_t batch, int64_t bsc, int row0, int64_t ldc, int col0) {
