@@ -259,12 +259,12 @@ def main():
         g = [a.elapsed_time(b) for a, b in rec["ti8_gemm_i8_nt_multi"]]
         assert len(g) == ev_steps
         gemm_ms, gemms_per_launch = [sum(g) / ev_steps], 3
-        kernel = "gemm_i8_multi_kernel<256,256,2,4,EPI_PROMOTE_CHAIN>"
+        kernel = "gemm_i8_chain_kernel (persistent workgroups, 256x256 tiles, chained block-channel promotion)"
     else:
         g = [a.elapsed_time(b) for a, b in rec["ti8_gemm_i8_nt"]]
         assert len(g) == 3 * ev_steps
         gemm_ms, gemms_per_launch = [sum(g[i::3]) / ev_steps for i in range(3)], 1
-        kernel = "gemm_i8_kernel<256,256,2,4,EPI_ROWS>" if args.scheme == "double_channel" else "gemm_i8_kernel<256,256,2,4,EPI_PROMOTE_CHAIN>"
+        kernel = "gemm_i8_kernel<256,256,2,4,EPI_ROWS>" if args.scheme == "double_channel" else "gemm_i8_chain_kernel (persistent workgroups, 256x256 tiles, chained block-channel promotion)"
     avg_ms = sum(gemm_ms) / len(gemm_ms)
     ops_per_launch = gemms_per_launch * 2.0 * M * N * K
     achieved = ops_per_launch / (avg_ms * 1e-3) / 1e12

@@ -397,6 +397,106 @@ int walk_gemm(int64_t bsa, int64_t lda, int64_t bsb, int64_t ldb, int64_t bsc, i
     return r.bad;
 }
 
+// Persistent chained kernel (gemm_chain.hip: gemm_i8_chain_kernel) on one GEMM with `batch` batches and `grid`
+// workgroups: workgroup w walks tiles w, w + grid, ...; a tile's K tiles are fetched by its own iterations except
+// K tiles 0 and 1, which the previous tile's last iterations (or, for a workgroup's first tile, its start) fetch, and
+// the workgroup's last tile fetches its own K tiles 0 and 1 once more.  Checked: every tile of every batch is taken
+// exactly once, every global -> LDS load, scale load, slab access and store lies inside its buffer, every element
+// of C is stored exactly once.
+int walk_gemm_chain(int64_t bsa, int64_t lda, int64_t bsb, int64_t ldb, int64_t bsc, int64_t ldc, const ScaleArg* sa_in,
+                    const ScaleArg* sb_in, int64_t batch, int64_t M, int64_t N, int64_t K, int grid, int64_t a_elems,
+                    int64_t b_elems, int64_t c_elems, int64_t* n_checked, char* msg, int msglen) {
+    Report r{msg, msglen};
+    const ScaleArg sa = *sa_in, sb = *sb_in;
+    const int BM = 256, BN = 256, WN = 4, NW = 8, TM = 4, TN = 2, A_INSTR = 4, B_INSTR = 4, WCOLS = 64, RPI = 8;
+    const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN), per_batch = tiles_m * tiles_n;
+    const int total = per_batch * (int)batch, nk = (int)(K >> 7), GROUP = gemm_group_rows(BM);
+    const int64_t lds_words = (2 * (BM + BN) * 128 + NW * 16 * WCOLS * 4) / 4, slab0 = 2 * (BM + BN) * 128 / 4;
+    if (nk < 2 || nk > 64) { r.fail("gemm chain: K / 128 = %d outside [2, 64]", nk); *n_checked = 0; return 1; }
+    std::vector<uint8_t> stored(c_elems <= (int64_t)1 << 30 ? (size_t)c_elems : 0, 0);
+    std::vector<uint8_t> seen((size_t)total, 0);
+    const bool a_in = sa.mode != 0, b_in = sb.mode != 0;
+    for (int w = 0; w < grid && !r.bad; ++w)
+        for (int T = w; T < total && !r.bad; T += grid) {
+            ++seen[(size_t)T];
+            const int64_t by = T / per_batch;
+            const TileCoord tc = gemm_tile_of(T - (int)by * per_batch, tiles_m, tiles_n, GROUP);
+            if (tc.tile_m < 0 || tc.tile_m >= tiles_m || tc.tile_n < 0 || tc.tile_n >= tiles_n) {
+                r.fail("gemm chain: tile %d maps to (%d, %d) outside %d x %d", T, tc.tile_m, tc.tile_n, tiles_m, tiles_n);
+                break;
+            }
+            const int m0 = tc.tile_m * BM, n0 = tc.tile_n * BN;
+            for (int wave = 0; wave < NW; ++wave) {
+                const int wm = wave / WN, wn = wave % WN;
+                const int rA0 = gemm_wave_first_row(m0, wave, A_INSTR, (int)M), rB0 = gemm_wave_first_row(n0, wave, B_INSTR, (int)N);
+                const int tA0 = wave * A_INSTR, tB0 = wave * B_INSTR;
+                const int kts[4] = {0, 1, nk - 2, nk - 1};
+                for (int lane = 0; lane < 64; ++lane) {
+                    for (int q = 0; q < 4; ++q) {
+                        const int koff = kts[q] * 128;
+                        for (int i = 0; i < A_INSTR; ++i) {
+                            const uint32_t vo = gemm_lane_offset_bytes(lane, (tA0 + i) & 1, (int)lda);
+                            r.access("gemm chain A", by * bsa + gemm_load_offset_bytes(rA0, lda, koff, i, vo), 16, a_elems, T, wave, lane, kts[q]);
+                        }
+                        for (int i = 0; i < B_INSTR; ++i) {
+                            const uint32_t vo = gemm_lane_offset_bytes(lane, (tB0 + i) & 1, (int)ldb);
+                            r.access("gemm chain B", by * bsb + gemm_load_offset_bytes(rB0, ldb, koff, i, vo), 16, b_elems, T, wave, lane, kts[q]);
+                        }
+                    }
+                    // per-K-tile factors: scalar base + (K tile >> shift) * stride per lane
+                    const int64_t fa = gemm_factor_index(by, sa.bs, gemm_factor_block(m0 + wm * TM * 32, (int)M), sa.rs, 0, 0, 0);
+                    const int64_t fb = gemm_factor_index(by, sb.bs, gemm_factor_block(n0 + wn * TN * 32, (int)N), sb.rs, 0, 0, 0);
+                    const uint32_t kt = (uint32_t)gemm_factor_kt(0, lane, nk);
+                    r.access("gemm chain factor A", fa + (int64_t)((kt >> (sa.mode == 3 ? 1 : 0)) * (uint32_t)(a_in ? sa.ks : 0)), 1, sa.elems, T, wave, lane, 0);
+                    r.access("gemm chain factor B", fb + (int64_t)((kt >> (sb.mode == 3 ? 1 : 0)) * (uint32_t)(b_in ? sb.ks : 0)), 1, sb.elems, T, wave, lane, 0);
+                    // column scales: 4 per lane from the wave tile's first column (clamped for a tile outside N)
+                    const uint32_t cs = b_in ? 0u : (uint32_t)sb.rs;
+                    const int64_t colp = epi_col_scale_index(by, sb.bs, chain_col_scale_first(n0 + wn * WCOLS, (int)N), (int)N, cs);
+                    for (int c = 0; c < 4; ++c)
+                        r.access("gemm chain column scale", colp + (int64_t)(((uint32_t)epi_scale_col_of_lane(lane) + c) * cs), 1, sb.elems, T, wave, lane, c);
+                    if (m0 + wm * TM * 32 >= M || n0 + wn * WCOLS >= N) continue;   // this wave stores nothing
+                    const int rb_col = epi_col_of_lane(lane, WCOLS), rb_row = epi_row_of_lane(lane, WCOLS);
+                    for (int c = 0; c < 8; ++c) {
+                        const int src = epi_scale_lane(lane, c);
+                        if (src < 0 || src >= 64 || epi_scale_col_of_lane(src) + (c & 3) != rb_col + c)
+                            r.fail("gemm chain: lane %d takes column scale %d from lane %d", lane, c, src);
+                    }
+                    const int row0 = m0 + wm * TM * 32 + rb_row;
+                    if (!a_in) {
+                        const int64_t base = epi_row_scale_base(by, sa.bs, row0, sa.rs);
+                        for (int q = 0; q < TM * 4; ++q) r.access("gemm chain row scale", base + (int64_t)(q * RPI) * sa.rs, 1, sa.elems, T, wave, lane, q);
+                    }
+                    const int fr_row = lane & 31, fr_half = lane >> 5;
+                    for (int e = 0; e < 8; ++e)
+                        for (int j = 0; j < TN; ++j)
+                            r.access("gemm chain slab write", slab0 + wave * 16 * WCOLS + epi_chain_slab_word(epi_chain_slab_row(e, fr_half), j * 32 + fr_row), 1,
+                                     lds_words, T, wave, lane, e);
+                    for (int k = 0; k < 2; ++k)
+                        for (int half = 0; half < 2; ++half)
+                            r.access("gemm chain slab read", slab0 + wave * 16 * WCOLS + epi_chain_slab_word(rb_row + k * RPI, rb_col + 4 * half), 4, lds_words,
+                                     T, wave, lane, k);
+                    int64_t off = epi_out_offset(by, bsc, row0, ldc, n0 + wn * WCOLS + rb_col);
+                    for (int q = 0; q < TM * 4; ++q, off += (int64_t)RPI * ldc)
+                        if (r.access("gemm chain C", off, 8, c_elems, T, wave, lane, q) && !stored.empty())
+                            for (int c = 0; c < 8; ++c) ++stored[(size_t)(off + c)];
+                }
+            }
+        }
+    for (int T = 0; T < total && !r.bad; ++T)
+        if (seen[(size_t)T] != 1) r.fail("gemm chain: tile %d is computed %d times", T, (int)seen[(size_t)T]);
+    if (!stored.empty() && !r.bad) {
+        for (int64_t b = 0; b < batch && !r.bad; ++b)
+            for (int64_t mm = 0; mm < M && !r.bad; ++mm)
+                for (int64_t n = 0; n < N; ++n)
+                    if (stored[(size_t)(b * bsc + mm * ldc + n)] != 1) {
+                        r.fail("gemm chain: C[%lld][%lld][%lld] stored %d times", (long long)b, (long long)mm, (long long)n, (int)stored[(size_t)(b * bsc + mm * ldc + n)]);
+                        break;
+                    }
+    }
+    *n_checked = r.checked;
+    return r.bad;
+}
+
 // Workgroup -> (GEMM, tile) map of a several-GEMM launch (gemm.hip: gemm_i8_multi_kernel, launch_multi):
 // tiles[i] = workgroups of GEMM i.  Every workgroup of the grid must land in a GEMM i < count with
 // a tile index in [0, tiles[i]), and every (GEMM, tile) must be taken exactly once.

@@ -41,6 +41,7 @@ def walker(tmp_path_factory):
     lib.walk_quant_row.argtypes = [i64] * 4 + [ci] + [i64] * 3 + [p64, cp, ci]
     lib.walk_quant_block.argtypes = [i64, i64, ci, i64, i64, ci, i64, i64, i64, i64, i64, i64, i64, i64, ci, i64, i64, i64, i64, p64, cp, ci]
     lib.walk_gemm.argtypes = [i64] * 6 + [ctypes.POINTER(ScaleArg)] * 2 + [i64] * 4 + [ci] * 5 + [i64] * 3 + [ctypes.POINTER(ci), p64, cp, ci]
+    lib.walk_gemm_chain.argtypes = [i64] * 6 + [ctypes.POINTER(ScaleArg)] * 2 + [i64] * 4 + [ci] + [i64] * 3 + [p64, cp, ci]
     lib.walk_gemm_multi_map.argtypes = [ctypes.POINTER(ci), ci, p64, cp, ci]
     return lib
 
@@ -110,6 +111,12 @@ def walk(lib, allocs, name, a):
             sb = ScaleArg(mB, sb_bs, sb_rs, sb_ks, allocs.room(sB, 4))
             rc = lib.walk_gemm(bsa, lda, bsb, ldb, bsc, ldc, ctypes.byref(sa), ctypes.byref(sb), batch, M, N, K, acc, flags & 1, (flags >> 3) & 1, 0,
                                NUM_CU, allocs.room(A, 1), allocs.room(B, 1), allocs.room(C, 2), picked, ctypes.byref(n), msg, 512)
+            if rc == 0 and picked[2] == 5 and 2 <= K // 128 <= 64:   # the chained promotion runs on persistent workgroups
+                first = n.value
+                tiles = -(-M // 256) * -(-N // 256) * batch
+                rc = lib.walk_gemm_chain(bsa, lda, bsb, ldb, bsc, ldc, ctypes.byref(sa), ctypes.byref(sb), batch, M, N, K, min(tiles, NUM_CU),
+                                         allocs.room(A, 1), allocs.room(B, 1), allocs.room(C, 2), ctypes.byref(n), msg, 512)
+                n.value += first
         else:
             A, bsa, lda, B, bsb, ldb, C, bsc, ldc, batch, M, N, K = a[:13]
             rc = lib.walk_gemm(bsa, lda, bsb, ldb, bsc, ldc, None, None, batch, M, N, K, 0, 0, 0, 1,
@@ -129,6 +136,11 @@ def walk(lib, allocs, name, a):
             assert rc == 0, f"{name}, GEMM {i}: {msg.value.decode()}"
             total += n.value
             tiles[i] = -(-p.M // picked[0]) * -(-p.N // picked[1])
+            if picked[2] == 5 and 2 <= p.K // 128 <= 64:   # persistent workgroups: each GEMM's tiles as one workgroup list walks them
+                rc = lib.walk_gemm_chain(p.bsa, p.lda, p.bsb, p.ldb, p.bsc, p.ldc, ctypes.byref(sa), ctypes.byref(sb), 1, p.M, p.N, p.K,
+                                         min(tiles[i], NUM_CU), allocs.room(p.A, 1), allocs.room(p.B, 1), allocs.room(p.C, 2), ctypes.byref(n), msg, 512)
+                assert rc == 0, f"{name}, GEMM {i} (persistent): {msg.value.decode()}"
+                total += n.value
         rc = lib.walk_gemm_multi_map(tiles, count, ctypes.byref(n), msg, 512)
         n.value += total
     else:
@@ -246,3 +258,24 @@ def test_multi_launch_map(walker, tiles):
     arr = (ctypes.c_int * len(tiles))(*tiles)
     assert walker.walk_gemm_multi_map(arr, len(tiles), ctypes.byref(n), msg, 512) == 0, msg.value.decode()
     assert n.value == sum(tiles)
+
+
+@pytest.mark.parametrize("M,N,K,batch,mA,mB,grid", [(8192, 4096, 4096, 1, 1, 0, 256), (4096, 4096, 8192, 1, 1, 1, 256), (4224, 4480, 256, 1, 1, 0, 256),
+                                                    (2048, 2304, 1024, 3, 0, 1, 256), (1152, 1408, 512, 2, 3, 0, 7), (8192, 8192, 512, 1, 0, 0, 256)])
+def test_persistent_chain_kernel_geometries(walker, M, N, K, batch, mA, mB, grid):
+    """gemm_i8_chain_kernel: tile lists of persistent workgroups, tiles that hang over M or N, batches, every scale layout."""
+    def desc(mode, rows):
+        if mode == 0:
+            return ScaleArg(0, rows, 1, 0, batch * rows)
+        g = (rows // 128, K // 128 // (2 if mode == 3 else 1))
+        return ScaleArg(mode, g[0] * g[1], g[1], 1, batch * g[0] * g[1])
+    sa, sb = desc(mA, M), desc(mB, N)
+    msg, n = ctypes.create_string_buffer(512), ctypes.c_int64(0)
+    rc = walker.walk_gemm_chain(M * K, K, N * K, K, M * N, N, ctypes.byref(sa), ctypes.byref(sb), batch, M, N, K, grid,
+                                batch * M * K, batch * N * K, batch * M * N, ctypes.byref(n), msg, 512)
+    assert rc == 0, msg.value.decode()
+    assert n.value > 0
+    # one row less of A than the kernel assumes must be noticed
+    rc = walker.walk_gemm_chain(M * K, K, N * K, K, M * N, N, ctypes.byref(sa), ctypes.byref(sb), batch, M, N, K, grid,
+                                batch * M * K - K, batch * N * K, batch * M * N, ctypes.byref(n), msg, 512)
+    assert rc != 0 and b"gemm chain A" in msg.value

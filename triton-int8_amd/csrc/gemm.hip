@@ -15,6 +15,7 @@
 // operand and the 16 bytes k = 16*(l / 32) .. +15 of the 32-deep slice (the same map
 // for both operands, which is all an NT dot product needs); result register r of lane
 // l is C[8*(r/4) + 4*(l/32) + r%4][l % 32] with rows from A and columns from B.
+#include <cstdlib>
 #include <type_traits>
 #include "gemm_args.h"
 
@@ -545,13 +546,6 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_kernel(const GemmArgs g)
 // GEMM i whose range holds w.  The three GEMMs of a training step (Y, dX, dW) run this way when all
 // their operands are at hand: no kernel boundary between them, and the last tiles of one GEMM run
 // beside the first tiles of the next instead of beside idle CUs.
-constexpr int GEMM_MULTI_MAX = 3;
-struct GemmMulti {
-    GemmArgs g[GEMM_MULTI_MAX];
-    int first[GEMM_MULTI_MAX + 1];
-    int count;
-};
-
 template <int BM, int BN, int WM, int WN, int EPI>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_multi_kernel(const GemmMulti m) {
     static_assert(GEMM_MULTI_MAX == 3, "gemm_multi_pick knows three ranges");
@@ -659,6 +653,9 @@ static int prepare_gemm(const char* fn, const ti8_gemm_problem& p, int gemm_flag
     return TI8_OK;
 }
 
+// the chained promotion runs on persistent workgroups (gemm_chain.hip) unless TI8_ONE_TILE_CHAIN is set in the environment
+static const bool PERSISTENT_CHAIN = getenv("TI8_ONE_TILE_CHAIN") == nullptr;
+
 static int device_cu_count() {
     static int num_cu = 0;
     if (num_cu == 0) {
@@ -670,8 +667,31 @@ static int device_cu_count() {
     return num_cu;
 }
 
+// The chained promotion on persistent workgroups where its limits allow (gemm_chain.hip); CHAIN_UNAVAILABLE otherwise
+static int try_chain_persistent(GemmMulti& m, const int64_t* batch, hipStream_t st) {
+    if (!chain_persistent_supported(m)) return CHAIN_UNAVAILABLE;
+    int64_t total = 0;
+    for (int i = 0; i < m.count; ++i) {
+        m.g[i].tiles_m = (m.g[i].M + 255) / 256;
+        m.g[i].tiles_n = (m.g[i].N + 255) / 256;
+        m.first[i] = (int)total;
+        total += (int64_t)m.g[i].tiles_m * m.g[i].tiles_n * batch[i];
+    }
+    if (total > 0x3fffffff) return CHAIN_UNAVAILABLE;
+    for (int i = m.count; i <= GEMM_MULTI_MAX; ++i) m.first[i] = (int)total;
+    for (int i = m.count; i < GEMM_MULTI_MAX; ++i) m.g[i] = m.g[0];
+    return launch_chain_persistent(m, (int)total, device_cu_count(), st);
+}
+
 // One GEMM on the LDS-tiled kernel that `c` names
 static int launch_tiled(const char* fn, const GemmArgs& a, int64_t batch, const idx::GemmConfig& c, hipStream_t st) {
+    if (c.epi == EPI_PROMOTE_CHAIN && PERSISTENT_CHAIN) {
+        GemmMulti m;
+        m.count = 1;
+        m.g[0] = a;
+        const int rc = try_chain_persistent(m, &batch, st);
+        if (rc != CHAIN_UNAVAILABLE) return rc;
+    }
 #define TI8_GEMM_CASE(BM, BN, WM, WN, EPI) \
     if (c.bm == BM && c.bn == BN && c.epi == EPI) return launch<BM, BN, WM, WN, EPI>(a, batch, st)
     TI8_GEMM_CASE(128, 128, 2, 2, EPI_ROWS);
@@ -731,6 +751,11 @@ extern "C" int ti8_gemm_i8_nt_multi(const ti8_gemm_problem* problems, int count,
     }
     one_launch = one_launch && c[0].epi != EPI_STRICT && c[0].epi != EPI_PROMOTE_LANE;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (one_launch && c[0].epi == EPI_PROMOTE_CHAIN && PERSISTENT_CHAIN) {
+        const int64_t ones[GEMM_MULTI_MAX] = {1, 1, 1};
+        const int rc = try_chain_persistent(m, ones, st);
+        if (rc != CHAIN_UNAVAILABLE) return rc;
+    }
     if (one_launch) {
 #define TI8_GEMM_CASE(BM, BN, WM, WN, EPI) \
         if (c[0].bm == BM && c[0].bn == BN && c[0].epi == EPI) return launch_multi<BM, BN, WM, WN, EPI>(m, st)

@@ -55,6 +55,23 @@ __device__ __forceinline__ void issue_tile_loads(const int8_t* base, int64_t str
 #endif
 }
 
+// Several GEMMs in one launch: GEMM i owns the workgroups (one-tile kernels) or the tile numbers (persistent
+// kernel) [first[i], first[i + 1]), first[0] = 0.
+constexpr int GEMM_MULTI_MAX = 3;
+struct GemmMulti {
+    GemmArgs g[GEMM_MULTI_MAX];
+    int first[GEMM_MULTI_MAX + 1];
+    int count;
+};
+
+// Persistent-workgroup kernel for the chained block-channel promotion on 256 x 256 tiles (gemm_chain.hip).
+// `m.g[i].tiles_m / tiles_n` and `m.first` must be filled for 256 x 256 tiles, batches included
+// (first[i + 1] - first[i] = tiles_m * tiles_n * batch of GEMM i).  launch returns TI8_OK, an error, or
+// CHAIN_UNAVAILABLE when the device refuses the 160 KiB of LDS (the caller then takes the one-tile kernel).
+constexpr int CHAIN_UNAVAILABLE = -1;
+bool chain_persistent_supported(const GemmMulti& m);
+int launch_chain_persistent(const GemmMulti& m, int total_tiles, int num_cu, hipStream_t st);
+
 // Kernel for few rows (gemm_skinny.hip): M a multiple of 128, operand A without per-(row, K tile)
 // scales.  i32_full: int32 accumulation over the whole K with per-row scales (bit-exact path).
 bool skinny_supported(const GemmArgs& a);

@@ -1,0 +1,430 @@
+// Block-channel promotion GEMM (EPI_PROMOTE_CHAIN arithmetic of gemm.hip) with PERSISTENT workgroups:
+// one workgroup per CU walks its output tiles (256 x 256, 8 waves of 128 x 64) one after the other,
+// and the K loop never stops at a tile boundary:
+//   * the loads that the one-tile kernel spends on re-reading the last K tile (it fetches one to two K
+//     tiles ahead without a branch) fetch the NEXT output tile's K tiles 0 and 1 instead, and the last
+//     iteration reads that tile's first fragments as it would read the next K tile's: a tile starts with
+//     its operands in LDS and in registers, no prologue;
+//   * the epilogue goes through an LDS slab of its own (32 KiB beyond the operand buffers, 16 tile rows
+//     at a time), so that it does not wait for, or disturb, the operand loads in flight;
+//   * its global stores drain while the next tile's first K tile is multiplied.
+// Per tile this leaves the epilogue's own instructions; measured against one workgroup per tile: the
+// prologue, the workgroup turn-over and most of the store drain.
+// Arithmetic, operand layout in LDS, fragment reads and accumulator layout are those of the chained loop
+// in gemm.hip; results are bit-identical.  Limits: 2 <= K / 128 <= 64 for every GEMM of the launch (one
+// register holds a tile's per-K-tile factors; the launcher sends other shapes to the one-tile kernel).
+#include <type_traits>
+#include "gemm_args.h"
+
+namespace ti8 {
+
+namespace {
+
+constexpr int BM = 256, BN = 256, WM = 2, WN = 4, NW = WM * WN, TM = 4, TN = 2;
+constexpr int A_INSTR = BM / 8 / NW, B_INSTR = BN / 8 / NW;
+constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128;
+constexpr int WCOLS = TN * 32;
+constexpr int SLAB_ROWS = 16;                                   // tile rows per pass through the slab
+constexpr int SLAB_BYTES = NW * SLAB_ROWS * WCOLS * 4;          // 32 KiB
+constexpr int LDS_BYTES = 2 * (A_BYTES + B_BYTES) + SLAB_BYTES; // 160 KiB
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+// What a wave needs to know about one output tile; every member is wave-uniform.
+struct Tile {
+    int gi;                  // GEMM of the launch
+    int batch;
+    int m0, n0;              // first row / column of the tile
+    int nk;                  // K tiles
+    const int8_t* baseA;     // first row of this wave's share of the tile's A (B) rows, K offset 0
+    const int8_t* baseB;
+    int64_t strideA8, strideB8;
+    int lda, ldb;
+    // scale values that a wave fetches with one register of per-lane offset each (32-bit: checked on the host)
+    const float* fa_p;       // A's scale grid at this wave tile's row block, K block 0
+    const float* fb_p;       // B's, at its column block
+    uint32_t fa_ks, fb_ks;   // stride between K blocks (0 for an operand whose factor is not applied inside the loop)
+    int fa_sh, fb_sh;        // 1 for 256-wide scale groups
+    const float* col_p;      // B's per-row scales at the wave tile's first column (the operand's own first row when it has none)
+    uint32_t col_s;          // their stride (0 when B has none)
+};
+
+}  // namespace
+
+__global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti m, const int total_tiles) {
+    extern __shared__ __attribute__((aligned(1024))) int8_t smem[];
+    // layout: [A buf0][A buf1][B buf0][B buf1][epilogue slab]
+    int8_t* const ldsA = smem;
+    int8_t* const ldsB = smem + 2 * A_BYTES;
+    uint32_t* const slab = reinterpret_cast<uint32_t*>(smem + 2 * (A_BYTES + B_BYTES)) +
+                           __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) * (SLAB_ROWS * WCOLS);
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+    const int tA0 = wave * A_INSTR, tB0 = wave * B_INSTR;
+    int8_t* const wA = ldsA + wave * A_INSTR * 1024;  // this wave's share of an A buffer
+    int8_t* const wB = ldsB + wave * B_INSTR * 1024;
+
+    // LDS -> register mapping (as in gemm.hip)
+    const int fr_row = lane & 31;
+    const int fr_half = lane >> 5;
+    const int sw = (lane & 7) ^ ((lane >> 3) & 1);
+    const int a_row_off = (wm * TM * 32 + fr_row) * 128;
+    const int b_row_off = (wn * TN * 32 + fr_row) * 128;
+    int choff[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) choff[ks] = ((ks * 2 + fr_half) ^ sw) * 16;
+
+    constexpr int GROUP = idx::gemm_group_rows(BM);
+    const int stride_t = gridDim.x;
+
+    // ---- tile T of the launch -> what the loops need --------------------------------------
+    auto locate = [&](int T) {
+        Tile t;
+        t.gi = idx::gemm_multi_pick(T, m.first[1], m.first[2], m.count);
+        const GemmArgs& g = m.g[t.gi];
+        const int local = T - m.first[t.gi];
+        const int per_batch = g.tiles_m * g.tiles_n;
+        // (divisions of uniform values come out of the vector unit: back into scalar registers)
+        t.batch = __builtin_amdgcn_readfirstlane(local / per_batch);
+        const idx::TileCoord tc = idx::gemm_tile_of(local - t.batch * per_batch, g.tiles_m, g.tiles_n, GROUP);
+        t.m0 = __builtin_amdgcn_readfirstlane(tc.tile_m) * BM;
+        t.n0 = __builtin_amdgcn_readfirstlane(tc.tile_n) * BN;
+        t.nk = g.K >> 7;
+        t.lda = (int)g.lda;
+        t.ldb = (int)g.ldb;
+        const int rA0 = idx::gemm_wave_first_row(t.m0, wave, A_INSTR, g.M), rB0 = idx::gemm_wave_first_row(t.n0, wave, B_INSTR, g.N);
+        t.baseA = g.A + (int64_t)t.batch * g.bsa + (int64_t)rA0 * g.lda;   // scalar arithmetic: every term is wave-uniform
+        t.baseB = g.B + (int64_t)t.batch * g.bsb + (int64_t)rB0 * g.ldb;
+        t.strideA8 = 8 * g.lda;
+        t.strideB8 = 8 * g.ldb;
+        const bool a_in = g.sa.mode != TI8_SCALE_ROW, b_in = g.sb.mode != TI8_SCALE_ROW;
+        t.fa_p = g.sa.p + idx::gemm_factor_index(t.batch, g.sa.bs, idx::gemm_factor_block(t.m0 + wm * TM * 32, g.M), g.sa.rs, 0, 0, 0);
+        t.fb_p = g.sb.p + idx::gemm_factor_index(t.batch, g.sb.bs, idx::gemm_factor_block(t.n0 + wn * TN * 32, g.N), g.sb.rs, 0, 0, 0);
+        t.fa_ks = a_in ? (uint32_t)g.sa.ks : 0u;
+        t.fb_ks = b_in ? (uint32_t)g.sb.ks : 0u;
+        t.fa_sh = g.sa.mode == TI8_SCALE_BLOCK_K256 ? 1 : 0;
+        t.fb_sh = g.sb.mode == TI8_SCALE_BLOCK_K256 ? 1 : 0;
+        t.col_s = b_in ? 0u : (uint32_t)g.sb.rs;
+        t.col_p = g.sb.p + idx::epi_col_scale_index(t.batch, g.sb.bs, idx::chain_col_scale_first(t.n0 + wn * WCOLS, g.N), g.N, t.col_s);
+        return t;
+    };
+    // one wave's global -> LDS loads of one K tile of an operand (per-lane offsets rebuilt from the leading
+    // dimension each time: one multiply-add per parity instead of registers held across the loop)
+    auto load_a = [&](const Tile& t, int koff, int8_t* dst) {
+        const uint32_t vo[2] = {idx::gemm_lane_offset_bytes(lane, 0, t.lda), idx::gemm_lane_offset_bytes(lane, 1, t.lda)};
+        issue_tile_loads<A_INSTR>(t.baseA + koff, t.strideA8, vo, tA0, dst);
+    };
+    auto load_b = [&](const Tile& t, int koff, int8_t* dst) {
+        const uint32_t vo[2] = {idx::gemm_lane_offset_bytes(lane, 0, t.ldb), idx::gemm_lane_offset_bytes(lane, 1, t.ldb)};
+        issue_tile_loads<B_INSTR>(t.baseB + koff, t.strideB8, vo, tB0, dst);
+    };
+    // per-K-tile factors of a tile, K tile `lane` in each lane (raw scale values; `finish_factors` combines them).
+    // Unconditional loads: an operand without in-loop factors is read with stride 0 and its value dropped.
+    // (lane-derived values of the once-per-tile code are rebuilt from an opaque copy of the lane number: hoisted out
+    // of the tile loop they would sit in registers that the K loop has no room for)
+    auto opaque_lane = [&]() {
+        int l = lane;
+        asm volatile("" : "+v"(l));
+        return l;
+    };
+    auto load_raw_factors = [&](const Tile& t, float& ra, float& rb) {
+        const uint32_t kt = (uint32_t)idx::gemm_factor_kt(0, opaque_lane(), t.nk);
+        ra = t.fa_p[(kt >> t.fa_sh) * t.fa_ks];
+        rb = t.fb_p[(kt >> t.fb_sh) * t.fb_ks];
+    };
+    auto finish_factors = [&](const Tile& t, float ra, float rb) {
+        const GemmArgs& g = m.g[t.gi];
+        float f = g.sa.mode != TI8_SCALE_ROW ? ra : 1.0f;
+        if (g.sb.mode != TI8_SCALE_ROW) f = f * rb;
+        if (g.combine == TI8_COMBINE_DIV_PROD) f = 1.0f / f;
+        return f;
+    };
+    // the 4 column scales this lane fetches for the epilogue (16 lanes cover the wave tile's 64 columns)
+    auto load_col_scales = [&](const Tile& t, float (&cn)[4]) {
+        const uint32_t c0 = (uint32_t)idx::epi_scale_col_of_lane(opaque_lane());
+#pragma unroll
+        for (int c = 0; c < 4; ++c) cn[c] = t.col_p[(c0 + c) * t.col_s];
+    };
+
+    float accf[TM][TN][16];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) accf[i][j][r] = 0.0f;
+    const v16i vzero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+
+    v4i fa[2][4], fbv[TN][4];
+    auto read_a = [&](int buf, const int8_t* stage_a, int i) {
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) fa[buf][ks] = *reinterpret_cast<const v4i*>(stage_a + a_row_off + i * 4096 + choff[ks]);
+    };
+    auto read_b = [&](const int8_t* stage_b, int ks) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fbv[j][ks] = *reinterpret_cast<const v4i*>(stage_b + b_row_off + j * 4096 + choff[ks]);
+    };
+    float f_cur = 1.0f;
+    auto fold = [&](int i, const v16i& d0, const v16i& d1) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) accf[i][0][r] = __builtin_fmaf(static_cast<float>(d0[r]), f_cur, accf[i][0][r]);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) accf[i][1][r] = __builtin_fmaf(static_cast<float>(d1[r]), f_cur, accf[i][1][r]);
+    };
+
+    // One K tile.  `step` counts K tiles since the kernel started (LDS buffer = step & 1); the B half of the K tile
+    // after this one is issued at the top, the A half of the one after that behind the barrier: `nb` / `na` say where
+    // those come from (this tile or the next output tile).
+    // `read_next`: whether the last block row also reads the next K tile's first fragments (not across a tile
+    // boundary: the epilogue needs the registers, and reads them afterwards)
+    auto ktile = [&](auto read_next_tag, int step, float fvec, int kt, const Tile& nb, int koff_b, const Tile& na, int koff_a) {
+        constexpr bool READ_NEXT = decltype(read_next_tag)::value;
+        const int cur = step & 1;
+        const int8_t* stA = ldsA + cur * A_BYTES;
+        const int8_t* stAn = ldsA + (cur ^ 1) * A_BYTES;
+        const int8_t* stBn = ldsB + (cur ^ 1) * B_BYTES;
+        f_cur = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fvec), kt));
+        load_b(nb, koff_b, wB + (cur ^ 1) * B_BYTES);
+#pragma unroll
+        for (int i = 0; i < TM - 1; ++i) {
+            read_a((i + 1) & 1, stA, i + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            v16i d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i & 1][0], fbv[0][0], vzero, 0, 0, 0);
+            v16i d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i & 1][0], fbv[1][0], vzero, 0, 0, 0);
+#pragma unroll
+            for (int ks = 1; ks < 4; ++ks) {
+                d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i & 1][ks], fbv[0][ks], d0, 0, 0, 0);
+                d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i & 1][ks], fbv[1][ks], d1, 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            fold(i, d0, d1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // last block row: the next K tile has landed, its fragments replace this one's as they retire
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        load_a(na, koff_a, wA + cur * A_BYTES);
+        constexpr int LB = (TM - 1) & 1;   // buffer that holds the last block row
+        static_assert(LB == 1, "an even number of block rows keeps the A fragment buffers in phase");
+        if (READ_NEXT) read_a(LB ^ 1, stAn, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        v16i d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[LB][0], fbv[0][0], vzero, 0, 0, 0);
+        v16i d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[LB][0], fbv[1][0], vzero, 0, 0, 0);
+        d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[LB][1], fbv[0][1], d0, 0, 0, 0);
+        d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[LB][1], fbv[1][1], d1, 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (READ_NEXT) {
+            read_b(stBn, 0);
+            read_b(stBn, 1);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[LB][2], fbv[0][2], d0, 0, 0, 0);
+        d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[LB][2], fbv[1][2], d1, 0, 0, 0);
+        d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[LB][3], fbv[0][3], d0, 0, 0, 0);
+        d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[LB][3], fbv[1][3], d1, 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (READ_NEXT) {
+            read_b(stBn, 2);
+            read_b(stBn, 3);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        fold(TM - 1, d0, d1);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    // ---- epilogue of one tile: accumulators -> slab (16 rows at a time) -> bf16 rows in C -----------------
+    // Slab word (row, col) of a wave sits at row * 64 + (col ^ 4 (row & 1)): the two rows that 16 lanes read
+    // together then fall in different banks.  A wave's tile lies inside one 128-row and one 128-column block and
+    // M, N are multiples of 128, so a wave either stores its whole tile or nothing.
+    constexpr int RPI = 64 / (WCOLS / 8);   // rows per store instruction
+    auto epilogue = [&](const Tile& t, const float (&coln)[4]) {
+        const GemmArgs& g = m.g[t.gi];
+        if (t.m0 + wm * TM * 32 >= g.M || t.n0 + wn * WCOLS >= g.N) return;
+        const int el = opaque_lane();
+        const int rb_col = idx::epi_col_of_lane(el, WCOLS), rb_row = idx::epi_row_of_lane(el, WCOLS);
+        const int e_row = el & 31, e_half = el >> 5;
+        const bool divide = g.combine == TI8_COMBINE_DIV_PROD;
+        const bool row_part = g.sa.mode == TI8_SCALE_ROW, col_part = g.sb.mode == TI8_SCALE_ROW;
+        float cm[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const float v = __int_as_float(__builtin_amdgcn_ds_bpermute(idx::epi_scale_lane(el, c) * 4, __float_as_int(coln[c & 3])));
+            cm[c] = divide ? 1.0f / v : v;
+        }
+        const int row0 = t.m0 + wm * TM * 32 + rb_row;
+        const int64_t c_off = idx::epi_out_offset(t.batch, g.bsc, row0, g.ldc, t.n0 + wn * WCOLS + rb_col);
+        const int64_t c_step = (int64_t)RPI * g.ldc;
+        const float* prow0 = g.sa.p + idx::epi_row_scale_base(t.batch, g.sa.bs, row0, g.sa.rs);
+        auto store_tile = [&](auto extra_tag, auto mrow_tag, auto mcol_tag) {
+            constexpr bool EXTRA = decltype(extra_tag)::value;
+            constexpr bool MROW = decltype(mrow_tag)::value;
+            constexpr bool MCOL = decltype(mcol_tag)::value;
+            int64_t off = c_off;
+            float rm_all[MROW ? TM * 4 : 1];
+            if (MROW) {   // every row scale of the tile before the first store (loads and stores share one in-order counter)
+#pragma unroll
+                for (int q = 0; q < TM * 4; ++q) rm_all[q] = prow0[(int64_t)(q * RPI) * g.sa.rs];
+                if (divide) {
+#pragma unroll
+                    for (int q = 0; q < TM * 4; ++q) rm_all[q] = 1.0f / rm_all[q];
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {   // rows 16 h .. 16 h + 15 of block row i: accumulator registers 8 h .. 8 h + 7
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            const int rr = idx::epi_chain_slab_row(e, e_half);
+                            slab[idx::epi_chain_slab_word(rr, j * 32 + e_row)] = __float_as_uint(accf[i][j][8 * h + e]);
+                        }
+                    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): same wave reads what it wrote, no barrier
+                    __builtin_amdgcn_wave_barrier();
+                    uint4 w[2][2];
+#pragma unroll
+                    for (int k = 0; k < 2; ++k) {
+                        const int rr = rb_row + k * RPI;
+                        w[k][0] = *reinterpret_cast<const uint4*>(slab + idx::epi_chain_slab_word(rr, rb_col));
+                        w[k][1] = *reinterpret_cast<const uint4*>(slab + idx::epi_chain_slab_word(rr, rb_col + 4));
+                    }
+#pragma unroll
+                    for (int k = 0; k < 2; ++k, off += c_step) {
+                        const uint32_t wb[8] = {w[k][0].x, w[k][0].y, w[k][0].z, w[k][0].w, w[k][1].x, w[k][1].y, w[k][1].z, w[k][1].w};
+                        float v[8];
+#pragma unroll
+                        for (int c = 0; c < 8; ++c) {
+                            v[c] = __uint_as_float(wb[c]);
+                            if (MROW) v[c] = v[c] * rm_all[MROW ? (i * 2 + h) * 2 + k : 0];
+                            if (MCOL) v[c] = v[c] * cm[c];
+                            if (EXTRA) v[c] = v[c] * g.out_scale;
+                        }
+                        uint16_t* dst = reinterpret_cast<uint16_t*>(g.C) + off;
+                        *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+                        *reinterpret_cast<uint2*>(dst + 4) = make_uint2(pack_bf16x2(v[4], v[5]), pack_bf16x2(v[6], v[7]));
+                    }
+                    __builtin_amdgcn_s_waitcnt(0xc07f);
+                    __builtin_amdgcn_wave_barrier();
+                }
+        };
+        using T_ = std::true_type;
+        using F_ = std::false_type;
+        if (g.out_scale != 1.0f) {
+            if (row_part && col_part) store_tile(T_{}, T_{}, T_{});
+            else if (row_part) store_tile(T_{}, T_{}, F_{});
+            else if (col_part) store_tile(T_{}, F_{}, T_{});
+            else store_tile(T_{}, F_{}, F_{});
+        } else {
+            if (row_part && col_part) store_tile(F_{}, T_{}, T_{});
+            else if (row_part) store_tile(F_{}, T_{}, F_{});
+            else if (col_part) store_tile(F_{}, F_{}, T_{});
+            else store_tile(F_{}, F_{}, F_{});
+        }
+    };
+
+    // ---- first tile: operands of K tile 0 into LDS and registers, K tile 1's A half in flight ------------
+    int T = blockIdx.x;
+    Tile cur = locate(T);
+    // without a next tile the loads that run ahead fetch this tile's K tiles 0 and 1 again (nobody reads them)
+    bool more = T + stride_t < total_tiles;
+    Tile nxt = more ? locate(T + stride_t) : cur;
+    float fvec;
+    {
+        load_a(cur, 0, wA);
+        load_b(cur, 0, wB);
+        float ra, rb;
+        load_raw_factors(cur, ra, rb);
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        fvec = finish_factors(cur, ra, rb);
+        load_a(cur, 128, wA + A_BYTES);
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) read_b(ldsB, ks);
+        read_a(0, ldsA, 0);
+    }
+    int step = 0;
+    while (true) {
+        const int nk = cur.nk;
+        // all but the last K tile: B of kt + 1 from this tile; A of kt + 2 from this tile, in the last of them K tile 0 of the next
+        for (int kt = 0; kt < nk - 1; ++kt, ++step) {
+            const bool a_next = kt + 2 >= nk;
+            ktile(std::true_type{}, step, fvec, kt, cur, (kt + 1) * 128, a_next ? nxt : cur, a_next ? 0 : (kt + 2) * 128);
+        }
+        // last K tile: the column scales of this tile's epilogue and the next tile's factors travel beside it
+        float coln[4], ra, rb;
+        load_col_scales(cur, coln);
+        load_raw_factors(nxt, ra, rb);
+        __builtin_amdgcn_sched_barrier(0);
+        ktile(std::false_type{}, step, fvec, nk - 1, nxt, 0, nxt, 128);
+        ++step;
+        // the accumulators are complete HERE: without this the optimiser moves the last K tile's convert + fma behind
+        // the epilogue's branches and keeps that tile's 128 int32 results alive until then
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                float* a = accf[i][j];
+                asm volatile("" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7]),
+                                  "+v"(a[8]), "+v"(a[9]), "+v"(a[10]), "+v"(a[11]), "+v"(a[12]), "+v"(a[13]), "+v"(a[14]), "+v"(a[15]));
+            }
+        fvec = finish_factors(nxt, ra, rb);
+        epilogue(cur, coln);
+        if (!more) break;
+        // the next tile's K tile 0 has been in LDS since the barrier of the last K tile: its first fragments
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) read_b(ldsB + (step & 1) * B_BYTES, ks);
+        read_a(0, ldsA + (step & 1) * A_BYTES, 0);
+        // the accumulators are free: the place for the integer divisions that find the tile after the next
+        T += stride_t;
+        cur = nxt;
+        more = T + stride_t < total_tiles;
+        if (more) nxt = locate(T + stride_t);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) accf[i][j][r] = 0.0f;
+    }
+    // loads that ran ahead of the last tile are still landing in this workgroup's LDS
+    __builtin_amdgcn_s_waitcnt(0);
+}
+
+bool chain_persistent_supported(const GemmMulti& m) {
+    for (int i = 0; i < m.count; ++i) {
+        const int nk = m.g[i].K >> 7;
+        if (nk < 2 || nk > 64 || m.g[i].strict) return false;
+        if (m.g[i].sa.mode == TI8_SCALE_ROW_K128 || m.g[i].sb.mode == TI8_SCALE_ROW_K128) return false;
+        // per-lane offsets into the scale arrays are kept in 32 bits: 64 K blocks x stride, 64 columns x stride
+        const int64_t lim = (int64_t)1 << 24;
+        if (m.g[i].sa.ks < 0 || m.g[i].sa.ks >= lim || m.g[i].sb.ks < 0 || m.g[i].sb.ks >= lim || m.g[i].sb.rs < 0 || m.g[i].sb.rs >= lim) return false;
+    }
+    return true;
+}
+
+// `m` with tiles_m / tiles_n / first[] filled for 256 x 256 tiles and first[i + 1] - first[i] = tiles of GEMM i times
+// its batch count; one workgroup per CU (fewer when there are fewer tiles)
+int launch_chain_persistent(const GemmMulti& m, int total_tiles, int num_cu, hipStream_t st) {
+    static thread_local int attr_dev = -1;
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    static thread_local int refused_dev = -1;
+    if (refused_dev == dev) return CHAIN_UNAVAILABLE;
+    if (attr_dev != dev) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_i8_chain_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess) {
+            (void)hipGetLastError();
+            refused_dev = dev;
+            return CHAIN_UNAVAILABLE;
+        }
+        attr_dev = dev;
+    }
+    const int grid = total_tiles < num_cu ? total_tiles : num_cu;
+    hipLaunchKernelGGL(gemm_i8_chain_kernel, dim3((unsigned)grid), dim3(64 * NW), LDS_BYTES, st, m, total_tiles);
+    return check_launch("ti8_gemm_i8_nt");
+}
+
+}  // namespace ti8

@@ -113,6 +113,14 @@ TI8_HD int epi_row_of_lane(int lane, int wcols) { return lane / (wcols / 8); }
 // takes scale c of them from lane 2 q + c / 4 (register c % 4 there)
 TI8_HD int epi_scale_col_of_lane(int lane) { return (lane % 16) * 4; }
 TI8_HD int epi_scale_lane(int lane, int c) { return 2 * (lane % 8) + (c >> 2); }
+// persistent chained kernel (gemm_chain.hip): its slab holds 16 tile rows of 64 words per wave; accumulator
+// register 8 h + e (e < 8) of a 32 x 32 block is row 16 h + epi_chain_slab_row(e, lane / 32) of the block, and
+// word (row, col) sits at row * 64 + (col ^ 4 (row & 1))
+// first column whose per-row scale of B a wave of the persistent kernel fetches: its tile's first column, or, for a
+// tile outside the operand (N is a multiple of 128, the wave tile has 64 columns), the operand's last 64 columns
+TI8_HD int chain_col_scale_first(int first_col_of_wave_tile, int ncols) { return imin(first_col_of_wave_tile, ncols - 64); }
+TI8_HD int epi_chain_slab_row(int e, int fr_half) { return 8 * (e >> 2) + 4 * fr_half + (e & 3); }
+TI8_HD int epi_chain_slab_word(int row, int col) { return row * 64 + (col ^ (4 * (row & 1))); }
 // index of the column scale of column `col` (clamped to the last column; stride 0 when absent)
 TI8_HD int64_t epi_col_scale_index(int64_t batch, int64_t bs, int col, int ncols, int64_t cs) {
     return batch * bs + (int64_t)imin(col, ncols - 1) * cs;
