@@ -27,6 +27,12 @@ constexpr int WCOLS = TN * 32;
 constexpr int SLAB_ROWS = 16;                                   // tile rows per pass through the slab
 constexpr int SLAB_BYTES = NW * SLAB_ROWS * WCOLS * 4;          // 32 KiB
 constexpr int LDS_BYTES = 2 * (A_BYTES + B_BYTES) + SLAB_BYTES; // 160 KiB
+// a wave whose tile lies inside the output stores it with 32 instructions (16 x 8 rows, two 8-byte stores each);
+// s_waitcnt vmcnt(32) lgkmcnt(0): vector-memory operations complete in issue order, so everything issued
+// before those stores has completed when at most 32 are outstanding
+constexpr int EPILOGUE_STORES = TM * 2 * 2 * 2;
+constexpr int WAIT_ALL_BUT_STORES = ((EPILOGUE_STORES >> 4) << 14) | (EPILOGUE_STORES & 15) | 0x70;
+static_assert(EPILOGUE_STORES == 32 && WAIT_ALL_BUT_STORES == 0x8070, "s_waitcnt encoding: vmcnt[3:0] | expcnt << 4 | lgkmcnt << 8 | vmcnt[5:4] << 14");
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
@@ -180,14 +186,19 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
     // those come from (this tile or the next output tile).
     // `read_next`: whether the last block row also reads the next K tile's first fragments (not across a tile
     // boundary: the epilogue needs the registers, and reads them afterwards)
-    auto ktile = [&](auto read_next_tag, int step, float fvec, int kt, const Tile& nb, int koff_b, const Tile& na, int koff_a) {
+    // `first`: the first K tile of an output tile.  The B half of its successor is already on its way (issued before the
+    // previous tile's epilogue), and it waits only for the loads issued before that epilogue's stores: the stores
+    // (`stores_pending` of them at most, the youngest operations of this wave) drain while this K tile is multiplied.
+    auto ktile = [&](auto first_tag, auto read_next_tag, bool stores_pending, int step, float fvec, int kt, const Tile& nb, int koff_b,
+                     const Tile& na, int koff_a) {
+        constexpr bool FIRST = decltype(first_tag)::value;
         constexpr bool READ_NEXT = decltype(read_next_tag)::value;
         const int cur = step & 1;
         const int8_t* stA = ldsA + cur * A_BYTES;
         const int8_t* stAn = ldsA + (cur ^ 1) * A_BYTES;
         const int8_t* stBn = ldsB + (cur ^ 1) * B_BYTES;
         f_cur = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fvec), kt));
-        load_b(nb, koff_b, wB + (cur ^ 1) * B_BYTES);
+        if (!FIRST) load_b(nb, koff_b, wB + (cur ^ 1) * B_BYTES);
 #pragma unroll
         for (int i = 0; i < TM - 1; ++i) {
             read_a((i + 1) & 1, stA, i + 1);
@@ -204,8 +215,17 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
             __builtin_amdgcn_sched_barrier(0);
         }
         // last block row: the next K tile has landed, its fragments replace this one's as they retire
-        __builtin_amdgcn_s_waitcnt(0);
-        __syncthreads();
+        if (FIRST) {
+            // what this barrier orders is in LDS: this wave's operand loads have landed and its fragment reads have returned once
+            // the counters below are down.  The barrier instruction is written out because the compiler puts a wait for ALL
+            // vector-memory operations in front of the one it knows, which would wait for the stores after all.
+            if (stores_pending) __builtin_amdgcn_s_waitcnt(WAIT_ALL_BUT_STORES);
+            else __builtin_amdgcn_s_waitcnt(0);
+            asm volatile("s_barrier" ::: "memory");
+        } else {
+            __builtin_amdgcn_s_waitcnt(0);
+            __syncthreads();
+        }
         load_a(na, koff_a, wA + cur * A_BYTES);
         constexpr int LB = (TM - 1) & 1;   // buffer that holds the last block row
         static_assert(LB == 1, "an even number of block rows keeps the A fragment buffers in phase");
@@ -242,7 +262,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
     constexpr int RPI = 64 / (WCOLS / 8);   // rows per store instruction
     auto epilogue = [&](const Tile& t, const float (&coln)[4]) {
         const GemmArgs& g = m.g[t.gi];
-        if (t.m0 + wm * TM * 32 >= g.M || t.n0 + wn * WCOLS >= g.N) return;
+        if (t.m0 + wm * TM * 32 >= g.M || t.n0 + wn * WCOLS >= g.N) return false;
         const int el = opaque_lane();
         const int rb_col = idx::epi_col_of_lane(el, WCOLS), rb_row = idx::epi_row_of_lane(el, WCOLS);
         const int e_row = el & 31, e_half = el >> 5;
@@ -324,6 +344,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
             else if (col_part) store_tile(F_{}, F_{}, T_{});
             else store_tile(F_{}, F_{}, F_{});
         }
+        return true;
     };
 
     // ---- first tile: operands of K tile 0 into LDS and registers, K tile 1's A half in flight ------------
@@ -342,24 +363,34 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
         __syncthreads();
         fvec = finish_factors(cur, ra, rb);
         load_a(cur, 128, wA + A_BYTES);
+        load_b(cur, 128, wB + B_BYTES);
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) read_b(ldsB, ks);
         read_a(0, ldsA, 0);
     }
     int step = 0;
+    bool stored = false;   // whether this wave's previous epilogue left stores behind
     while (true) {
         const int nk = cur.nk;
-        // all but the last K tile: B of kt + 1 from this tile; A of kt + 2 from this tile, in the last of them K tile 0 of the next
-        for (int kt = 0; kt < nk - 1; ++kt, ++step) {
+        // all but the last K tile: B of kt + 1 from this tile (for kt = 0 it is under way already); A of kt + 2 from this tile,
+        // in the last of them K tile 0 of the next
+        using T_ = std::true_type;
+        using F_ = std::false_type;
+        if (nk > 1) {
+            const bool a_next = 2 >= nk;
+            ktile(T_{}, T_{}, stored, step, fvec, 0, cur, 128, a_next ? nxt : cur, a_next ? 0 : 256);
+            ++step;
+        }
+        for (int kt = 1; kt < nk - 1; ++kt, ++step) {
             const bool a_next = kt + 2 >= nk;
-            ktile(std::true_type{}, step, fvec, kt, cur, (kt + 1) * 128, a_next ? nxt : cur, a_next ? 0 : (kt + 2) * 128);
+            ktile(F_{}, T_{}, false, step, fvec, kt, cur, (kt + 1) * 128, a_next ? nxt : cur, a_next ? 0 : (kt + 2) * 128);
         }
         // last K tile: the column scales of this tile's epilogue and the next tile's factors travel beside it
         float coln[4], ra, rb;
         load_col_scales(cur, coln);
         load_raw_factors(nxt, ra, rb);
         __builtin_amdgcn_sched_barrier(0);
-        ktile(std::false_type{}, step, fvec, nk - 1, nxt, 0, nxt, 128);
+        ktile(F_{}, F_{}, false, step, fvec, nk - 1, nxt, 0, nxt, 128);
         ++step;
         // the accumulators are complete HERE: without this the optimiser moves the last K tile's convert + fma behind
         // the epilogue's branches and keeps that tile's 128 int32 results alive until then
@@ -372,7 +403,10 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
                                   "+v"(a[8]), "+v"(a[9]), "+v"(a[10]), "+v"(a[11]), "+v"(a[12]), "+v"(a[13]), "+v"(a[14]), "+v"(a[15]));
             }
         fvec = finish_factors(nxt, ra, rb);
-        epilogue(cur, coln);
+        // the B half of the next tile's K tile 1, into the buffer the last K tile's B has left: issued before the epilogue's
+        // stores, so that the next tile's first K tile need not wait for them
+        load_b(nxt, 128, wB + ((step - 1) & 1) * B_BYTES);
+        stored = epilogue(cur, coln);
         if (!more) break;
         // the next tile's K tile 0 has been in LDS since the barrier of the last K tile: its first fragments
 #pragma unroll
