@@ -11,8 +11,10 @@
 // Per tile this leaves the epilogue's own instructions; measured against one workgroup per tile: the
 // prologue, the workgroup turn-over and most of the store drain.
 // Arithmetic, operand layout in LDS, fragment reads and accumulator layout are those of the chained loop
-// in gemm.hip; results are bit-identical.  Limits: 2 <= K / 128 <= 64 for every GEMM of the launch (one
-// register holds a tile's per-K-tile factors; the launcher sends other shapes to the one-tile kernel).
+// in gemm.hip; results are bit-identical.  Limits: K / 128 even and in [2, 64] for every GEMM of the launch (one
+// register holds a tile's per-K-tile factors, and a tile's K tiles alternate between the two LDS buffers from a
+// fixed start, which makes every LDS address a register plus an immediate; the launcher sends other shapes to
+// the one-tile kernel).
 #include <type_traits>
 #include "gemm_args.h"
 
@@ -32,10 +34,15 @@ constexpr int LDS_BYTES = 2 * (A_BYTES + B_BYTES) + SLAB_BYTES; // 160 KiB
 // before those stores has completed when at most 32 are outstanding
 constexpr int EPILOGUE_STORES = TM * 2 * 2 * 2;
 constexpr int WAIT_ALL_BUT_STORES = ((EPILOGUE_STORES >> 4) << 14) | (EPILOGUE_STORES & 15) | 0x70;
+// vmcnt(B_INSTR) / vmcnt(B_INSTR + 32) with the other counters left alone
+constexpr int WAIT_FACTORS = B_INSTR | 0x70 | 0xF00;
+constexpr int WAIT_FACTORS_BEHIND_STORES = (((B_INSTR + EPILOGUE_STORES) >> 4) << 14) | ((B_INSTR + EPILOGUE_STORES) & 15) | 0x70 | 0xF00;
+static_assert(B_INSTR == 4 && WAIT_FACTORS == 0xF74 && WAIT_FACTORS_BEHIND_STORES == 0x8F74, "s_waitcnt encoding");
 static_assert(EPILOGUE_STORES == 32 && WAIT_ALL_BUT_STORES == 0x8070, "s_waitcnt encoding: vmcnt[3:0] | expcnt << 4 | lgkmcnt << 8 | vmcnt[5:4] << 14");
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 // What a wave needs to know about one output tile; every member is wave-uniform.
 struct Tile {
@@ -45,13 +52,12 @@ struct Tile {
     int nk;                  // K tiles
     const int8_t* baseA;     // first row of this wave's share of the tile's A (B) rows, K offset 0
     const int8_t* baseB;
-    int64_t strideA8, strideB8;
     int lda, ldb;
     // scale values that a wave fetches with one register of per-lane offset each (32-bit: checked on the host)
     const float* fa_p;       // A's scale grid at this wave tile's row block, K block 0
     const float* fb_p;       // B's, at its column block
     uint32_t fa_ks, fb_ks;   // stride between K blocks (0 for an operand whose factor is not applied inside the loop)
-    int fa_sh, fb_sh;        // 1 for 256-wide scale groups
+    int wide;                // bit 0 / bit 1: A / B has 256-wide scale groups (two K tiles per scale)
     const float* col_p;      // B's per-row scales at the wave tile's first column (the operand's own first row when it has none)
     uint32_t col_s;          // their stride (0 when B has none)
 };
@@ -79,9 +85,16 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
     const int sw = (lane & 7) ^ ((lane >> 3) & 1);
     const int a_row_off = (wm * TM * 32 + fr_row) * 128;
     const int b_row_off = (wn * TN * 32 + fr_row) * 128;
-    int choff[4];
+    // byte address in LDS of this lane's 16 bytes of k-step ks in row 0 of its wave's A (B) rows of buffer 0: the ONLY
+    // registers fragment reads are addressed with (made opaque so that every read is one of them plus an immediate)
+    uint32_t abase[4], bbase[4];
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) choff[ks] = ((ks * 2 + fr_half) ^ sw) * 16;
+    for (int ks = 0; ks < 4; ++ks) {
+        const int choff = ((ks * 2 + fr_half) ^ sw) * 16;
+        abase[ks] = (uint32_t)(a_row_off + choff);
+        bbase[ks] = (uint32_t)(2 * A_BYTES + b_row_off + choff);
+        asm volatile("" : "+v"(abase[ks]), "+v"(bbase[ks]));
+    }
 
     constexpr int GROUP = idx::gemm_group_rows(BM);
     const int stride_t = gridDim.x;
@@ -104,15 +117,12 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
         const int rA0 = idx::gemm_wave_first_row(t.m0, wave, A_INSTR, g.M), rB0 = idx::gemm_wave_first_row(t.n0, wave, B_INSTR, g.N);
         t.baseA = g.A + (int64_t)t.batch * g.bsa + (int64_t)rA0 * g.lda;   // scalar arithmetic: every term is wave-uniform
         t.baseB = g.B + (int64_t)t.batch * g.bsb + (int64_t)rB0 * g.ldb;
-        t.strideA8 = 8 * g.lda;
-        t.strideB8 = 8 * g.ldb;
         const bool a_in = g.sa.mode != TI8_SCALE_ROW, b_in = g.sb.mode != TI8_SCALE_ROW;
         t.fa_p = g.sa.p + idx::gemm_factor_index(t.batch, g.sa.bs, idx::gemm_factor_block(t.m0 + wm * TM * 32, g.M), g.sa.rs, 0, 0, 0);
         t.fb_p = g.sb.p + idx::gemm_factor_index(t.batch, g.sb.bs, idx::gemm_factor_block(t.n0 + wn * TN * 32, g.N), g.sb.rs, 0, 0, 0);
         t.fa_ks = a_in ? (uint32_t)g.sa.ks : 0u;
         t.fb_ks = b_in ? (uint32_t)g.sb.ks : 0u;
-        t.fa_sh = g.sa.mode == TI8_SCALE_BLOCK_K256 ? 1 : 0;
-        t.fb_sh = g.sb.mode == TI8_SCALE_BLOCK_K256 ? 1 : 0;
+        t.wide = __builtin_amdgcn_readfirstlane((g.sa.mode == TI8_SCALE_BLOCK_K256 ? 1 : 0) | (g.sb.mode == TI8_SCALE_BLOCK_K256 ? 2 : 0));
         t.col_s = b_in ? 0u : (uint32_t)g.sb.rs;
         t.col_p = g.sb.p + idx::epi_col_scale_index(t.batch, g.sb.bs, idx::chain_col_scale_first(t.n0 + wn * WCOLS, g.N), g.N, t.col_s);
         return t;
@@ -121,11 +131,11 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
     // dimension each time: one multiply-add per parity instead of registers held across the loop)
     auto load_a = [&](const Tile& t, int koff, int8_t* dst) {
         const uint32_t vo[2] = {idx::gemm_lane_offset_bytes(lane, 0, t.lda), idx::gemm_lane_offset_bytes(lane, 1, t.lda)};
-        issue_tile_loads<A_INSTR>(t.baseA + koff, t.strideA8, vo, tA0, dst);
+        issue_tile_loads<A_INSTR>(t.baseA + koff, (int64_t)8 * t.lda, vo, tA0, dst);
     };
     auto load_b = [&](const Tile& t, int koff, int8_t* dst) {
         const uint32_t vo[2] = {idx::gemm_lane_offset_bytes(lane, 0, t.ldb), idx::gemm_lane_offset_bytes(lane, 1, t.ldb)};
-        issue_tile_loads<B_INSTR>(t.baseB + koff, t.strideB8, vo, tB0, dst);
+        issue_tile_loads<B_INSTR>(t.baseB + koff, (int64_t)8 * t.ldb, vo, tB0, dst);
     };
     // per-K-tile factors of a tile, K tile `lane` in each lane (raw scale values; `finish_factors` combines them).
     // Unconditional loads: an operand without in-loop factors is read with stride 0 and its value dropped.
@@ -138,8 +148,25 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
     };
     auto load_raw_factors = [&](const Tile& t, float& ra, float& rb) {
         const uint32_t kt = (uint32_t)idx::gemm_factor_kt(0, opaque_lane(), t.nk);
-        ra = t.fa_p[(kt >> t.fa_sh) * t.fa_ks];
-        rb = t.fb_p[(kt >> t.fb_sh) * t.fb_ks];
+        ra = t.fa_p[(kt >> (t.wide & 1)) * t.fa_ks];
+        rb = t.fb_p[(kt >> ((t.wide >> 1) & 1)) * t.fb_ks];
+    };
+    // the same two loads written out, for the place where the compiler must not count them: it would wait for the
+    // epilogue's stores along with them (the caller waits with the counts it knows, then calls `landed`)
+    auto load_raw_factors_uncounted = [&](const Tile& t, float& ra, float& rb) {
+        const uint32_t kt = (uint32_t)idx::gemm_factor_kt(0, opaque_lane(), t.nk);
+        const float* pa = t.fa_p + (kt >> (t.wide & 1)) * t.fa_ks;
+        const float* pb = t.fb_p + (kt >> ((t.wide >> 1) & 1)) * t.fb_ks;
+        asm volatile("global_load_dword %0, %1, off" : "=v"(ra) : "v"(pa) : "memory");
+        asm volatile("global_load_dword %0, %1, off" : "=v"(rb) : "v"(pb) : "memory");
+    };
+    auto landed = [&](float& ra, float& rb) { asm volatile("" : "+v"(ra), "+v"(rb)); };
+    // 16 bytes from LDS that the compiler does not count (the caller waits for lgkmcnt itself)
+    auto lds_read_uncounted = [&](const uint32_t* p) {
+        u32x4 v;
+        const uint32_t addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint32_t*)p;
+        asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(addr) : "memory");
+        return v;
     };
     auto finish_factors = [&](const Tile& t, float ra, float rb) {
         const GemmArgs& g = m.g[t.gi];
@@ -165,13 +192,14 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
     const v16i vzero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 
     v4i fa[2][4], fbv[TN][4];
-    auto read_a = [&](int buf, const int8_t* stage_a, int i) {
+    // block row i of the A rows (block column j of the B rows) of LDS buffer `stage`
+    auto read_a = [&](int buf, int stage, int i) {
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) fa[buf][ks] = *reinterpret_cast<const v4i*>(stage_a + a_row_off + i * 4096 + choff[ks]);
+        for (int ks = 0; ks < 4; ++ks) fa[buf][ks] = *reinterpret_cast<const v4i*>(smem + abase[ks] + (stage * A_BYTES + i * 4096));
     };
-    auto read_b = [&](const int8_t* stage_b, int ks) {
+    auto read_b = [&](int stage, int ks) {
 #pragma unroll
-        for (int j = 0; j < TN; ++j) fbv[j][ks] = *reinterpret_cast<const v4i*>(stage_b + b_row_off + j * 4096 + choff[ks]);
+        for (int j = 0; j < TN; ++j) fbv[j][ks] = *reinterpret_cast<const v4i*>(smem + bbase[ks] + (stage * B_BYTES + j * 4096));
     };
     float f_cur = 1.0f;
     auto fold = [&](int i, const v16i& d0, const v16i& d1) {
@@ -181,7 +209,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
         for (int r = 0; r < 16; ++r) accf[i][1][r] = __builtin_fmaf(static_cast<float>(d1[r]), f_cur, accf[i][1][r]);
     };
 
-    // One K tile.  `step` counts K tiles since the kernel started (LDS buffer = step & 1); the B half of the K tile
+    // One K tile in LDS buffer `parity` (a tile's K tile kt sits in buffer kt & 1); the B half of the K tile
     // after this one is issued at the top, the A half of the one after that behind the barrier: `nb` / `na` say where
     // those come from (this tile or the next output tile).
     // `read_next`: whether the last block row also reads the next K tile's first fragments (not across a tile
@@ -189,14 +217,14 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
     // `first`: the first K tile of an output tile.  The B half of its successor is already on its way (issued before the
     // previous tile's epilogue), and it waits only for the loads issued before that epilogue's stores: the stores
     // (`stores_pending` of them at most, the youngest operations of this wave) drain while this K tile is multiplied.
-    auto ktile = [&](auto first_tag, auto read_next_tag, bool stores_pending, int step, float fvec, int kt, const Tile& nb, int koff_b,
-                     const Tile& na, int koff_a) {
+    // `parity` is a compile-time value, so that every LDS address of the K tile is a register plus an immediate
+    // (with the buffer chosen at run time each fragment read costs a vector add: 17 per K tile and wave).
+    auto ktile_p = [&](auto first_tag, auto read_next_tag, auto parity_tag, bool stores_pending, float fvec, int kt, const Tile& nb, int koff_b,
+                       const Tile& na, int koff_a) {
         constexpr bool FIRST = decltype(first_tag)::value;
         constexpr bool READ_NEXT = decltype(read_next_tag)::value;
-        const int cur = step & 1;
-        const int8_t* stA = ldsA + cur * A_BYTES;
-        const int8_t* stAn = ldsA + (cur ^ 1) * A_BYTES;
-        const int8_t* stBn = ldsB + (cur ^ 1) * B_BYTES;
+        constexpr int cur = decltype(parity_tag)::value;
+        constexpr int stA = cur, stAn = cur ^ 1, stBn = cur ^ 1;
         f_cur = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fvec), kt));
         if (!FIRST) load_b(nb, koff_b, wB + (cur ^ 1) * B_BYTES);
 #pragma unroll
@@ -305,13 +333,18 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
                         }
                     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): same wave reads what it wrote, no barrier
                     __builtin_amdgcn_wave_barrier();
-                    uint4 w[2][2];
+                    // the read-back is written out: before an LDS read that it knows, the compiler waits for the operand loads
+                    // in flight (they write LDS too), i.e. for the next tile's K tile 1 issued a moment ago
+                    u32x4 w[2][2];
 #pragma unroll
                     for (int k = 0; k < 2; ++k) {
                         const int rr = rb_row + k * RPI;
-                        w[k][0] = *reinterpret_cast<const uint4*>(slab + idx::epi_chain_slab_word(rr, rb_col));
-                        w[k][1] = *reinterpret_cast<const uint4*>(slab + idx::epi_chain_slab_word(rr, rb_col + 4));
+                        w[k][0] = lds_read_uncounted(slab + idx::epi_chain_slab_word(rr, rb_col));
+                        w[k][1] = lds_read_uncounted(slab + idx::epi_chain_slab_word(rr, rb_col + 4));
                     }
+                    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+#pragma unroll
+                    for (int k = 0; k < 2; ++k) asm volatile("" : "+v"(w[k][0]), "+v"(w[k][1]));
 #pragma unroll
                     for (int k = 0; k < 2; ++k, off += c_step) {
                         const uint32_t wb[8] = {w[k][0].x, w[k][0].y, w[k][0].z, w[k][0].w, w[k][1].x, w[k][1].y, w[k][1].z, w[k][1].w};
@@ -365,10 +398,9 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
         load_a(cur, 128, wA + A_BYTES);
         load_b(cur, 128, wB + B_BYTES);
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) read_b(ldsB, ks);
-        read_a(0, ldsA, 0);
+        for (int ks = 0; ks < 4; ++ks) read_b(0, ks);
+        read_a(0, 0, 0);
     }
-    int step = 0;
     bool stored = false;   // whether this wave's previous epilogue left stores behind
     while (true) {
         const int nk = cur.nk;
@@ -376,22 +408,23 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
         // in the last of them K tile 0 of the next
         using T_ = std::true_type;
         using F_ = std::false_type;
-        if (nk > 1) {
+        using P0 = std::integral_constant<int, 0>;
+        using P1 = std::integral_constant<int, 1>;
+        // K / 128 is even: a tile starts in LDS buffer 0 and its K tiles alternate 0, 1, 0, 1, ...
+        {
             const bool a_next = 2 >= nk;
-            ktile(T_{}, T_{}, stored, step, fvec, 0, cur, 128, a_next ? nxt : cur, a_next ? 0 : 256);
-            ++step;
+            ktile_p(T_{}, T_{}, P0{}, stored, fvec, 0, cur, 128, a_next ? nxt : cur, a_next ? 0 : 256);
         }
-        for (int kt = 1; kt < nk - 1; ++kt, ++step) {
-            const bool a_next = kt + 2 >= nk;
-            ktile(F_{}, T_{}, false, step, fvec, kt, cur, (kt + 1) * 128, a_next ? nxt : cur, a_next ? 0 : (kt + 2) * 128);
+        for (int kt = 1; kt < nk - 1; kt += 2) {
+            ktile_p(F_{}, T_{}, P1{}, false, fvec, kt, cur, (kt + 1) * 128, cur, (kt + 2) * 128);
+            const bool a_next = kt + 3 >= nk;
+            ktile_p(F_{}, T_{}, P0{}, false, fvec, kt + 1, cur, (kt + 2) * 128, a_next ? nxt : cur, a_next ? 0 : (kt + 3) * 128);
         }
-        // last K tile: the column scales of this tile's epilogue and the next tile's factors travel beside it
-        float coln[4], ra, rb;
+        // last K tile: the column scales of this tile's epilogue travel beside it
+        float coln[4];
         load_col_scales(cur, coln);
-        load_raw_factors(nxt, ra, rb);
         __builtin_amdgcn_sched_barrier(0);
-        ktile(F_{}, F_{}, false, step, fvec, nk - 1, nxt, 0, nxt, 128);
-        ++step;
+        ktile_p(F_{}, F_{}, P1{}, false, fvec, nk - 1, nxt, 0, nxt, 128);
         // the accumulators are complete HERE: without this the optimiser moves the last K tile's convert + fma behind
         // the epilogue's branches and keeps that tile's 128 int32 results alive until then
 #pragma unroll
@@ -402,16 +435,25 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
                 asm volatile("" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7]),
                                   "+v"(a[8]), "+v"(a[9]), "+v"(a[10]), "+v"(a[11]), "+v"(a[12]), "+v"(a[13]), "+v"(a[14]), "+v"(a[15]));
             }
-        fvec = finish_factors(nxt, ra, rb);
+        // the next tile's factors: fetched here, ahead of the stores, and combined behind the epilogue (operations complete in
+        // issue order, so waiting for them does not wait for the stores)
+        float ra, rb;
+        load_raw_factors_uncounted(nxt, ra, rb);
         // the B half of the next tile's K tile 1, into the buffer the last K tile's B has left: issued before the epilogue's
         // stores, so that the next tile's first K tile need not wait for them
-        load_b(nxt, 128, wB + ((step - 1) & 1) * B_BYTES);
+        load_b(nxt, 128, wB + B_BYTES);
         stored = epilogue(cur, coln);
         if (!more) break;
+        // the factor loads were issued before the 4 loads of the B half and the stores: done once at most that many operations are
+        // outstanding (said explicitly: the compiler would wait for everything, stores included, at the head of the tile loop)
+        if (stored) __builtin_amdgcn_s_waitcnt(WAIT_FACTORS_BEHIND_STORES);
+        else __builtin_amdgcn_s_waitcnt(WAIT_FACTORS);
+        landed(ra, rb);
+        fvec = finish_factors(nxt, ra, rb);
         // the next tile's K tile 0 has been in LDS since the barrier of the last K tile: its first fragments
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) read_b(ldsB + (step & 1) * B_BYTES, ks);
-        read_a(0, ldsA + (step & 1) * A_BYTES, 0);
+        for (int ks = 0; ks < 4; ++ks) read_b(0, ks);
+        read_a(0, 0, 0);
         // the accumulators are free: the place for the integer divisions that find the tile after the next
         T += stride_t;
         cur = nxt;
@@ -431,7 +473,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
 bool chain_persistent_supported(const GemmMulti& m) {
     for (int i = 0; i < m.count; ++i) {
         const int nk = m.g[i].K >> 7;
-        if (nk < 2 || nk > 64 || m.g[i].strict) return false;
+        if (nk < 2 || nk > 64 || (nk & 1) || m.g[i].strict) return false;
         if (m.g[i].sa.mode == TI8_SCALE_ROW_K128 || m.g[i].sb.mode == TI8_SCALE_ROW_K128) return false;
         // per-lane offsets into the scale arrays are kept in 32 bits: 64 K blocks x stride, 64 columns x stride
         const int64_t lim = (int64_t)1 << 24;
