@@ -91,6 +91,8 @@ enum ti8_gemm_flags {
                              moves results by a few fp32 ulps before the bf16 rounding */
     TI8_GEMM_TILED = 2,   /* always take an LDS-tiled kernel (tile size still chosen by the shape) */
     TI8_GEMM_LARGE_TILES = 8, /* LDS-tiled kernel with the largest tiles (256 x 256) whatever the shape */
+    TI8_GEMM_ONE_TILE = 16,   /* one workgroup per output tile also where the block-channel promotion would run on
+                                 persistent workgroups (one per CU walking its tiles); same bits either way */
     TI8_GEMM_SKINNY = 4   /* take the few-rows kernel (no LDS staging, K split over waves) whenever
                              it supports the scale modes; by default it is used for M <= 256.  Both
                              kernels give bit-identical results with acc_i32_full; otherwise their

@@ -153,6 +153,48 @@ def test_gemms_of_a_step_in_one_launch(T, dev):
     assert torch.equal(Yr, Y1[:300]) and torch.equal(dXr, dX1[:300]) and torch.equal(dWr, dW1)
 
 
+@pytest.mark.parametrize("M,N,K,batch", [(640, 896, 256, 1), (384, 1152, 512, 3), (1024, 768, 1024, 2), (896, 640, 8192, 1), (4096, 4096, 512, 1)])
+def test_persistent_workgroups_match_one_tile_kernel(T, dev, M, N, K, batch):
+    """The chained block-channel promotion on persistent workgroups (one per CU walking its 256 x 256 tiles, the next tile's
+    operands fetched by the current tile's last K tiles) against the same arithmetic with one workgroup per tile, bit for bit,
+    and against the oracle per element: tiles that hang over M and N, batches, 2 to 64 K tiles, fewer tiles than CUs and
+    several tiles per workgroup, every scale layout, the extra output factor."""
+    from triton_int8_amd import ops
+    from triton_int8_amd._lib import COMBINE_MUL_PROD, SCALE_BLOCK128, SCALE_ROW
+    g = make_gen(M + N + K + batch)
+    A = torch.randint(-127, 128, (batch, M, K), generator=g, dtype=torch.int8)
+    B = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+    B3 = torch.randint(-127, 128, (batch, N, K), generator=g, dtype=torch.int8)
+    pos = lambda *shape: torch.rand(*shape, generator=g) * 1e-2 + 1e-4
+    sa_row, sa_blk = pos(batch, M), pos(batch, M // 128, K // 128)
+    sb_row, sb_blk, sb3_blk = pos(N), pos(N // 128, K // 128), pos(batch, N // 128, K // 128)
+    Ad, Bd, B3d = A.to(dev), B.to(dev), B3.to(dev)
+
+    def run(persistent, *args, **kw):
+        ops.GEMM_PATH, ops.GEMM_PERSISTENT = "large", persistent
+        try:
+            with T._lib.timed_launches() as rec:
+                out = ops.gemm_i8_nt(*args, **kw)
+            assert list(rec) == ["ti8_gemm_i8_nt"]
+            return out
+        finally:
+            ops.GEMM_PATH, ops.GEMM_PERSISTENT = "auto", True
+
+    cases = [(sa_blk, SCALE_BLOCK128, olin.BLOCK, B, Bd, sb_row, SCALE_ROW, olin.ROW, {}),
+             (sa_blk, SCALE_BLOCK128, olin.BLOCK, B3, B3d, sb3_blk, SCALE_BLOCK128, olin.BLOCK, {}),
+             (sa_row, SCALE_ROW, olin.ROW, B, Bd, sb_blk, SCALE_BLOCK128, olin.BLOCK, {"out_scale": 2.0 ** -7}),
+             (sa_blk, SCALE_BLOCK128, olin.BLOCK, B, Bd, sb_row, SCALE_ROW, olin.ROW, {"combine": COMBINE_MUL_PROD})]
+    for sA, mA, oA, Bq, Bqd, sB, mB, oB, kw in cases:
+        args = (Ad, Bqd, sA.to(dev), mA, sB.to(dev), mB)
+        got = run(True, *args, **kw)
+        assert torch.equal(got, run(False, *args, **kw)), (mA, mB, kw)
+        for b in (0, batch - 1):   # the oracle on the first and the last batch
+            want = olin.gemm_scaled(A[b], sA[b], oA, Bq[b] if Bq.dim() == 3 else Bq, sB[b] if sB.dim() == 3 else sB, oB,
+                                    out_scale=kw.get("out_scale"))
+            assert rel_err(got[b], want) <= FAST_TOL
+            assert_one_ulp(got[b], want, f"persistent {M}x{N}x{K} batch {b} modes {mA}/{mB}")
+
+
 def test_block_quant_of_several_operands_in_one_launch(T, dev):
     """ti8_quant_block_multi = separate ti8_quant_block calls, bit for bit: operands of different shapes,
     with and without the transposed copy, and the layer step that uses it for X and dY."""

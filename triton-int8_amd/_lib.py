@@ -54,7 +54,7 @@ Q_CLAMP, Q_EPS_ADD, Q_SCALE_BF16, Q_HAD128, Q_WS_PINGPONG, Q_WS_SECOND, Q_TORCH_
 INV_RCP_OF_SCALE, INV_AMAX_DIV_127, INV_AMAX_MUL_RCP127, INV_MULTIPLIER = 0, 1, 2, 3
 SCALE_ROW, SCALE_BLOCK128, SCALE_ROW_K128, SCALE_BLOCK_K256 = 0, 1, 2, 3
 COMBINE_MUL_MUL, COMBINE_MUL_PROD, COMBINE_DIV_PROD = 0, 1, 2
-GEMM_STRICT, GEMM_TILED, GEMM_SKINNY, GEMM_LARGE_TILES = 1, 2, 4, 8
+GEMM_STRICT, GEMM_TILED, GEMM_SKINNY, GEMM_LARGE_TILES, GEMM_ONE_TILE = 1, 2, 4, 8, 16
 NOALLOC_MAX_ROWS_PLUS_COLS = 65536
 
 _lib = None

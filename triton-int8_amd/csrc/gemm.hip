@@ -15,7 +15,6 @@
 // operand and the 16 bytes k = 16*(l / 32) .. +15 of the 32-deep slice (the same map
 // for both operands, which is all an NT dot product needs); result register r of lane
 // l is C[8*(r/4) + 4*(l/32) + r%4][l % 32] with rows from A and columns from B.
-#include <cstdlib>
 #include <type_traits>
 #include "gemm_args.h"
 
@@ -631,7 +630,7 @@ static int prepare_gemm(const char* fn, const ti8_gemm_problem& p, int gemm_flag
     if (p.modeA == TI8_SCALE_ROW && (p.sa_rs < 0 || p.sa_rs > 0x00ffffff))
         return fail(TI8_ERR_SHAPE, "%s: row stride of A's scales must be in [0, 2^24)", fn);
     if (p.combine < 0 || p.combine > 2) return fail(TI8_ERR_MODE, "%s: unknown combine %d", fn, p.combine);
-    if (gemm_flags & ~(TI8_GEMM_STRICT | TI8_GEMM_TILED | TI8_GEMM_SKINNY | TI8_GEMM_LARGE_TILES)) return fail(TI8_ERR_MODE, "%s: unknown flag 0x%x", fn, gemm_flags);
+    if (gemm_flags & ~(TI8_GEMM_STRICT | TI8_GEMM_TILED | TI8_GEMM_SKINNY | TI8_GEMM_LARGE_TILES | TI8_GEMM_ONE_TILE)) return fail(TI8_ERR_MODE, "%s: unknown flag 0x%x", fn, gemm_flags);
     if ((gemm_flags & TI8_GEMM_SKINNY) && (gemm_flags & (TI8_GEMM_TILED | TI8_GEMM_LARGE_TILES)))
         return fail(TI8_ERR_MODE, "%s: TI8_GEMM_SKINNY excludes TI8_GEMM_TILED and TI8_GEMM_LARGE_TILES", fn);
     if (p.acc_i32_full && (p.modeA != TI8_SCALE_ROW || p.modeB != TI8_SCALE_ROW))
@@ -652,9 +651,6 @@ static int prepare_gemm(const char* fn, const ti8_gemm_problem& p, int gemm_flag
     *out = a;
     return TI8_OK;
 }
-
-// the chained promotion runs on persistent workgroups (gemm_chain.hip) unless TI8_ONE_TILE_CHAIN is set in the environment
-static const bool PERSISTENT_CHAIN = getenv("TI8_ONE_TILE_CHAIN") == nullptr;
 
 static int device_cu_count() {
     static int num_cu = 0;
@@ -684,8 +680,8 @@ static int try_chain_persistent(GemmMulti& m, const int64_t* batch, hipStream_t 
 }
 
 // One GEMM on the LDS-tiled kernel that `c` names
-static int launch_tiled(const char* fn, const GemmArgs& a, int64_t batch, const idx::GemmConfig& c, hipStream_t st) {
-    if (c.epi == EPI_PROMOTE_CHAIN && PERSISTENT_CHAIN) {
+static int launch_tiled(const char* fn, const GemmArgs& a, int64_t batch, const idx::GemmConfig& c, bool persistent, hipStream_t st) {
+    if (c.epi == EPI_PROMOTE_CHAIN && persistent) {
         GemmMulti m;
         m.count = 1;
         m.g[0] = a;
@@ -727,7 +723,8 @@ extern "C" int ti8_gemm_i8_nt(const int8_t* A, int64_t bsa, int64_t lda, const i
     if (M % 128)
         return fail(TI8_ERR_SHAPE, "%s: M = %lld is not a multiple of 128, which only the few-rows kernel accepts "
                     "(not with TI8_GEMM_STRICT / TI8_GEMM_TILED, per-(row, K tile) scales or K > 32768)", fn, (long long)M);
-    return launch_tiled(fn, a, batch, idx::gemm_config(M, N, K, batch, acc_i32_full != 0, a.strict != 0, modeA, modeB, large, device_cu_count()), st);
+    return launch_tiled(fn, a, batch, idx::gemm_config(M, N, K, batch, acc_i32_full != 0, a.strict != 0, modeA, modeB, large, device_cu_count()),
+                        !(gemm_flags & TI8_GEMM_ONE_TILE), st);
 }
 
 extern "C" int ti8_gemm_i8_nt_multi(const ti8_gemm_problem* problems, int count, int gemm_flags, ti8_stream_t stream) {
@@ -751,7 +748,8 @@ extern "C" int ti8_gemm_i8_nt_multi(const ti8_gemm_problem* problems, int count,
     }
     one_launch = one_launch && c[0].epi != EPI_STRICT && c[0].epi != EPI_PROMOTE_LANE;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (one_launch && c[0].epi == EPI_PROMOTE_CHAIN && PERSISTENT_CHAIN) {
+    const bool persistent = !(gemm_flags & TI8_GEMM_ONE_TILE);
+    if (one_launch && c[0].epi == EPI_PROMOTE_CHAIN && persistent) {
         const int64_t ones[GEMM_MULTI_MAX] = {1, 1, 1};
         const int rc = try_chain_persistent(m, ones, st);
         if (rc != CHAIN_UNAVAILABLE) return rc;
@@ -767,7 +765,7 @@ extern "C" int ti8_gemm_i8_nt_multi(const ti8_gemm_problem* problems, int count,
 #undef TI8_GEMM_CASE
     }
     for (int i = 0; i < count; ++i)
-        if (int e = launch_tiled(fn, m.g[i], 1, c[i], st)) return e;
+        if (int e = launch_tiled(fn, m.g[i], 1, c[i], persistent, st)) return e;
     return TI8_OK;
 }
 

@@ -11,7 +11,7 @@ import threading
 import torch
 
 from . import _lib
-from ._lib import (COMBINE_DIV_PROD, COMBINE_MUL_MUL, COMBINE_MUL_PROD, GEMM_LARGE_TILES, GEMM_SKINNY, GEMM_STRICT, GEMM_TILED, INV_AMAX_DIV_127,
+from ._lib import (COMBINE_DIV_PROD, COMBINE_MUL_MUL, COMBINE_MUL_PROD, GEMM_LARGE_TILES, GEMM_ONE_TILE, GEMM_SKINNY, GEMM_STRICT, GEMM_TILED, INV_AMAX_DIV_127,
                    INV_AMAX_MUL_RCP127, INV_MULTIPLIER, INV_RCP_OF_SCALE, Q_CLAMP, Q_EPS_ADD, Q_HAD128, Q_SCALE_BF16, Q_TORCH_BF16, Q_TORCH_ROUND,
                    Q_WS_PINGPONG, Q_WS_SECOND,
                    SCALE_BLOCK128, SCALE_BLOCK_K256, SCALE_ROW, SCALE_ROW_K128)
@@ -24,6 +24,8 @@ __all__ = ["quant_block", "quant_block_multi", "quant_block_had128", "quant_row"
 # whatever the shape) or "skinny" (wherever it supports the scale modes).  Tests set it to run
 # the same cases through every kernel.
 GEMM_PATH = "auto"
+# False: one workgroup per output tile also where the block-channel promotion would run on persistent workgroups (same bits)
+GEMM_PERSISTENT = True
 
 
 def _stream():
@@ -337,7 +339,8 @@ def gemm_i8_nt(A, B, sA, modeA, sB, modeB, *, acc_i32_full=False, combine=COMBIN
               out.data_ptr(), out.stride(0), out.stride(1),
               sAv.data_ptr(), modeA, sa_bs, sa_rs, sa_ks, sBv.data_ptr(), modeB, sb_bs, sb_rs, sb_ks,
               batch, M, N, K, 1 if acc_i32_full else 0, combine, float(out_scale), float(post_scale),
-              (GEMM_STRICT if strict else 0) | {"auto": 0, "tiled": GEMM_TILED, "skinny": GEMM_SKINNY, "large": GEMM_LARGE_TILES}[GEMM_PATH],
+              (GEMM_STRICT if strict else 0) | {"auto": 0, "tiled": GEMM_TILED, "skinny": GEMM_SKINNY, "large": GEMM_LARGE_TILES}[GEMM_PATH]
+              | (0 if GEMM_PERSISTENT else GEMM_ONE_TILE),
               _stream())
     return out
 
@@ -372,7 +375,7 @@ def gemm_i8_nt_multi(problems):
                                     float(p.get("out_scale", 1.0)), float(p.get("post_scale", 0.0)))
         outs.append(out)
         keep.append((A, B, sAv, sBv))     # contiguous copies stay alive until the launch is queued
-    _lib.call("ti8_gemm_i8_nt_multi", descs, len(problems), {"auto": 0, "tiled": GEMM_TILED, "large": GEMM_LARGE_TILES}.get(GEMM_PATH, 0), _stream())
+    _lib.call("ti8_gemm_i8_nt_multi", descs, len(problems), {"auto": 0, "tiled": GEMM_TILED, "large": GEMM_LARGE_TILES}.get(GEMM_PATH, 0) | (0 if GEMM_PERSISTENT else GEMM_ONE_TILE), _stream())
     return outs
 
 
