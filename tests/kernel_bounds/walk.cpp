@@ -412,7 +412,7 @@ int walk_gemm_chain(int64_t bsa, int64_t lda, int64_t bsb, int64_t ldb, int64_t 
     const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN), per_batch = tiles_m * tiles_n;
     const int total = per_batch * (int)batch, nk = (int)(K >> 7), GROUP = gemm_group_rows(BM);
     const int64_t lds_words = (2 * (BM + BN) * 128 + NW * 16 * WCOLS * 4) / 4, slab0 = 2 * (BM + BN) * 128 / 4;
-    if (nk < 2 || nk > 64) { r.fail("gemm chain: K / 128 = %d outside [2, 64]", nk); *n_checked = 0; return 1; }
+    if (nk < 2 || nk > 256 || (nk & 1)) { r.fail("gemm chain: K / 128 = %d is odd or outside [2, 256]", nk); *n_checked = 0; return 1; }
     std::vector<uint8_t> stored(c_elems <= (int64_t)1 << 30 ? (size_t)c_elems : 0, 0);
     std::vector<uint8_t> seen((size_t)total, 0);
     const bool a_in = sa.mode != 0, b_in = sb.mode != 0;
@@ -446,9 +446,11 @@ int walk_gemm_chain(int64_t bsa, int64_t lda, int64_t bsb, int64_t ldb, int64_t 
                     // per-K-tile factors: scalar base + (K tile >> shift) * stride per lane
                     const int64_t fa = gemm_factor_index(by, sa.bs, gemm_factor_block(m0 + wm * TM * 32, (int)M), sa.rs, 0, 0, 0);
                     const int64_t fb = gemm_factor_index(by, sb.bs, gemm_factor_block(n0 + wn * TN * 32, (int)N), sb.rs, 0, 0, 0);
-                    const uint32_t kt = (uint32_t)gemm_factor_kt(0, lane, nk);
-                    r.access("gemm chain factor A", fa + (int64_t)((kt >> (sa.mode == 3 ? 1 : 0)) * (uint32_t)(a_in ? sa.ks : 0)), 1, sa.elems, T, wave, lane, 0);
-                    r.access("gemm chain factor B", fb + (int64_t)((kt >> (sb.mode == 3 ? 1 : 0)) * (uint32_t)(b_in ? sb.ks : 0)), 1, sb.elems, T, wave, lane, 0);
+                    for (int c = 0; c <= (nk - 1) >> 6; ++c) {   // the factor register is refilled every 64 K tiles
+                        const uint32_t kt = (uint32_t)gemm_factor_kt(c, lane, nk);
+                        r.access("gemm chain factor A", fa + (int64_t)((kt >> (sa.mode == 3 ? 1 : 0)) * (uint32_t)(a_in ? sa.ks : 0)), 1, sa.elems, T, wave, lane, c);
+                        r.access("gemm chain factor B", fb + (int64_t)((kt >> (sb.mode == 3 ? 1 : 0)) * (uint32_t)(b_in ? sb.ks : 0)), 1, sb.elems, T, wave, lane, c);
+                    }
                     // column scales: 4 per lane from the wave tile's first column (clamped for a tile outside N)
                     const uint32_t cs = b_in ? 0u : (uint32_t)sb.rs;
                     const int64_t colp = epi_col_scale_index(by, sb.bs, chain_col_scale_first(n0 + wn * WCOLS, (int)N), (int)N, cs);

@@ -153,11 +153,11 @@ def test_gemms_of_a_step_in_one_launch(T, dev):
     assert torch.equal(Yr, Y1[:300]) and torch.equal(dXr, dX1[:300]) and torch.equal(dWr, dW1)
 
 
-@pytest.mark.parametrize("M,N,K,batch", [(640, 896, 256, 1), (384, 1152, 512, 3), (1024, 768, 1024, 2), (896, 640, 8192, 1), (4096, 4096, 512, 1)])
+@pytest.mark.parametrize("M,N,K,batch", [(640, 896, 256, 1), (384, 1152, 512, 3), (1024, 768, 1024, 2), (896, 640, 8192, 1), (4096, 4096, 512, 1), (640, 384, 14336, 1), (384, 640, 16640, 2), (512, 512, 32768, 1)])
 def test_persistent_workgroups_match_one_tile_kernel(T, dev, M, N, K, batch):
     """The chained block-channel promotion on persistent workgroups (one per CU walking its 256 x 256 tiles, the next tile's
     operands fetched by the current tile's last K tiles) against the same arithmetic with one workgroup per tile, bit for bit,
-    and against the oracle per element: tiles that hang over M and N, batches, 2 to 64 K tiles, fewer tiles than CUs and
+    and against the oracle per element: tiles that hang over M and N, batches, 2 to 256 K tiles (the factor register refilled every 64), fewer tiles than CUs and
     several tiles per workgroup, every scale layout, the extra output factor."""
     from triton_int8_amd import ops
     from triton_int8_amd._lib import COMBINE_MUL_PROD, SCALE_BLOCK128, SCALE_ROW

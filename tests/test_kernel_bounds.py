@@ -111,7 +111,7 @@ def walk(lib, allocs, name, a):
             sb = ScaleArg(mB, sb_bs, sb_rs, sb_ks, allocs.room(sB, 4))
             rc = lib.walk_gemm(bsa, lda, bsb, ldb, bsc, ldc, ctypes.byref(sa), ctypes.byref(sb), batch, M, N, K, acc, flags & 1, (flags >> 3) & 1, 0,
                                NUM_CU, allocs.room(A, 1), allocs.room(B, 1), allocs.room(C, 2), picked, ctypes.byref(n), msg, 512)
-            if rc == 0 and picked[2] == 5 and 2 <= K // 128 <= 64 and K % 256 == 0:   # the chained promotion runs on persistent workgroups
+            if rc == 0 and picked[2] == 5 and 2 <= K // 128 <= 256 and K % 256 == 0:   # the chained promotion runs on persistent workgroups
                 first = n.value
                 tiles = -(-M // 256) * -(-N // 256) * batch
                 rc = lib.walk_gemm_chain(bsa, lda, bsb, ldb, bsc, ldc, ctypes.byref(sa), ctypes.byref(sb), batch, M, N, K, min(tiles, NUM_CU),
@@ -136,7 +136,7 @@ def walk(lib, allocs, name, a):
             assert rc == 0, f"{name}, GEMM {i}: {msg.value.decode()}"
             total += n.value
             tiles[i] = -(-p.M // picked[0]) * -(-p.N // picked[1])
-            if picked[2] == 5 and 2 <= p.K // 128 <= 64 and p.K % 256 == 0:   # persistent workgroups: each GEMM's tiles as one workgroup list walks them
+            if picked[2] == 5 and 2 <= p.K // 128 <= 256 and p.K % 256 == 0:   # persistent workgroups: each GEMM's tiles as one workgroup list walks them
                 rc = lib.walk_gemm_chain(p.bsa, p.lda, p.bsb, p.ldb, p.bsc, p.ldc, ctypes.byref(sa), ctypes.byref(sb), 1, p.M, p.N, p.K,
                                          min(tiles[i], NUM_CU), allocs.room(p.A, 1), allocs.room(p.B, 1), allocs.room(p.C, 2), ctypes.byref(n), msg, 512)
                 assert rc == 0, f"{name}, GEMM {i} (persistent): {msg.value.decode()}"
@@ -261,7 +261,7 @@ def test_multi_launch_map(walker, tiles):
 
 
 @pytest.mark.parametrize("M,N,K,batch,mA,mB,grid", [(8192, 4096, 4096, 1, 1, 0, 256), (4096, 4096, 8192, 1, 1, 1, 256), (4224, 4480, 256, 1, 1, 0, 256),
-                                                    (2048, 2304, 1024, 3, 0, 1, 256), (1152, 1408, 512, 2, 3, 0, 7), (8192, 8192, 512, 1, 0, 0, 256)])
+                                                    (2048, 2304, 1024, 3, 0, 1, 256), (1152, 1408, 512, 2, 3, 0, 7), (8192, 8192, 512, 1, 0, 0, 256), (4096, 4096, 16384, 1, 1, 1, 256), (1280, 768, 32768, 1, 1, 0, 15)])
 def test_persistent_chain_kernel_geometries(walker, M, N, K, batch, mA, mB, grid):
     """gemm_i8_chain_kernel: tile lists of persistent workgroups, tiles that hang over M or N, batches, every scale layout."""
     def desc(mode, rows):

@@ -11,10 +11,10 @@
 // Per tile this leaves the epilogue's own instructions; measured against one workgroup per tile: the
 // prologue, the workgroup turn-over and most of the store drain.
 // Arithmetic, operand layout in LDS, fragment reads and accumulator layout are those of the chained loop
-// in gemm.hip; results are bit-identical.  Limits: K / 128 even and in [2, 64] for every GEMM of the launch (one
-// register holds a tile's per-K-tile factors, and a tile's K tiles alternate between the two LDS buffers from a
-// fixed start, which makes every LDS address a register plus an immediate; the launcher sends other shapes to
-// the one-tile kernel).
+// in gemm.hip; results are bit-identical.  Limits: K / 128 even and in [2, 256] for every GEMM of the launch (a
+// tile's K tiles alternate between the two LDS buffers from a fixed start, which makes every LDS address a register
+// plus an immediate; one register holds the per-K-tile factors of 64 K tiles and is refilled every 64; the launcher
+// sends other shapes to the one-tile kernel).
 #include <type_traits>
 #include "gemm_args.h"
 
@@ -137,7 +137,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
         const uint32_t vo[2] = {idx::gemm_lane_offset_bytes(lane, 0, t.ldb), idx::gemm_lane_offset_bytes(lane, 1, t.ldb)};
         issue_tile_loads<B_INSTR>(t.baseB + koff, (int64_t)8 * t.ldb, vo, tB0, dst);
     };
-    // per-K-tile factors of a tile, K tile `lane` in each lane (raw scale values; `finish_factors` combines them).
+    // per-K-tile factors of a tile, K tile 64 `block64` + lane in each lane (raw scale values; `finish_factors` combines them).
     // Unconditional loads: an operand without in-loop factors is read with stride 0 and its value dropped.
     // (lane-derived values of the once-per-tile code are rebuilt from an opaque copy of the lane number: hoisted out
     // of the tile loop they would sit in registers that the K loop has no room for)
@@ -146,8 +146,8 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
         asm volatile("" : "+v"(l));
         return l;
     };
-    auto load_raw_factors = [&](const Tile& t, float& ra, float& rb) {
-        const uint32_t kt = (uint32_t)idx::gemm_factor_kt(0, opaque_lane(), t.nk);
+    auto load_raw_factors = [&](const Tile& t, int block64, float& ra, float& rb) {
+        const uint32_t kt = (uint32_t)idx::gemm_factor_kt(block64, opaque_lane(), t.nk);
         ra = t.fa_p[(kt >> (t.wide & 1)) * t.fa_ks];
         rb = t.fb_p[(kt >> ((t.wide >> 1) & 1)) * t.fb_ks];
     };
@@ -225,7 +225,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
         constexpr bool READ_NEXT = decltype(read_next_tag)::value;
         constexpr int cur = decltype(parity_tag)::value;
         constexpr int stA = cur, stAn = cur ^ 1, stBn = cur ^ 1;
-        f_cur = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fvec), kt));
+        f_cur = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fvec), kt & 63));
         if (!FIRST) load_b(nb, koff_b, wB + (cur ^ 1) * B_BYTES);
 #pragma unroll
         for (int i = 0; i < TM - 1; ++i) {
@@ -391,7 +391,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
         load_a(cur, 0, wA);
         load_b(cur, 0, wB);
         float ra, rb;
-        load_raw_factors(cur, ra, rb);
+        load_raw_factors(cur, 0, ra, rb);
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
         fvec = finish_factors(cur, ra, rb);
@@ -415,10 +415,25 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
             const bool a_next = 2 >= nk;
             ktile_p(T_{}, T_{}, P0{}, stored, fvec, 0, cur, 128, a_next ? nxt : cur, a_next ? 0 : 256);
         }
-        for (int kt = 1; kt < nk - 1; kt += 2) {
+        // K tiles 1 .. nk - 2 in pairs (buffer 1, buffer 0).  The register `fvec` holds the factors of 64 K tiles: the pair that
+        // straddles a multiple of 64 sits outside the inner loop and refills it in between (waited for on the spot: once per 64 K tiles)
+        for (int kt = 1; kt < nk - 1;) {
+            const int last = (kt | 63) - 2 < nk - 3 ? (kt | 63) - 2 : nk - 3;   // last odd K tile whose pair lies inside this block of 64
+            for (; kt <= last; kt += 2) {
+                ktile_p(F_{}, T_{}, P1{}, false, fvec, kt, cur, (kt + 1) * 128, cur, (kt + 2) * 128);
+                const bool a_next = kt + 3 >= nk;
+                ktile_p(F_{}, T_{}, P0{}, false, fvec, kt + 1, cur, (kt + 2) * 128, a_next ? nxt : cur, a_next ? 0 : (kt + 3) * 128);
+            }
+            if (kt >= nk - 1) break;
             ktile_p(F_{}, T_{}, P1{}, false, fvec, kt, cur, (kt + 1) * 128, cur, (kt + 2) * 128);
+            {
+                float ra, rb;
+                load_raw_factors(cur, (kt + 1) >> 6, ra, rb);
+                fvec = finish_factors(cur, ra, rb);
+            }
             const bool a_next = kt + 3 >= nk;
             ktile_p(F_{}, T_{}, P0{}, false, fvec, kt + 1, cur, (kt + 2) * 128, a_next ? nxt : cur, a_next ? 0 : (kt + 3) * 128);
+            kt += 2;
         }
         // last K tile: the column scales of this tile's epilogue travel beside it
         float coln[4];
@@ -473,7 +488,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
 bool chain_persistent_supported(const GemmMulti& m) {
     for (int i = 0; i < m.count; ++i) {
         const int nk = m.g[i].K >> 7;
-        if (nk < 2 || nk > 64 || (nk & 1) || m.g[i].strict) return false;
+        if (nk < 2 || nk > 256 || (nk & 1) || m.g[i].strict) return false;
         if (m.g[i].sa.mode == TI8_SCALE_ROW_K128 || m.g[i].sb.mode == TI8_SCALE_ROW_K128) return false;
         // per-lane offsets into the scale arrays are kept in 32 bits: 64 K blocks x stride, 64 columns x stride
         const int64_t lim = (int64_t)1 << 24;
