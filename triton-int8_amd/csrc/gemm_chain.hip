@@ -191,7 +191,9 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
             for (int r = 0; r < 16; ++r) accf[i][j][r] = 0.0f;
     const v16i vzero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 
-    v4i fa[2][4], fbv[TN][4];
+    // A fragments of ONE block row: the next row's are read behind the MFMAs that use the registers and in front of the convert + fma
+    // that follows, which covers the LDS latency (a second set, read one row ahead, measured 1 % slower and costs 16 registers)
+    v4i fa[1][4], fbv[TN][4];
     // block row i of the A rows (block column j of the B rows) of LDS buffer `stage`
     auto read_a = [&](int buf, int stage, int i) {
 #pragma unroll
@@ -229,15 +231,16 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
         if (!FIRST) load_b(nb, koff_b, wB + (cur ^ 1) * B_BYTES);
 #pragma unroll
         for (int i = 0; i < TM - 1; ++i) {
-            read_a((i + 1) & 1, stA, i + 1);
             __builtin_amdgcn_sched_barrier(0);
-            v16i d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i & 1][0], fbv[0][0], vzero, 0, 0, 0);
-            v16i d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i & 1][0], fbv[1][0], vzero, 0, 0, 0);
+            v16i d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[0][0], fbv[0][0], vzero, 0, 0, 0);
+            v16i d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[0][0], fbv[1][0], vzero, 0, 0, 0);
 #pragma unroll
             for (int ks = 1; ks < 4; ++ks) {
-                d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i & 1][ks], fbv[0][ks], d0, 0, 0, 0);
-                d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i & 1][ks], fbv[1][ks], d1, 0, 0, 0);
+                d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[0][ks], fbv[0][ks], d0, 0, 0, 0);
+                d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[0][ks], fbv[1][ks], d1, 0, 0, 0);
             }
+            __builtin_amdgcn_sched_barrier(0);
+            read_a(0, stA, i + 1);   // behind the MFMAs that read the registers, in front of the fold that covers the latency
             __builtin_amdgcn_sched_barrier(0);
             fold(i, d0, d1);
             __builtin_amdgcn_sched_barrier(0);
@@ -255,28 +258,26 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
             __syncthreads();
         }
         load_a(na, koff_a, wA + cur * A_BYTES);
-        constexpr int LB = (TM - 1) & 1;   // buffer that holds the last block row
-        static_assert(LB == 1, "an even number of block rows keeps the A fragment buffers in phase");
-        if (READ_NEXT) read_a(LB ^ 1, stAn, 0);
         __builtin_amdgcn_sched_barrier(0);
-        v16i d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[LB][0], fbv[0][0], vzero, 0, 0, 0);
-        v16i d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[LB][0], fbv[1][0], vzero, 0, 0, 0);
-        d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[LB][1], fbv[0][1], d0, 0, 0, 0);
-        d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[LB][1], fbv[1][1], d1, 0, 0, 0);
+        v16i d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[0][0], fbv[0][0], vzero, 0, 0, 0);
+        v16i d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[0][0], fbv[1][0], vzero, 0, 0, 0);
+        d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[0][1], fbv[0][1], d0, 0, 0, 0);
+        d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[0][1], fbv[1][1], d1, 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
         if (READ_NEXT) {
             read_b(stBn, 0);
             read_b(stBn, 1);
         }
         __builtin_amdgcn_sched_barrier(0);
-        d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[LB][2], fbv[0][2], d0, 0, 0, 0);
-        d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[LB][2], fbv[1][2], d1, 0, 0, 0);
-        d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[LB][3], fbv[0][3], d0, 0, 0, 0);
-        d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[LB][3], fbv[1][3], d1, 0, 0, 0);
+        d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[0][2], fbv[0][2], d0, 0, 0, 0);
+        d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[0][2], fbv[1][2], d1, 0, 0, 0);
+        d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[0][3], fbv[0][3], d0, 0, 0, 0);
+        d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[0][3], fbv[1][3], d1, 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
         if (READ_NEXT) {
             read_b(stBn, 2);
             read_b(stBn, 3);
+            read_a(0, stAn, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
         fold(TM - 1, d0, d1);
