@@ -53,6 +53,8 @@ enum ti8_qflags {
                                butterflies, one bf16 rounding) before the absmax */
     TI8_Q_WS_PINGPONG = 16, /* ti8_quant_row_col_t only: two-part workspace that the calls keep clear for each */
     TI8_Q_WS_SECOND = 32,   /* other, and which part this call works in (see there) */
+    TI8_Q_WS_IS_ZERO = 256, /* ti8_quant_row_col_t only: the caller guarantees that the R + C words of ws are all zero on
+                               entry (it cleared them beside earlier work), so the call needs no clearing launch */
     TI8_Q_TORCH_ROUND = 64, /* ti8_quant_block (128 x 128 groups, q only) and ti8_quant_row (group = 0): the arithmetic of the
                                reference's pure-torch quantisers instead of its Triton kernels' -- scale =
                                reciprocal(max(amax, 1e-4)) * 127, q = clamp(round_half_even(x * scale), -127, 127), stored
@@ -105,6 +107,29 @@ int ti8_version(void);
 const char* ti8_last_error(void);
 /* Name of the GPU architecture the kernels were compiled for ("gfx950"). */
 const char* ti8_arch(void);
+
+/* One-time set-up on the CURRENT device, for callers that want none of it inside their first (timed or
+ * captured) call: raises the dynamic-LDS limit of every kernel that needs more than 64 KiB, looks up the
+ * device's compute-unit count and the address of the library's fixed scratch array.  Optional -- every entry
+ * point does its own part of this on first use -- and idempotent; call it once per device.  It plays the part
+ * of the warm-up call in which the reference's Triton kernels are compiled and autotuned
+ * (triton/block_channel_fwd32.py:12-21).  A device that refuses the persistent GEMM kernel's 160 KiB of LDS
+ * is not an error: ti8_last_error() then says so and the one-workgroup-per-tile kernel serves its shapes. */
+int ti8_init(void);
+
+/* Which GEMM kernel the last ti8_gemm_i8_nt / _multi / _i32 / ti8_linear_fwd_bwd call of THIS thread launched
+ * (the last one when a call launches several): kind | epilogue << 8 | (tile rows / 64) << 16 | (tile columns / 64) << 20.
+ * The kernels of one family give bit-identical results whichever of them runs, so a caller (or a test) that
+ * cares about WHICH one ran -- the persistent kernel is the fast one -- asks here. */
+enum ti8_gemm_kernel {
+    TI8_KERNEL_NONE = 0,
+    TI8_KERNEL_ONE_TILE = 1,          /* one workgroup per output tile */
+    TI8_KERNEL_ONE_TILE_MULTI = 2,    /* the same, several GEMMs in one launch */
+    TI8_KERNEL_PERSISTENT_CHAIN = 3,  /* persistent workgroups, chained block-channel promotion (256 x 256 tiles) */
+    TI8_KERNEL_FEW_ROWS = 4           /* M <= 256: 32 x 32 blocks, K split over the waves */
+};
+#define TI8_KERNEL_KIND(id) ((id) & 0xff)
+int ti8_last_gemm_kernel(void);
 
 /* ---------------------------------------------------------------------------------
  * Per-block absmax quantiser: replaces triton_per_block_quant + per_block_quant_kernel
@@ -295,6 +320,36 @@ typedef struct ti8_gemm_problem {
     float out_scale, post_scale;
 } ti8_gemm_problem;
 int ti8_gemm_i8_nt_multi(const ti8_gemm_problem* problems, int count, int gemm_flags, ti8_stream_t stream);
+
+/* ---------------------------------------------------------------------------------
+ * One whole training step of the layer in ONE call: Y = X W^T, dX = dY W, dW = dY^T X with every operand
+ * quantised on the way, i.e. the launches of
+ *   Y  = fwd_32(X, W)        int8_gemm_pipeline of triton/block_channel_fwd32.py:216-241  /  triton/double-channle_fwd32.py:269-285
+ *   dX = fwd_32(dY, W^T)     the same pipeline on the transposed weight
+ *   dW = bwd_33(dY^T, X^T)   int8_gemm_pipeline of triton/block_channel_bwd33.py:148-172  /  triton/double_channel_bwd33.py:186-201
+ * enqueued back to back from C (the reference pays one Python-side wrapper per quantiser and per GEMM, each with
+ * its own allocations).  Same kernels on the same operands as the separate entry points, so the same bits:
+ *   TI8_SCHEME_BLOCK_CHANNEL   ti8_quant_block_multi(X, dY; q and qT) -> ti8_quant_row_col_t(W) ->
+ *                              ti8_gemm_i8_nt_multi(Y, dX, dW)          (3 launches + W's absmax pass)
+ *   TI8_SCHEME_DOUBLE_CHANNEL  ti8_quant_row_col_t on X, W, dY (TI8_INV_AMAX_DIV_127) -> three
+ *                              ti8_gemm_i8_nt(acc_i32_full = 1, TI8_GEMM_TILED)
+ *   X bf16 [T][K] (ldx), W bf16 [N][K] (ldw), dY bf16 [T][N] (lddy)  ->  Y bf16 [T][N], dX bf16 [T][K], dW bf16 [N][K]
+ *   T, K, N multiples of 128 (zero-pad the tokens: padded rows change no absmax and add nothing to dW).
+ *   workspace: ti8_linear_fwd_bwd_workspace(T, K, N, scheme) bytes of device memory, 256-byte aligned, contents
+ *   undefined before and after (it holds the int8 operands, their transposes, scales and maxima; the call clears
+ *   what it needs cleared itself, so the same buffer serves any sequence of calls in stream order).
+ *   gemm_flags: TI8_GEMM_TILED / TI8_GEMM_LARGE_TILES / TI8_GEMM_ONE_TILE or 0.
+ * Nothing is allocated; the call only enqueues kernels, so it may be captured into a graph. */
+enum ti8_scheme {
+    TI8_SCHEME_BLOCK_CHANNEL = 0,
+    TI8_SCHEME_DOUBLE_CHANNEL = 2
+};
+/* bytes of workspace the call below needs, or -1 for sizes / a scheme it does not take */
+int64_t ti8_linear_fwd_bwd_workspace(int64_t T, int64_t K, int64_t N, int scheme);
+int ti8_linear_fwd_bwd(const void* X, int64_t ldx, const void* W, int64_t ldw, const void* dY, int64_t lddy,
+                       void* Y, int64_t ldy, void* dX, int64_t lddx, void* dW, int64_t lddw,
+                       int64_t T, int64_t K, int64_t N, int scheme, int gemm_flags,
+                       void* workspace, int64_t workspace_bytes, ti8_stream_t stream);
 
 /* Raw int32 accumulators of the same GEMM over the whole K, C int32 [batch][M][N]:
  * the accumulator of int8_gemm_kernel in triton/double-channle_fwd32.py:44,56.

@@ -56,11 +56,44 @@ def bf16_ulp(v):
     return torch.ldexp(torch.ones_like(v, dtype=torch.float32), e - 8)
 
 
-def assert_one_ulp(got, want, what="", slack=2.0 ** -18):
-    """Every element of `got` within one bf16 ulp of `want`, plus `slack` x max|want| for the elements
-    whose K-block terms cancel (re-associating the fp32 sum moves those by a few 2^-24 of the terms,
-    which are of the size of the large elements, not of the result)."""
-    got, want = got.float().cpu(), want.float().cpu()
-    assert got.shape == want.shape, what
-    bad = (got - want).abs() > bf16_ulp(want) + slack * want.abs().max()
-    assert not bool(bad.any()), f"{what}: {int(bad.sum())} of {bad.numel()} elements off by more than one bf16 ulp, first at {bad.nonzero()[0].tolist()}"
+def assert_promoted_close(got, want, mag, K, what=""):
+    """The bar for the default (re-associated) block-channel promotion, per element:
+        |got - want| <= 1 bf16 ulp of want + (K/128 + 4) * 2^-23 * mag
+    with mag >= sum over the K blocks of |term|: what summing the same K/128 fp32 terms in another order, or with an
+    fma, can move an element by.  It scales with the magnitudes that went into THAT element, so a small output next to
+    large ones gets no extra room; a wrong scale, a dropped K tile or a misplaced tile is off by orders of magnitude more."""
+    got, want, mag = got.float().cpu(), want.float().cpu(), mag.float().cpu()
+    assert got.shape == want.shape == mag.shape, what
+    bound = bf16_ulp(want) + (K // 128 + 4) * 2.0 ** -23 * mag
+    bad = (got - want).abs() > bound
+    assert not bool(bad.any()), f"{what}: {int(bad.sum())} of {bad.numel()} elements outside one bf16 ulp, first at {bad.nonzero()[0].tolist()}"
+    assert torch.isfinite(got).all(), what
+
+
+def product_magnitude(a, b, out_scale=1.0):
+    """An upper bound of sum_kb |term_kb| of the quantised product a @ b^T from the bf16 operands themselves
+    (a [..., M, K], b [..., N, K]): a dequantised code differs from its element by at most half a quantisation step,
+    and no step exceeds max|operand| / 127, so sum_k (|a| + max|a|/254) (|b| + max|b|/254) bounds the sum of the
+    magnitudes of all products, hence of the K-block terms.  For `assert_promoted_close` where the int8 operands and
+    scales of the oracle are not at hand."""
+    a, b = a.float().abs(), b.float().abs()
+    a, b = a + a.max() / 254.0, b + b.max() / 254.0
+    return (a @ b.transpose(-1, -2)) * (1.0 + 2.0 ** -10) * out_scale
+
+
+def linear_magnitudes(X, W, dY, hadamard=None):
+    """[(magnitude bound, contraction length)] for Y, dX, dW of the layer (X [..., K], W [N, K], dY [..., N]; tokens
+    flattened), for `assert_promoted_close`.  With ``hadamard=128`` the operands are rotated as the layer rotates
+    them (oracle.hadamard.hadamard128 along the contraction dim, zero-padded to 128) and the result carries 2^-7."""
+    from oracle.hadamard import hadamard128
+    X2, dY2 = X.reshape(-1, X.shape[-1]), dY.reshape(-1, dY.shape[-1])
+    out = []
+    for a, b in ((X2, W), (dY2, W.t()), (dY2.t(), X2.t())):
+        pad = (-a.shape[1]) % 128
+        a = torch.nn.functional.pad(a.contiguous(), (0, pad))
+        b = torch.nn.functional.pad(b.contiguous(), (0, pad))
+        if hadamard == 128:
+            out.append((product_magnitude(hadamard128(a), hadamard128(b), 2.0 ** -7), a.shape[1]))
+        else:
+            out.append((product_magnitude(a, b), a.shape[1]))
+    return out

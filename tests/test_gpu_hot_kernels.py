@@ -13,7 +13,7 @@ magnitude more.  The literal mode (strict) and the int32 path are bit-exact."""
 import pytest
 import torch
 
-from conftest import bf16_ulp, bits_equal, make_gen, randn_bf16, rel_err
+from conftest import assert_promoted_close, bits_equal, make_gen, randn_bf16, rel_err
 from oracle import double_channel_fwd32 as odf
 from oracle import linear as olin
 
@@ -25,15 +25,6 @@ FAST_REL_TOL = 2e-4   # Frobenius norm; the task's bar for bf16 outputs is 1e-2
 def T():
     import triton_int8_amd
     return triton_int8_amd
-
-
-def assert_promoted_close(got, want, mag, K, what=""):
-    got, want, mag = got.float().cpu(), want.float().cpu(), mag.float().cpu()
-    assert got.shape == want.shape, what
-    bound = bf16_ulp(want) + (K // 128 + 4) * 2.0 ** -23 * mag
-    bad = (got - want).abs() > bound
-    assert not bool(bad.any()), f"{what}: {int(bad.sum())} of {bad.numel()} elements outside one bf16 ulp, first at {bad.nonzero()[0].tolist()}"
-    assert torch.isfinite(got).all(), what
 
 
 def run_gemm(T, path, *args, **kw):
@@ -190,6 +181,109 @@ def block_channel_step_pieces(T, X, W, dY, hadamard=None):
             ("dW", dW, dqT[0], ds[0].t(), olin.BLOCK, xqT[0], xs[0].t(), olin.BLOCK, None)]
 
 
+@pytest.mark.parametrize("M,N,K", [(4224, 4096, 512),      # 272 tiles: 16 workgroups walk two tiles; the last tile row hangs over M
+                                   (4224, 4352, 8448),     # the same with 66 K tiles: the factor register refilled at K tile 64
+                                   (2048, 1024, 8448),     # 32 tiles: one tile per workgroup, refill, no next tile
+                                   (384, 640, 256)])       # two K tiles: no inner loop; tiles hang over M and N
+def test_persistent_kernel_wait_variants(T, dev, M, N, K):
+    """The persistent kernel's hand-placed waits, one shape per variant, bit for bit against the one-tile kernel over
+    the whole output (NaN-filled before), and against the oracle on sampled tiles: a workgroup with a next tile waits
+    for that tile's operands and factors behind its own epilogue stores (`stored`, vmcnt(16) / vmcnt(20)); a wave whose
+    tile hangs over the output stored nothing and waits for everything; the last tile of a workgroup has nothing
+    behind it; more than 64 K tiles refill the factor register between two K tiles.  The kernel that ran is read
+    back from the library: a comparison of the one-tile kernel with itself proves nothing."""
+    from triton_int8_amd import ops
+    from triton_int8_amd._lib import KERNEL_ONE_TILE, KERNEL_PERSISTENT_CHAIN, SCALE_BLOCK128, SCALE_ROW
+    g = make_gen(M * 3 + N * 5 + K)
+    A = torch.randint(-127, 128, (1, M, K), generator=g, dtype=torch.int8)
+    B = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+    sa_blk, sb_row, sb_blk = scales(g, 1, M // 128, K // 128), scales(g, N), scales(g, N // 128, K // 128)
+    if K // 128 > 64:   # a factor that only K tile 64 carries: a stale register shows as a large error
+        sa_blk[:, :, 64] *= 37.0
+    Ad, Bd = A.to(dev), B.to(dev)
+
+    def run(persistent, sB, mB):
+        ops.GEMM_PATH, ops.GEMM_PERSISTENT = "large", persistent
+        try:
+            out = torch.full((1, M, N), float("nan"), dtype=torch.bfloat16, device=dev)
+            ops.gemm_i8_nt(Ad, Bd, sa_blk.to(dev), SCALE_BLOCK128, sB.to(dev), mB, out=out)
+            assert T.last_gemm_kernel() == (KERNEL_PERSISTENT_CHAIN if persistent else KERNEL_ONE_TILE)
+            return out
+        finally:
+            ops.GEMM_PATH, ops.GEMM_PERSISTENT = "auto", True
+
+    for sB, mB, oB in ((sb_row, SCALE_ROW, olin.ROW), (sb_blk, SCALE_BLOCK128, olin.BLOCK)):
+        got = run(True, sB, mB)
+        assert torch.equal(got, run(False, sB, mB)) and torch.isfinite(got).all(), (mB,)
+        tile = 128   # sampled 128 x 128 pieces (the shapes are multiples of 128, not of 256)
+        check_sampled_tiles(got[0], Ad[0], sa_blk[0], olin.BLOCK, Bd, sB, oB, g, f"persistent {M}x{N}x{K} B:{oB}", tile=tile)
+
+
+def test_config5_skinny_shapes_at_their_own_size(T, dev):
+    """Config 5's decode shapes as worded: M = 16 and M = 128 tokens at K = N = 4096, seed 4, every scheme, the whole
+    layer step (Y, dX, dW) and the forward-only module against the oracle -- per element for the promoted
+    schemes, bit for bit for the int32 one."""
+    from conftest import linear_magnitudes
+    g = make_gen(4)
+    K = N = 4096
+    W = config_operand(N, K, g, std=0.02)
+    for M in (16, 128):
+        X, dY = config_operand(M, K, g), config_operand(M, N, g, std=1e-3)
+        mags = linear_magnitudes(X, W, dY)
+        for scheme in ("block_channel", "row_block", "double_channel"):
+            got = T.linear_fwd_bwd(X.to(dev), W.to(dev), dY.to(dev), scheme)
+            want = olin.linear_fwd_bwd(X, W, dY, scheme)
+            for name, a, b, (mag, kk) in zip(("Y", "dX", "dW"), got, want, mags):
+                assert a.shape == b.shape and rel_err(a, b) <= FAST_REL_TOL, (scheme, M, name)
+                if scheme == "double_channel":
+                    assert bits_equal(a, b), (scheme, M, name)
+                else:
+                    assert_promoted_close(a, b, mag, kk, f"{scheme} M={M} {name}")
+            lin = T.Int8Linear(K, N, scheme=scheme, device=dev)
+            with torch.no_grad():
+                lin.weight.copy_(W)
+                y = lin(X.to(dev))
+            if scheme == "double_channel":
+                assert bits_equal(y, want[0]), (scheme, M)
+            else:
+                assert_promoted_close(y, want[0], mags[0][0], K, f"{scheme} M={M} forward-only module")
+
+
+def test_one_call_step_matches_the_assembled_step(T, dev):
+    """ti8_linear_fwd_bwd (the whole step enqueued by one library call on caller-provided outputs and workspace) against
+    the same step assembled from the separate entry points: same bits, with fresh and with reused outputs / workspace,
+    on the kernel the shape is meant to take; the outputs start as NaN, the workspace as garbage."""
+    from triton_int8_amd import linear, ops
+    from triton_int8_amd._lib import KERNEL_ONE_TILE, KERNEL_PERSISTENT_CHAIN
+    g = make_gen(31)
+    for (M, K, N) in ((640, 512, 384), (4096, 4096, 4096)):     # the second: 256 tiles of 256 x 256 per GEMM, the persistent kernel
+        X = config_operand(M, K, g, outlier_frac=0.01, outlier_mul=20.0).to(dev)
+        W, dY = config_operand(N, K, g, std=0.02).to(dev), config_operand(M, N, g, std=1e-3).to(dev)
+        for scheme in ("block_channel", "double_channel"):
+            linear.ONE_CALL_STEP = False
+            try:
+                want = T.linear_fwd_bwd(X, W, dY, scheme)
+            finally:
+                linear.ONE_CALL_STEP = True
+            with T._lib.timed_launches() as rec:
+                got = T.linear_fwd_bwd(X, W, dY, scheme)
+            assert list(rec) == ["ti8_linear_fwd_bwd"], list(rec)
+            if scheme == "block_channel" and M >= 4096:
+                assert T.last_gemm_kernel() == KERNEL_PERSISTENT_CHAIN
+            for a, b in zip(got, want):
+                assert torch.equal(a, b), (scheme, M)
+            out = tuple(torch.full_like(t, float("nan")) for t in want)
+            ws = torch.randint(0, 255, (ops.linear_step_workspace_bytes(M, K, N, scheme),), dtype=torch.uint8, device=dev)
+            for _ in range(2):     # the second call finds the first call's leftovers in the workspace
+                res = T.linear_fwd_bwd(X, W, dY, scheme, out=out, workspace=ws)
+                for a, b, o in zip(res, want, out):
+                    assert a.data_ptr() == o.data_ptr() and torch.equal(a, b), (scheme, M)
+    with pytest.raises(ValueError):
+        T.linear_fwd_bwd(X[:100], W, dY[:100], "block_channel", out=out)
+    with pytest.raises(ValueError):
+        T.linear_fwd_bwd(X, W, dY, "row_block", workspace=ws)
+
+
 def test_config2_sampled_tiles_per_element(T, dev):
     """The headline workload (8192 x 4096 x 4096, block-channel, seed 1): Y, dX and dW of the layer
     call, element by element on 12 sampled 256 x 256 tiles each, against the oracle's literal loop
@@ -207,6 +301,7 @@ def test_config2_sampled_tiles_per_element(T, dev):
         check_sampled_tiles(C, Aq, sA, oA, Bq, sB, oB, g, f"config 2 {name}", sc)
     # the layer call returns these very tensors
     Y, dX, dW = T.linear_fwd_bwd(Xd, Wd, dYd, "block_channel")
+    assert T.last_gemm_kernel() == T._lib.KERNEL_PERSISTENT_CHAIN      # the kernel the benchmark is quoted on ran here
     for (name, C, *_), got in zip(pieces, (Y, dX, dW)):
         assert torch.equal(C, got), name
     # quantised operands against the oracle: a band of 256 rows of X, a band of rows of W
@@ -279,6 +374,7 @@ def test_config4_hadamard_block_channel_sampled_tiles(T, dev):
     for name, C, Aq, sA, oA, Bq, sB, oB, sc in pieces:
         check_sampled_tiles(C, Aq, sA, oA, Bq, sB, oB, g, f"config 4 {name}", sc)
     Y, dX, dW = T.linear_fwd_bwd(Xd, Wd, dYd, "block_channel", 128)
+    assert T.last_gemm_kernel() == T._lib.KERNEL_PERSISTENT_CHAIN
     for (name, C, *_), got in zip(pieces, (Y, dX, dW)):
         assert torch.equal(C, got), name
     band = slice(2048, 2304)

@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 import torch
 
-from conftest import assert_one_ulp, bits_equal, make_gen, randn_bf16, rel_err
+from conftest import assert_promoted_close, bits_equal, linear_magnitudes, make_gen, product_magnitude, randn_bf16, rel_err
 from golden_util import bf16, load, t
 from oracle import block_channel_bwd33 as obb
 from oracle import block_channel_fwd32 as obf
@@ -22,10 +22,8 @@ from oracle import tilelang_block_channel_fwd as otf
 
 pytestmark = pytest.mark.gpu
 REL_TOL = 1e-2     # the tolerance the task states for bf16 outputs
-FAST_TOL = 2e-4    # Frobenius bound for the default (re-associated fp32) promotion arithmetic, beside the
-                   # element-wise one-ulp bound (assert_one_ulp); 33 of 393216 elements one bf16 ulp off, the
-                   # large ones of outlier channels, already make 1.2e-4, and the literal arithmetic is no
-                   # closer to the exact sum than the re-associated one (27 against 16 such elements)
+FAST_TOL = 2.0 ** -8   # Frobenius norm: what the per-element bar (assert_promoted_close: one bf16 ulp plus the room of a
+                       # re-associated fp32 sum) implies when every element is a whole ulp off; the per-element bar is the test
 
 
 @pytest.fixture(scope="module")
@@ -122,7 +120,15 @@ def test_gemms_of_a_step_in_one_launch(T, dev):
     X, W, dY = randn_bf16(g, 640, 512).to(dev), randn_bf16(g, 384, 512, std=0.02).to(dev), randn_bf16(g, 640, 384, std=1e-3).to(dev)
     with T._lib.timed_launches() as rec:
         Y, dX, dW = T.linear_fwd_bwd(X, W, dY, "block_channel")
-    assert len(rec["ti8_gemm_i8_nt_multi"]) == 1 and "ti8_gemm_i8_nt" not in rec
+    assert list(rec) == ["ti8_linear_fwd_bwd"]          # the whole step is one library call, which makes that launch
+    T.linear.ONE_CALL_STEP = False
+    try:
+        with T._lib.timed_launches() as rec:
+            Ya, dXa, dWa = T.linear_fwd_bwd(X, W, dY, "block_channel")
+    finally:
+        T.linear.ONE_CALL_STEP = True
+    assert len(rec["ti8_gemm_i8_nt_multi"]) == 1 and "ti8_gemm_i8_nt" not in rec and "ti8_linear_fwd_bwd" not in rec
+    assert torch.equal(Y, Ya) and torch.equal(dX, dXa) and torch.equal(dW, dWa)
     Y0, saved = T.linear.linear_forward(X, W, "block_channel")
     dX0, dW0 = T.linear.linear_backward(dY, X, W, "block_channel", None, saved)
     assert torch.equal(Y, Y0) and torch.equal(dX, dX0) and torch.equal(dW, dW0)
@@ -160,7 +166,7 @@ def test_persistent_workgroups_match_one_tile_kernel(T, dev, M, N, K, batch):
     and against the oracle per element: tiles that hang over M and N, batches, 2 to 256 K tiles (the factor register refilled every 64), fewer tiles than CUs and
     several tiles per workgroup, every scale layout, the extra output factor."""
     from triton_int8_amd import ops
-    from triton_int8_amd._lib import COMBINE_MUL_PROD, SCALE_BLOCK128, SCALE_ROW
+    from triton_int8_amd._lib import COMBINE_MUL_PROD, KERNEL_ONE_TILE, KERNEL_PERSISTENT_CHAIN, SCALE_BLOCK128, SCALE_ROW
     g = make_gen(M + N + K + batch)
     A = torch.randint(-127, 128, (batch, M, K), generator=g, dtype=torch.int8)
     B = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
@@ -176,6 +182,9 @@ def test_persistent_workgroups_match_one_tile_kernel(T, dev, M, N, K, batch):
             with T._lib.timed_launches() as rec:
                 out = ops.gemm_i8_nt(*args, **kw)
             assert list(rec) == ["ti8_gemm_i8_nt"]
+            # which kernel ran is read back from the library: the two give the same bits by design, so only this
+            # tells a comparison of the two from a comparison of one with itself
+            assert T.last_gemm_kernel() == (KERNEL_PERSISTENT_CHAIN if persistent else KERNEL_ONE_TILE)
             return out
         finally:
             ops.GEMM_PATH, ops.GEMM_PERSISTENT = "auto", True
@@ -189,10 +198,10 @@ def test_persistent_workgroups_match_one_tile_kernel(T, dev, M, N, K, batch):
         got = run(True, *args, **kw)
         assert torch.equal(got, run(False, *args, **kw)), (mA, mB, kw)
         for b in (0, batch - 1):   # the oracle on the first and the last batch
-            want = olin.gemm_scaled(A[b], sA[b], oA, Bq[b] if Bq.dim() == 3 else Bq, sB[b] if sB.dim() == 3 else sB, oB,
-                                    out_scale=kw.get("out_scale"))
+            want, mag = olin.gemm_scaled(A[b], sA[b], oA, Bq[b] if Bq.dim() == 3 else Bq, sB[b] if sB.dim() == 3 else sB, oB,
+                                         out_scale=kw.get("out_scale"), with_magnitude=True)
             assert rel_err(got[b], want) <= FAST_TOL
-            assert_one_ulp(got[b], want, f"persistent {M}x{N}x{K} batch {b} modes {mA}/{mB}")
+            assert_promoted_close(got[b], want, mag, K, f"persistent {M}x{N}x{K} batch {b} modes {mA}/{mB}")
 
 
 def test_block_quant_of_several_operands_in_one_launch(T, dev):
@@ -446,7 +455,7 @@ def test_entry_points_match_oracle(T, dev, module, fn, oracle_fn, three_d, gemm_
     Co = oracle_fn(a, b)
     assert C.dtype == torch.bfloat16 and C.shape == Co.shape
     assert rel_err(C, Co) <= FAST_TOL
-    assert_one_ulp(C, Co, f"{module}.{fn}")
+    assert_promoted_close(C, Co, product_magnitude(a, b), 2048, f"{module}.{fn}")
     if module.startswith("double_channel"):
         assert bits_equal(C, Co)          # integer accumulation + literal epilogue: exact
     ref = torch.matmul(a.float(), b.float().transpose(-1, -2))
@@ -520,7 +529,7 @@ def test_bwd33_on_transposed_views(T, dev, gemm_path):
     bt = randn_bf16(g, 1, 1024, 384).transpose(1, 2)
     C = T.block_channel_bwd33.bwd_33(at.to(dev), bt.to(dev))
     assert rel_err(C, obb.bwd_33(at, bt)) <= FAST_TOL
-    assert_one_ulp(C, obb.bwd_33(at, bt))
+    assert_promoted_close(C, obb.bwd_33(at, bt), product_magnitude(at, bt), 1024)
 
 
 @pytest.mark.parametrize("scheme,h", [("block_channel", None), ("row_block", None), ("double_channel", None),
@@ -533,11 +542,13 @@ def test_linear_fwd_bwd(T, dev, scheme, h, gemm_path):
     W, dY = randn_bf16(g, N, 1024, std=0.02), randn_bf16(g, 2, 256, N, std=1e-3)
     Y, dX, dW = T.linear_fwd_bwd(X.to(dev), W.to(dev), dY.to(dev), scheme, h)
     Yo, dXo, dWo = olin.linear_fwd_bwd(X, W, dY, scheme, h)
-    for got, want in ((Y, Yo), (dX, dXo), (dW, dWo)):
+    mags = linear_magnitudes(X, W, dY, h if h == 128 else None)
+    for got, want, (mag, kk) in zip((Y, dX, dW), (Yo, dXo, dWo), mags):
         assert got.shape == want.shape and rel_err(got, want) <= FAST_TOL
-        assert_one_ulp(got, want, f"{scheme} hadamard={h}")
         if scheme == "double_channel":
             assert bits_equal(got, want)
+        else:
+            assert_promoted_close(got, want, mag.reshape(want.shape), kk, f"{scheme} hadamard={h}")
     for got, ref in ((Y, X.float() @ W.float().t()), (dX, dY.float() @ W.float()),
                      (dW, dY.float().reshape(-1, N).t() @ X.float().reshape(-1, 1024))):
         # sanity only: with x20 outlier channels int8 noise exceeds the reference's 1e-3 bar,
@@ -587,11 +598,12 @@ def test_skinny_and_ragged_token_counts(T, dev, tokens, gemm_path):
     for scheme in ("block_channel", "row_block", "double_channel"):
         got = T.linear_fwd_bwd(X.to(dev), W.to(dev), dY.to(dev), scheme)
         want = olin.linear_fwd_bwd(X, W, dY, scheme)
-        for a, b in zip(got, want):
+        for a, b, (mag, kk) in zip(got, want, linear_magnitudes(X, W, dY)):
             assert a.shape == b.shape and rel_err(a, b) <= FAST_TOL
-            assert_one_ulp(a, b, f"{scheme} {tokens} tokens")
             if scheme == "double_channel":
                 assert bits_equal(a, b)
+            else:
+                assert_promoted_close(a, b, mag, kk, f"{scheme} {tokens} tokens")
 
 
 @pytest.mark.parametrize("tokens,scheme,n_out", [(256, "block_channel", 256), (16, "block_channel", 256), (384, "double_channel", 256),
@@ -645,9 +657,10 @@ def test_decoder_layer_step_matches_bf16_twin(T, dev):
     for name in names:
         c, mod = seen[name], getattr(lay, name)
         Yo, dXo, dWo = olin.linear_fwd_bwd(c["x"].cpu(), mod.weight.detach().cpu(), c["dy"].cpu(), "block_channel")
-        for what, got, want in (("Y", c["y"], Yo), ("dX", c["dx"], dXo), ("dW", mod.weight.grad, dWo)):
+        mags = linear_magnitudes(c["x"].cpu(), mod.weight.detach().cpu(), c["dy"].cpu())
+        for (what, got, want), (mag, kk) in zip((("Y", c["y"], Yo), ("dX", c["dx"], dXo), ("dW", mod.weight.grad, dWo)), mags):
             assert rel_err(got, want) <= FAST_TOL, f"{name} {what}"
-            assert_one_ulp(got, want, f"{name} {what}")
+            assert_promoted_close(got, want, mag.reshape(want.shape), kk, f"{name} {what}")
     cos = lambda a, b: float(torch.nn.functional.cosine_similarity(a.float().flatten(), b.float().flatten(), dim=0))
     assert cos(outs[0][0], outs[1][0]) > 0.999
     assert abs(outs[0][1] - outs[1][1]) / outs[0][1] < 2e-2
@@ -787,9 +800,12 @@ def test_golden_vectors_on_gpu(T, dev, gemm_path):
     for scheme, h in (("block_channel", None), ("row_block", None), ("double_channel", None), ("block_channel", 128)):
         tag = scheme + ("_h128" if h else "")
         Y, dX, dW = T.linear_fwd_bwd(X, W, dY, scheme, h)
-        for got, key in ((Y, "_Y"), (dX, "_dX"), (dW, "_dW")):
+        for (got, key), (mag, kk) in zip(((Y, "_Y"), (dX, "_dX"), (dW, "_dW")), linear_magnitudes(X.cpu(), W.cpu(), dY.cpu(), h)):
             assert rel_err(got, bf16(z[tag + key])) <= FAST_TOL
-            assert_one_ulp(got, bf16(z[tag + key]), tag + key)
+            if scheme == "double_channel":
+                assert bits_equal(got, bf16(z[tag + key]))
+            else:
+                assert_promoted_close(got, bf16(z[tag + key]), mag, kk, tag + key)
 
 
 def test_full_size_properties(T, dev):

@@ -240,16 +240,44 @@ def test_transposed_hadamard_launches(walker, recorded, R, C):
 
 
 @pytest.mark.parametrize("M,K,N", [(1024, 512, 768), (8192, 4096, 4096)])
-def test_one_launch_step_is_in_bounds(walker, recorded, M, K, N):
+def test_one_launch_step_is_in_bounds(walker, recorded, monkeypatch, M, K, N):
     """The three GEMMs of a block-channel step in one launch: each GEMM's accesses stay inside its operands, and the
     launch's workgroups cover every tile of every GEMM exactly once."""
     T, allocs, calls = recorded
+    monkeypatch.setattr(T.linear, "ONE_CALL_STEP", False)    # the step assembled from the separate entry points
     X, W, dY = (allocs.add(torch.empty(s, dtype=torch.bfloat16)) for s in ((M, K), (N, K), (M, N)))
     T.linear_fwd_bwd(X, W, dY, "block_channel")
     names = [c[0] for c in calls]
     assert names.count("ti8_gemm_i8_nt_multi") == 1 and "ti8_gemm_i8_nt" not in names
     name, a = next(c for c in calls if c[0] == "ti8_gemm_i8_nt_multi")
     assert a[1] == 3 and walk(walker, allocs, name, a) > 3
+
+
+@pytest.mark.parametrize("scheme", ["block_channel", "double_channel"])
+@pytest.mark.parametrize("M,K,N", [(1024, 512, 768), (8192, 4096, 4096), (16384, 4096, 14336)])
+def test_one_call_step_workspace(recorded, scheme, M, K, N):
+    """The whole step as one library call: the wrapper hands over the three operands, three outputs and a workspace
+    of the size the library asks for, and that size holds every piece the step carves out of it (int8 copies and
+    transposes of the three operands, their scales, the maxima), each on a 256-byte boundary."""
+    T, allocs, calls = recorded
+    X, W, dY = (allocs.add(torch.empty(s, dtype=torch.bfloat16)) for s in ((M, K), (N, K), (M, N)))
+    Y, dX, dW = T.linear_fwd_bwd(X, W, dY, scheme)
+    assert [c[0] for c in calls] == ["ti8_linear_fwd_bwd"]
+    a = calls[0][1]
+    assert (a[12], a[13], a[14]) == (M, K, N) and (a[1], a[3], a[5], a[7], a[9], a[11]) == (K, K, N, N, K, K)
+    for ptr, elems in ((a[0], M * K), (a[2], N * K), (a[4], M * N), (a[6], M * N), (a[8], M * K), (a[10], N * K)):
+        assert allocs.room(ptr, 2) >= elems
+    ws_ptr, ws_bytes = a[17], a[18]
+    assert ws_ptr % 256 == 0 and allocs.room(ws_ptr, 1) >= ws_bytes == T.ops.linear_step_workspace_bytes(M, K, N, scheme)
+    int8_bytes = 2 * (M * K + M * N + N * K)                     # q and qT of every operand
+    if scheme == "block_channel":
+        floats = (M // 128) * (K // 128) + (M // 128) * (N // 128) + 2 * (N + K)
+        pieces = 11
+    else:
+        floats = 2 * ((M + K) + (N + K) + (M + N))
+        pieces = 13
+    assert int8_bytes + 4 * floats <= ws_bytes <= int8_bytes + 4 * floats + 256 * pieces
+    assert T._lib.lib().ti8_linear_fwd_bwd_workspace(M + 1, K, N, 0) == -1 and T._lib.lib().ti8_linear_fwd_bwd_workspace(M, K, N, 1) == -1
 
 
 @pytest.mark.parametrize("tiles", [[512, 512, 512], [1, 1, 1], [7, 300, 2], [5], [9, 4]])

@@ -14,6 +14,7 @@ from . import (block_channel_bwd33, block_channel_fwd32, decoder, double_channel
                double_channel_triton_bwd, double_channel_triton_fwd, fused_bwd33, fused_fwd32, graph, latency, linear, ops,
                tilelang_block_channel_bwd, tilelang_block_channel_fwd)
 from ._common import calc_diff
+from ._lib import init, last_gemm_kernel
 from .decoder import DecoderLayer
 from .graph import GraphedStep
 from .linear import Int8Linear, Int8LinearFunction, linear_fwd_bwd

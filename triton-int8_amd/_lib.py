@@ -45,17 +45,20 @@ PROTOTYPES = {
                        _i64, _i64, _i64, _i64, _int, _int, _f32, _f32, _int, _vp],
     "ti8_gemm_i8_nt_multi": [ctypes.POINTER(GemmProblem), _int, _int, _vp],
     "ti8_gemm_i8_nt_i32": [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp],
+    "ti8_linear_fwd_bwd": [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp, _i64, _vp],
     "ti8_probe_mfma": [_vp, _i64, _vp, _int, _int, _int, _int, _vp],
 }
-EXPORTS = ["ti8_version", "ti8_last_error", "ti8_arch"] + list(PROTOTYPES)
+EXPORTS = ["ti8_version", "ti8_last_error", "ti8_arch", "ti8_init", "ti8_last_gemm_kernel", "ti8_linear_fwd_bwd_workspace"] + list(PROTOTYPES)
 
 # enums of include/ti8.h
-Q_CLAMP, Q_EPS_ADD, Q_SCALE_BF16, Q_HAD128, Q_WS_PINGPONG, Q_WS_SECOND, Q_TORCH_ROUND, Q_TORCH_BF16 = 1, 2, 4, 8, 16, 32, 64, 128
+Q_CLAMP, Q_EPS_ADD, Q_SCALE_BF16, Q_HAD128, Q_WS_PINGPONG, Q_WS_SECOND, Q_TORCH_ROUND, Q_TORCH_BF16, Q_WS_IS_ZERO = 1, 2, 4, 8, 16, 32, 64, 128, 256
 INV_RCP_OF_SCALE, INV_AMAX_DIV_127, INV_AMAX_MUL_RCP127, INV_MULTIPLIER = 0, 1, 2, 3
 SCALE_ROW, SCALE_BLOCK128, SCALE_ROW_K128, SCALE_BLOCK_K256 = 0, 1, 2, 3
 COMBINE_MUL_MUL, COMBINE_MUL_PROD, COMBINE_DIV_PROD = 0, 1, 2
 GEMM_STRICT, GEMM_TILED, GEMM_SKINNY, GEMM_LARGE_TILES, GEMM_ONE_TILE = 1, 2, 4, 8, 16
 NOALLOC_MAX_ROWS_PLUS_COLS = 65536
+SCHEME_BLOCK_CHANNEL, SCHEME_DOUBLE_CHANNEL = 0, 2
+KERNEL_NONE, KERNEL_ONE_TILE, KERNEL_ONE_TILE_MULTI, KERNEL_PERSISTENT_CHAIN, KERNEL_FEW_ROWS = 0, 1, 2, 3, 4
 
 _lib = None
 
@@ -80,6 +83,12 @@ def lib():
         l.ti8_version.restype = _int
         l.ti8_last_error.restype = ctypes.c_char_p
         l.ti8_arch.restype = ctypes.c_char_p
+        l.ti8_init.restype = _int
+        l.ti8_init.argtypes = []
+        l.ti8_last_gemm_kernel.restype = _int
+        l.ti8_last_gemm_kernel.argtypes = []
+        l.ti8_linear_fwd_bwd_workspace.restype = _i64
+        l.ti8_linear_fwd_bwd_workspace.argtypes = [_i64, _i64, _i64, _int]
         for name, args in PROTOTYPES.items():
             fn = getattr(l, name)
             fn.argtypes = args
@@ -124,3 +133,21 @@ def call(name, *args):
         rec.setdefault(name, []).append((a, b))
     if rc != 0:
         raise Ti8Error(name, rc, l.ti8_last_error().decode())
+
+
+def init():
+    """One-time set-up of the library on the current device (``ti8_init``): kernel attributes, device
+    properties, the fixed scratch array.  Optional; a caller that times or captures its first call
+    runs it beforehand.  Returns the library's note (empty, or that the persistent GEMM kernel is not
+    available on this device)."""
+    l = lib()
+    rc = l.ti8_init()
+    if rc != 0:
+        raise Ti8Error("ti8_init", rc, l.ti8_last_error().decode())
+    return l.ti8_last_error().decode()
+
+
+def last_gemm_kernel():
+    """Kind of the GEMM kernel that the last GEMM entry point called from this thread launched
+    (``KERNEL_*``): kernels of one family give the same bits, so this is how a caller tells which ran."""
+    return lib().ti8_last_gemm_kernel() & 0xff

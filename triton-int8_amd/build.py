@@ -10,7 +10,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libti8.so")
-SOURCES = ["api.hip", "quant.hip", "fwht.hip", "gemm.hip", "gemm_chain.hip", "gemm_skinny.hip", "probe.hip"]
+SOURCES = ["api.hip", "quant.hip", "fwht.hip", "gemm.hip", "gemm_chain.hip", "gemm_skinny.hip", "step.hip", "probe.hip"]
 
 # -ffp-contract=off: x*scale+0.5 must round twice (bit-exact quantisation); kernels
 #   that want an fma ask for one explicitly.

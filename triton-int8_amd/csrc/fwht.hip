@@ -248,20 +248,39 @@ __global__ __launch_bounds__(256) void transpose_bf16_kernel(const uint16_t* __r
 
 using namespace ti8;
 
+constexpr int FWHT_LDS_LIMIT = 136 * 1024;
+
+template <int NT, int W>
+static int prepare_fwht_t() {
+    static OncePerDevice once;
+    const hipError_t e = raise_lds_limit(once, reinterpret_cast<const void*>(fwht_t_kernel<NT, W>), FWHT_LDS_LIMIT);
+    if (e != hipSuccess) return fail(TI8_ERR_HIP, "ti8_fwht_t: cannot raise the LDS limit: %s", hipGetErrorString(e));
+    return TI8_OK;
+}
+
+static int prepare_fwht() {
+    static OncePerDevice once;
+    const hipError_t e = raise_lds_limit(once, reinterpret_cast<const void*>(fwht_kernel<1024>), FWHT_LDS_LIMIT);
+    if (e != hipSuccess) return fail(TI8_ERR_HIP, "ti8_fwht: cannot raise the LDS limit: %s", hipGetErrorString(e));
+    return TI8_OK;
+}
+
+namespace ti8 {
+int init_fwht_kernels() {
+    if (int e = prepare_fwht()) return e;
+    if (int e = prepare_fwht_t<1024, 8>()) return e;
+    if (int e = prepare_fwht_t<1024, 4>()) return e;
+    if (int e = prepare_fwht_t<1024, 2>()) return e;
+    return prepare_fwht_t<1024, 1>();
+}
+}  // namespace ti8
+
 template <int NT, int W>
 static int launch_fwht_t(const void* x, int64_t ldx, void* y, int64_t ldy, int64_t R, int64_t C, int logn, float scale, hipStream_t st) {
     const size_t shmem = (size_t)W * idx::fwht_lds_words(R) * sizeof(float);
     auto kern = fwht_t_kernel<NT, W>;
-    if (shmem > 64 * 1024) {
-        static thread_local int attr_dev = -1;
-        int dev = 0;
-        (void)hipGetDevice(&dev);
-        if (attr_dev != dev) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 136 * 1024);
-            if (e != hipSuccess) return fail(TI8_ERR_HIP, "ti8_fwht_t: cannot raise the LDS limit: %s", hipGetErrorString(e));
-            attr_dev = dev;
-        }
-    }
+    if (shmem > 64 * 1024)
+        if (int e = prepare_fwht_t<NT, W>()) return e;
     const int64_t nblocks = C / W;
     hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(NT), shmem, st, static_cast<const uint16_t*>(x), ldx,
                        static_cast<uint16_t*>(y), ldy, (int)R, logn, nblocks, scale);
@@ -309,14 +328,7 @@ extern "C" int ti8_fwht(const void* x, int64_t ldx, void* y, int64_t ldy, int64_
     int logn = 0;
     while ((1LL << logn) < n) ++logn;
     const size_t shmem = (size_t)idx::fwht_lds_words(L) * sizeof(float);
-    static thread_local int attr_set_for = -1;
-    int dev = 0;
-    (void)hipGetDevice(&dev);
-    if (attr_set_for != dev) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fwht_kernel<1024>), hipFuncAttributeMaxDynamicSharedMemorySize, 136 * 1024);
-        if (e != hipSuccess) return fail(TI8_ERR_HIP, "ti8_fwht: cannot raise the LDS limit: %s", hipGetErrorString(e));
-        attr_set_for = dev;
-    }
+    if (int e = prepare_fwht()) return e;
     if (idx::fwht_threads(L) == 1024)
         hipLaunchKernelGGL(fwht_kernel<1024>, dim3((unsigned)nblocks), dim3(1024), shmem, static_cast<hipStream_t>(stream),
                            static_cast<const uint16_t*>(x), ldx, static_cast<uint16_t*>(y), ldy, (int)cols, logn, (int)L, scale);

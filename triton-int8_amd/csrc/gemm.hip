@@ -552,6 +552,22 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_multi_kernel(const GemmM
     gemm_i8_tile<BM, BN, WM, WN, EPI>(m.g[i], (int)blockIdx.x - m.first[i], 0);
 }
 
+constexpr size_t tile_lds_bytes(int bm, int bn) { return 2 * (size_t)(bm + bn) * 128; }
+
+// Per-device set-up of one kernel instance (MULTI: the several-GEMMs form): its dynamic LDS limit where the
+// double-buffered operand tiles exceed the 64 KiB a kernel gets by default.
+template <int BM, int BN, int WM, int WN, int EPI, bool MULTI>
+static int prepare_kernel() {
+    constexpr size_t shmem = tile_lds_bytes(BM, BN);
+    if (shmem <= 64 * 1024) return TI8_OK;
+    static OncePerDevice once;
+    const void* kern = MULTI ? reinterpret_cast<const void*>(gemm_i8_multi_kernel<BM, BN, WM, WN, EPI>)
+                             : reinterpret_cast<const void*>(gemm_i8_kernel<BM, BN, WM, WN, EPI>);
+    const hipError_t e = raise_lds_limit(once, kern, (int)shmem);
+    if (e != hipSuccess) return fail(TI8_ERR_HIP, "gemm: cannot raise the LDS limit to %zu: %s", shmem, hipGetErrorString(e));
+    return TI8_OK;
+}
+
 template <int BM, int BN, int WM, int WN, int EPI>
 static int launch_multi(GemmMulti& m, hipStream_t st) {
     int total = 0;
@@ -563,17 +579,9 @@ static int launch_multi(GemmMulti& m, hipStream_t st) {
     }
     for (int i = m.count; i <= GEMM_MULTI_MAX; ++i) m.first[i] = total;
     for (int i = m.count; i < GEMM_MULTI_MAX; ++i) m.g[i] = m.g[0];
-    const size_t shmem = 2 * (size_t)(BM + BN) * 128;
-    static thread_local int attr_dev = -1;
-    int dev = 0;
-    (void)hipGetDevice(&dev);
-    auto kern = gemm_i8_multi_kernel<BM, BN, WM, WN, EPI>;
-    if (shmem > 64 * 1024 && attr_dev != dev) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
-        if (e != hipSuccess) return fail(TI8_ERR_HIP, "gemm: cannot raise the LDS limit to %zu: %s", shmem, hipGetErrorString(e));
-        attr_dev = dev;
-    }
-    hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(64 * WM * WN), shmem, st, m);
+    if (int e = prepare_kernel<BM, BN, WM, WN, EPI, true>()) return e;
+    hipLaunchKernelGGL((gemm_i8_multi_kernel<BM, BN, WM, WN, EPI>), dim3((unsigned)total), dim3(64 * WM * WN), tile_lds_bytes(BM, BN), st, m);
+    note_gemm_kernel(TI8_KERNEL_ONE_TILE_MULTI, BM, BN, EPI);
     return check_launch("ti8_gemm_i8_nt_multi");
 }
 
@@ -582,18 +590,10 @@ static int launch(const GemmArgs& a0, int64_t batch, hipStream_t st) {
     GemmArgs a = a0;
     a.tiles_m = (a.M + BM - 1) / BM;
     a.tiles_n = (a.N + BN - 1) / BN;
-    const size_t shmem = 2 * (size_t)(BM + BN) * 128;
-    static thread_local int attr_dev = -1;
-    int dev = 0;
-    (void)hipGetDevice(&dev);
-    auto kern = gemm_i8_kernel<BM, BN, WM, WN, EPI>;
-    if (shmem > 64 * 1024 && attr_dev != dev) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
-        if (e != hipSuccess) return fail(TI8_ERR_HIP, "gemm: cannot raise the LDS limit to %zu: %s", shmem, hipGetErrorString(e));
-        attr_dev = dev;
-    }
+    if (int e = prepare_kernel<BM, BN, WM, WN, EPI, false>()) return e;
     dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)batch), block(64 * WM * WN);
-    hipLaunchKernelGGL(kern, grid, block, shmem, st, a);
+    hipLaunchKernelGGL((gemm_i8_kernel<BM, BN, WM, WN, EPI>), grid, block, tile_lds_bytes(BM, BN), st, a);
+    note_gemm_kernel(TI8_KERNEL_ONE_TILE, BM, BN, EPI);
     return check_launch("ti8_gemm_i8_nt");
 }
 
@@ -652,15 +652,23 @@ static int prepare_gemm(const char* fn, const ti8_gemm_problem& p, int gemm_flag
     return TI8_OK;
 }
 
-static int device_cu_count() {
-    static int num_cu = 0;
-    if (num_cu == 0) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        (void)hipGetDevice(&dev);
-        num_cu = (hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
-    }
-    return num_cu;
+// every kernel instance that the launchers below can select, for ti8_init()
+int init_gemm_kernels() {
+#define TI8_GEMM_CASE(BM, BN, WM, WN, EPI) \
+    if (int e = prepare_kernel<BM, BN, WM, WN, EPI, false>()) return e
+    TI8_GEMM_CASE(256, 256, 2, 4, EPI_ROWS);
+    TI8_GEMM_CASE(256, 256, 2, 4, EPI_I32);
+    TI8_GEMM_CASE(256, 128, 4, 2, EPI_PROMOTE_LANE);
+    TI8_GEMM_CASE(256, 256, 2, 4, EPI_PROMOTE_CHAIN);
+    TI8_GEMM_CASE(256, 128, 4, 2, EPI_PROMOTE);
+#undef TI8_GEMM_CASE
+#define TI8_GEMM_CASE(BM, BN, WM, WN, EPI) \
+    if (int e = prepare_kernel<BM, BN, WM, WN, EPI, true>()) return e
+    TI8_GEMM_CASE(256, 256, 2, 4, EPI_ROWS);
+    TI8_GEMM_CASE(256, 256, 2, 4, EPI_PROMOTE_CHAIN);
+    TI8_GEMM_CASE(256, 128, 4, 2, EPI_PROMOTE);
+#undef TI8_GEMM_CASE
+    return TI8_OK;
 }
 
 // The chained promotion on persistent workgroups where its limits allow (gemm_chain.hip); CHAIN_UNAVAILABLE otherwise

@@ -29,16 +29,25 @@ constexpr int WCOLS = TN * 32;
 constexpr int SLAB_ROWS = 16;                                   // tile rows per pass through the slab
 constexpr int SLAB_BYTES = NW * SLAB_ROWS * WCOLS * 4;          // 32 KiB
 constexpr int LDS_BYTES = 2 * (A_BYTES + B_BYTES) + SLAB_BYTES; // 160 KiB
-// a wave whose tile lies inside the output stores it with 32 instructions (16 x 8 rows, two 8-byte stores each);
-// s_waitcnt vmcnt(32) lgkmcnt(0): vector-memory operations complete in issue order, so everything issued
-// before those stores has completed when at most 32 are outstanding
-constexpr int EPILOGUE_STORES = TM * 2 * 2 * 2;
-constexpr int WAIT_ALL_BUT_STORES = ((EPILOGUE_STORES >> 4) << 14) | (EPILOGUE_STORES & 15) | 0x70;
-// vmcnt(B_INSTR) / vmcnt(B_INSTR + 32) with the other counters left alone
-constexpr int WAIT_FACTORS = B_INSTR | 0x70 | 0xF00;
-constexpr int WAIT_FACTORS_BEHIND_STORES = (((B_INSTR + EPILOGUE_STORES) >> 4) << 14) | ((B_INSTR + EPILOGUE_STORES) & 15) | 0x70 | 0xF00;
-static_assert(B_INSTR == 4 && WAIT_FACTORS == 0xF74 && WAIT_FACTORS_BEHIND_STORES == 0x8F74, "s_waitcnt encoding");
-static_assert(EPILOGUE_STORES == 32 && WAIT_ALL_BUT_STORES == 0x8070, "s_waitcnt encoding: vmcnt[3:0] | expcnt << 4 | lgkmcnt << 8 | vmcnt[5:4] << 14");
+// Epilogue stores and the waits that count them.  A wave whose tile lies inside the output stores it row by row:
+// every lane writes its 8 bf16 columns of a row with ONE 16-byte store, 8 rows (RPI) per instruction, so a wave
+// issues exactly ROWS_PER_WAVE / RPI of them.  Rows of C are ldc apart, so no compiler can merge two of them, and a
+// store that a compiler split in two would only make the waits below stronger: the count is a LOWER bound on the
+// vector-memory operations a wave issues in its epilogue, which is what `s_waitcnt vmcnt(count)` needs to be safe
+// (vector-memory operations complete in issue order: once at most `count` are outstanding, everything issued before
+// the stores has completed).  The store loop in `store_tile` runs over the same constants.
+constexpr int RPI = 64 / (WCOLS / 8);                  // rows per store instruction: 64 lanes, 8 columns per lane
+constexpr int STORE_PASSES = TM * 2;                  // slab passes per tile (16 rows each)
+constexpr int STORES_PER_PASS = SLAB_ROWS / RPI;      // store instructions per pass
+constexpr int EPILOGUE_STORES = STORE_PASSES * STORES_PER_PASS;
+constexpr int waitcnt_vm(int vm, int other) { return ((vm >> 4) << 14) | (vm & 15) | other; }   // vmcnt[3:0] | expcnt << 4 | lgkmcnt << 8 | vmcnt[5:4] << 14
+// vmcnt(EPILOGUE_STORES) lgkmcnt(0)
+constexpr int WAIT_ALL_BUT_STORES = waitcnt_vm(EPILOGUE_STORES, 0x70);
+// vmcnt(B_INSTR) / vmcnt(B_INSTR + EPILOGUE_STORES) with the other counters left alone
+constexpr int WAIT_FACTORS = waitcnt_vm(B_INSTR, 0x70 | 0xF00);
+constexpr int WAIT_FACTORS_BEHIND_STORES = waitcnt_vm(B_INSTR + EPILOGUE_STORES, 0x70 | 0xF00);
+static_assert(RPI == 8 && STORES_PER_PASS == 2 && EPILOGUE_STORES == 16 && EPILOGUE_STORES * RPI == TM * 32, "one 16-byte store per lane and row of the 128-row wave tile");
+static_assert(B_INSTR == 4 && WAIT_FACTORS == 0xF74 && WAIT_FACTORS_BEHIND_STORES == 0x4F74 && WAIT_ALL_BUT_STORES == 0x4070, "s_waitcnt encoding");
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
@@ -288,7 +297,6 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
     // Slab word (row, col) of a wave sits at row * 64 + (col ^ 4 (row & 1)): the two rows that 16 lanes read
     // together then fall in different banks.  A wave's tile lies inside one 128-row and one 128-column block and
     // M, N are multiples of 128, so a wave either stores its whole tile or nothing.
-    constexpr int RPI = 64 / (WCOLS / 8);   // rows per store instruction
     auto epilogue = [&](const Tile& t, const float (&coln)[4]) {
         const GemmArgs& g = m.g[t.gi];
         if (t.m0 + wm * TM * 32 >= g.M || t.n0 + wn * WCOLS >= g.N) return false;
@@ -312,19 +320,19 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
             constexpr bool MROW = decltype(mrow_tag)::value;
             constexpr bool MCOL = decltype(mcol_tag)::value;
             int64_t off = c_off;
-            float rm_all[MROW ? TM * 4 : 1];
+            float rm_all[MROW ? EPILOGUE_STORES : 1];   // one row scale per store instruction
             if (MROW) {   // every row scale of the tile before the first store (loads and stores share one in-order counter)
 #pragma unroll
-                for (int q = 0; q < TM * 4; ++q) rm_all[q] = prow0[(int64_t)(q * RPI) * g.sa.rs];
+                for (int q = 0; q < EPILOGUE_STORES; ++q) rm_all[q] = prow0[(int64_t)(q * RPI) * g.sa.rs];
                 if (divide) {
 #pragma unroll
-                    for (int q = 0; q < TM * 4; ++q) rm_all[q] = 1.0f / rm_all[q];
+                    for (int q = 0; q < EPILOGUE_STORES; ++q) rm_all[q] = 1.0f / rm_all[q];
                 }
             }
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int h = 0; h < 2; ++h) {   // rows 16 h .. 16 h + 15 of block row i: accumulator registers 8 h .. 8 h + 7
+                for (int h = 0; h < STORE_PASSES / TM; ++h) {   // rows 16 h .. 16 h + 15 of block row i: accumulator registers 8 h .. 8 h + 7
 #pragma unroll
                     for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -336,30 +344,30 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_chain_kernel(const GemmMulti 
                     __builtin_amdgcn_wave_barrier();
                     // the read-back is written out: before an LDS read that it knows, the compiler waits for the operand loads
                     // in flight (they write LDS too), i.e. for the next tile's K tile 1 issued a moment ago
-                    u32x4 w[2][2];
+                    u32x4 w[STORES_PER_PASS][2];
 #pragma unroll
-                    for (int k = 0; k < 2; ++k) {
+                    for (int k = 0; k < STORES_PER_PASS; ++k) {
                         const int rr = rb_row + k * RPI;
                         w[k][0] = lds_read_uncounted(slab + idx::epi_chain_slab_word(rr, rb_col));
                         w[k][1] = lds_read_uncounted(slab + idx::epi_chain_slab_word(rr, rb_col + 4));
                     }
                     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
 #pragma unroll
-                    for (int k = 0; k < 2; ++k) asm volatile("" : "+v"(w[k][0]), "+v"(w[k][1]));
+                    for (int k = 0; k < STORES_PER_PASS; ++k) asm volatile("" : "+v"(w[k][0]), "+v"(w[k][1]));
 #pragma unroll
-                    for (int k = 0; k < 2; ++k, off += c_step) {
+                    for (int k = 0; k < STORES_PER_PASS; ++k, off += c_step) {
                         const uint32_t wb[8] = {w[k][0].x, w[k][0].y, w[k][0].z, w[k][0].w, w[k][1].x, w[k][1].y, w[k][1].z, w[k][1].w};
                         float v[8];
 #pragma unroll
                         for (int c = 0; c < 8; ++c) {
                             v[c] = __uint_as_float(wb[c]);
-                            if (MROW) v[c] = v[c] * rm_all[MROW ? (i * 2 + h) * 2 + k : 0];
+                            if (MROW) v[c] = v[c] * rm_all[MROW ? (i * (STORE_PASSES / TM) + h) * STORES_PER_PASS + k : 0];
                             if (MCOL) v[c] = v[c] * cm[c];
                             if (EXTRA) v[c] = v[c] * g.out_scale;
                         }
-                        uint16_t* dst = reinterpret_cast<uint16_t*>(g.C) + off;
-                        *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
-                        *reinterpret_cast<uint2*>(dst + 4) = make_uint2(pack_bf16x2(v[4], v[5]), pack_bf16x2(v[6], v[7]));
+                        // the ONE store of this (pass, k): EPILOGUE_STORES counts these
+                        *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(g.C) + off) =
+                            make_uint4(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]), pack_bf16x2(v[4], v[5]), pack_bf16x2(v[6], v[7]));
                     }
                     __builtin_amdgcn_s_waitcnt(0xc07f);
                     __builtin_amdgcn_wave_barrier();
@@ -500,22 +508,30 @@ bool chain_persistent_supported(const GemmMulti& m) {
 
 // `m` with tiles_m / tiles_n / first[] filled for 256 x 256 tiles and first[i + 1] - first[i] = tiles of GEMM i times
 // its batch count; one workgroup per CU (fewer when there are fewer tiles)
+// Whether the current device grants the kernel its 160 KiB of LDS (asked once per device).  A refusal is remembered
+// and reported through ti8_last_error() by the call that met it; callers then take the one-tile kernel.
+static bool chain_kernel_available() {
+    static OncePerDevice granted, refused;
+    const uint64_t bit = 1ull << (current_device() & 63);
+    if (refused.done.load(std::memory_order_acquire) & bit) return false;
+    const hipError_t e = raise_lds_limit(granted, reinterpret_cast<const void*>(gemm_i8_chain_kernel), LDS_BYTES);
+    if (e == hipSuccess) return true;
+    refused.done.fetch_or(bit, std::memory_order_release);
+    (void)fail(TI8_OK, "gemm: device %d refuses %d bytes of LDS for the persistent kernel (%s); one workgroup per tile serves its shapes",
+               current_device(), LDS_BYTES, hipGetErrorString(e));
+    return false;
+}
+
+int init_chain_kernel() {
+    (void)chain_kernel_available();
+    return TI8_OK;
+}
+
 int launch_chain_persistent(const GemmMulti& m, int total_tiles, int num_cu, hipStream_t st) {
-    static thread_local int attr_dev = -1;
-    int dev = 0;
-    (void)hipGetDevice(&dev);
-    static thread_local int refused_dev = -1;
-    if (refused_dev == dev) return CHAIN_UNAVAILABLE;
-    if (attr_dev != dev) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_i8_chain_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess) {
-            (void)hipGetLastError();
-            refused_dev = dev;
-            return CHAIN_UNAVAILABLE;
-        }
-        attr_dev = dev;
-    }
+    if (!chain_kernel_available()) return CHAIN_UNAVAILABLE;
     const int grid = total_tiles < num_cu ? total_tiles : num_cu;
     hipLaunchKernelGGL(gemm_i8_chain_kernel, dim3((unsigned)grid), dim3(64 * NW), LDS_BYTES, st, m, total_tiles);
+    note_gemm_kernel(TI8_KERNEL_PERSISTENT_CHAIN, BM, BN, EPI_PROMOTE_CHAIN);
     return check_launch("ti8_gemm_i8_nt");
 }
 

@@ -232,23 +232,25 @@ bool skinny_supported(const GemmArgs& a) {
     return (int64_t)(a.N / 32) * (a.M / 32) <= 0x7fffffffLL;
 }
 
+constexpr size_t WAVERING_LDS_BYTES = (size_t)4 * WS_STAGES * WS_STAGE_BYTES;
+
+int init_skinny_kernels() {
+    static OncePerDevice once_i32, once_promote;
+    hipError_t e = raise_lds_limit(once_i32, reinterpret_cast<const void*>(gemm_i8_wavering_kernel<true>), (int)WAVERING_LDS_BYTES);
+    if (e == hipSuccess) e = raise_lds_limit(once_promote, reinterpret_cast<const void*>(gemm_i8_wavering_kernel<false>), (int)WAVERING_LDS_BYTES);
+    if (e != hipSuccess) return fail(TI8_ERR_HIP, "gemm: cannot raise the LDS limit to %zu: %s", WAVERING_LDS_BYTES, hipGetErrorString(e));
+    return TI8_OK;
+}
+
 static int launch_wavering(const GemmArgs& a, int64_t batch, bool i32_full, hipStream_t st) {
-    constexpr size_t shmem = (size_t)4 * WS_STAGES * WS_STAGE_BYTES;
-    static thread_local int attr_dev = -1;
-    int dev = 0;
-    (void)hipGetDevice(&dev);
-    if (attr_dev != dev) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_i8_wavering_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
-        if (e == hipSuccess)
-            e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_i8_wavering_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
-        if (e != hipSuccess) return fail(TI8_ERR_HIP, "gemm: cannot raise the LDS limit to %zu: %s", shmem, hipGetErrorString(e));
-        attr_dev = dev;
-    }
+    constexpr size_t shmem = WAVERING_LDS_BYTES;
+    if (int e = init_skinny_kernels()) return e;
     dim3 grid((unsigned)((a.N / 32) * (a.M / 32)), (unsigned)batch), block(256);
     if (i32_full)
         hipLaunchKernelGGL(gemm_i8_wavering_kernel<true>, grid, block, shmem, st, a);
     else
         hipLaunchKernelGGL(gemm_i8_wavering_kernel<false>, grid, block, shmem, st, a);
+    note_gemm_kernel(TI8_KERNEL_FEW_ROWS, 32, 32, i32_full ? EPI_ROWS : EPI_PROMOTE);
     return check_launch("ti8_gemm_i8_nt");
 }
 

@@ -315,12 +315,18 @@ struct QBlockMulti {
     QBlockOperand op[QBLOCK_MULTI_MAX];
     int first[QBLOCK_MULTI_MAX + 1];   // first workgroup of operand i; first[count] = grid size
     int count;
+    unsigned int* clear;               // words that the launch zeroes on the side (thread i of the grid clears word i), or NULL
+    int clear_words;
 };
 
 template <bool WRITE_Q, bool WRITE_QT>
 __global__ __launch_bounds__(256) void quant_block_multi_kernel(const QBlockMulti m, QMode mode) {
     __shared__ float red4[4];
     __shared__ uint32_t tileT[WRITE_QT ? 128 * 33 : 1];
+    {   // the next launch's maxima workspace, cleared here so that no launch exists only to clear it
+        const int64_t w = (int64_t)blockIdx.x * 256 + threadIdx.x;
+        if (w < m.clear_words) m.clear[w] = 0u;
+    }
     int i = 0;
 #pragma unroll
     for (int k = 1; k < QBLOCK_MULTI_MAX; ++k)
@@ -809,6 +815,18 @@ extern "C" int ti8_quant_block(const void* x, int64_t bsx, int64_t ldx, int8_t* 
 }
 
 extern "C" int ti8_quant_block_multi(const ti8_qblock_operand* operands, int count, int qflags, int inv_mode, ti8_stream_t stream) {
+    return ti8::quant_block_multi_and_clear(operands, count, qflags, inv_mode, nullptr, 0, stream);
+}
+
+int ti8::fill_words(unsigned int* p, int64_t words, unsigned int value, hipStream_t st) {
+    if (words <= 0) return TI8_OK;
+    if (!p || words > 0x7fffffffLL) return fail(TI8_ERR_SHAPE, "fill: bad buffer");
+    hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, st, p, (int)words, value);
+    return check_launch("fill");
+}
+
+int ti8::quant_block_multi_and_clear(const ti8_qblock_operand* operands, int count, int qflags, int inv_mode,
+                                     unsigned int* clear, int64_t clear_words, ti8_stream_t stream) {
     const char* fn = "ti8_quant_block_multi";
     QMode mode;
     if (int e = parse_mode(qflags, inv_mode, &mode)) return e;
@@ -832,6 +850,16 @@ extern "C" int ti8_quant_block_multi(const ti8_qblock_operand* operands, int cou
     m.first[QBLOCK_MULTI_MAX] = (int)total;
     m.count = count;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    m.clear = nullptr;
+    m.clear_words = 0;
+    if (clear && clear_words > 0) {
+        if (clear_words <= total * 256) {
+            m.clear = clear;
+            m.clear_words = (int)clear_words;
+        } else if (int e = fill_words(clear, clear_words, 0u, st)) {   // more words than threads: a launch of its own
+            return e;
+        }
+    }
     dim3 grid((unsigned)total), block(256);
     const bool wq = operands[0].q != nullptr, wqt = operands[0].qT != nullptr;
     if (wq && wqt) hipLaunchKernelGGL((quant_block_multi_kernel<true, true>), grid, block, 0, st, m, mode);
@@ -921,9 +949,11 @@ static int quant_row_col_t_impl(const char* fn, const void* x, int64_t ldx, int8
                                 int64_t ldqt, float* s_col, float* ws, int64_t R, int64_t C, int qflags, int inv_mode,
                                 ti8_stream_t stream) {
     const bool pingpong = (qflags & TI8_Q_WS_PINGPONG) != 0, second = (qflags & TI8_Q_WS_SECOND) != 0;
+    const bool is_zero = (qflags & TI8_Q_WS_IS_ZERO) != 0;
     if (second && !pingpong) return fail(TI8_ERR_MODE, "%s: TI8_Q_WS_SECOND needs TI8_Q_WS_PINGPONG", fn);
+    if (is_zero && pingpong) return fail(TI8_ERR_MODE, "%s: TI8_Q_WS_IS_ZERO and TI8_Q_WS_PINGPONG exclude each other", fn);
     QMode mode;
-    if (int e = parse_mode(qflags & ~(TI8_Q_WS_PINGPONG | TI8_Q_WS_SECOND), inv_mode, &mode)) return e;
+    if (int e = parse_mode(qflags & ~(TI8_Q_WS_PINGPONG | TI8_Q_WS_SECOND | TI8_Q_WS_IS_ZERO), inv_mode, &mode)) return e;
     if (qflags & TI8_Q_HAD128) return fail(TI8_ERR_MODE, "%s: the Hadamard rotation is not offered here", fn);
     if (!x || !q || !s_row || !qT || !s_col || !ws) return fail(TI8_ERR_NULL, "%s: x, q, s_row, qT, s_col and ws are required", fn);
     if (R <= 0 || C <= 0 || R % 128 || C % 128 || C > 0x7fffffffLL)
@@ -941,7 +971,7 @@ static int quant_row_col_t_impl(const char* fn, const void* x, int64_t ldx, int8
         ws = second ? ws + R + C : ws;
     }
     unsigned int* wsu = reinterpret_cast<unsigned int*>(ws);
-    if (!pingpong)
+    if (!pingpong && !is_zero)
         hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((R + C + 255) / 256)), dim3(256), 0, st, wsu, (int)(R + C), 0u);
     hipLaunchKernelGGL((absmax_kernel<ABSMAX_ROWS, true>), dim3((unsigned)((C + 255) / 256), (unsigned)(R / ABSMAX_ROWS)),
                        dim3(256), 0, st, xp, ldx, wsu, wsu + R, R, (int)C);
@@ -984,13 +1014,18 @@ static int scratch_address(const char* fn, float** out) {
     *out = addr[dev];
     return TI8_OK;
 }
+
+int init_quant_scratch() {
+    float* p = nullptr;
+    return scratch_address("ti8_init", &p);
+}
 }  // namespace ti8
 
 extern "C" int ti8_quant_row_col_t_noalloc(const void* x, int64_t ldx, int8_t* q, int64_t ldq, float* s_row, int8_t* qT,
                                            int64_t ldqt, float* s_col, int64_t R, int64_t C, int qflags,
                                            int inv_mode, ti8_stream_t stream) {
     const char* fn = "ti8_quant_row_col_t_noalloc";
-    if (qflags & (TI8_Q_WS_PINGPONG | TI8_Q_WS_SECOND))
+    if (qflags & (TI8_Q_WS_PINGPONG | TI8_Q_WS_SECOND | TI8_Q_WS_IS_ZERO))
         return fail(TI8_ERR_MODE, "%s: the workspace flags belong to ti8_quant_row_col_t (there is no workspace argument here)", fn);
     if (R > 0 && C > 0 && R + C > TI8_NOALLOC_MAX_ROWS_PLUS_COLS)
         return fail(TI8_ERR_SHAPE, "%s: R + C = %lld exceeds the library's fixed scratch of %d floats; use ti8_quant_row_col_t with a workspace",

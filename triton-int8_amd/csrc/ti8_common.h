@@ -4,6 +4,7 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <stdarg.h>
+#include <atomic>
 
 #include "../../include/ti8.h"
 
@@ -27,6 +28,47 @@ inline int check_launch(const char* what) {
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---- per-device one-time set-up (host) ---------------------------------------------
+inline int current_device() {
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    return dev;
+}
+
+// One bit per device index: whether a kernel's dynamic LDS limit has been raised there.  The call is idempotent,
+// so two threads that race through it only repeat it.  ti8_init() goes through every kernel that needs it, so that
+// nothing of the kind is left for the first launch.
+struct OncePerDevice {
+    std::atomic<uint64_t> done{0};
+};
+inline hipError_t raise_lds_limit(OncePerDevice& once, const void* kern, int bytes) {
+    const uint64_t bit = 1ull << (current_device() & 63);
+    if (once.done.load(std::memory_order_acquire) & bit) return hipSuccess;
+    const hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess) once.done.fetch_or(bit, std::memory_order_release);
+    else (void)hipGetLastError();
+    return e;
+}
+
+// Compute units of the current device (looked up once per device).
+int device_cu_count();
+
+// What ti8_init() calls: the per-device set-up of each source file's kernels (LDS limits, device symbols).
+int init_gemm_kernels();
+int init_chain_kernel();
+int init_skinny_kernels();
+int init_fwht_kernels();
+int init_quant_scratch();
+
+// ---- pieces of quant.hip that the one-call step (step.hip) uses --------------------
+// ti8_quant_block_multi that also zeroes `clear_words` 32-bit words at `clear` (NULL: nothing) in the same launch
+int quant_block_multi_and_clear(const ti8_qblock_operand* operands, int count, int qflags, int inv_mode,
+                                unsigned int* clear, int64_t clear_words, ti8_stream_t stream);
+int fill_words(unsigned int* p, int64_t words, unsigned int value, hipStream_t st);
+
+// ---- which kernel served the last GEMM call of this thread (ti8_last_gemm_kernel) ---
+void note_gemm_kernel(int kind, int bm, int bn, int epi);
 
 // ---- device helpers --------------------------------------------------------------
 typedef int v4i __attribute__((ext_vector_type(4)));

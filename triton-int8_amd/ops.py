@@ -16,7 +16,8 @@ from ._lib import (COMBINE_DIV_PROD, COMBINE_MUL_MUL, COMBINE_MUL_PROD, GEMM_LAR
                    Q_WS_PINGPONG, Q_WS_SECOND,
                    SCALE_BLOCK128, SCALE_BLOCK_K256, SCALE_ROW, SCALE_ROW_K128)
 
-__all__ = ["quant_block", "quant_block_multi", "quant_block_had128", "quant_row", "quant_col_t", "quant_row_col_t", "fwht", "fwht_t", "gemm_i8_nt", "gemm_i8_nt_i32"]
+__all__ = ["quant_block", "quant_block_multi", "quant_block_had128", "quant_row", "quant_col_t", "quant_row_col_t", "fwht", "fwht_t", "gemm_i8_nt", "gemm_i8_nt_i32",
+           "linear_step", "linear_step_workspace_bytes"]
 
 
 # Which GEMM kernel `gemm_i8_nt` asks for: "auto" (the few-rows kernel for M <= 256, else an
@@ -394,3 +395,54 @@ def gemm_i8_nt_i32(A, B):
               B.data_ptr(), B.stride(0) if B.dim() == 3 else 0, B.stride(-2),
               C.data_ptr(), C.stride(0), C.stride(1), batch, M, N, K, _stream())
     return C
+
+
+_STEP_SCHEMES = {"block_channel": _lib.SCHEME_BLOCK_CHANNEL, "double_channel": _lib.SCHEME_DOUBLE_CHANNEL}
+
+
+def linear_step_workspace_bytes(T, K, N, scheme):
+    """Bytes of workspace that :func:`linear_step` needs for T tokens (a multiple of 128), K inputs and N outputs."""
+    _need(scheme in _STEP_SCHEMES, f"linear_step serves the schemes {sorted(_STEP_SCHEMES)}")
+    n = _lib.lib().ti8_linear_fwd_bwd_workspace(T, K, N, _STEP_SCHEMES[scheme])
+    _need(n >= 0, f"T, K and N must be positive multiples of 128, got T={T} K={K} N={N}")
+    return n
+
+
+def linear_step(X2, W, dY2, scheme, *, out=None, workspace=None):
+    """A whole forward + backward of the layer in ONE library call (``ti8_linear_fwd_bwd``): X2 bf16 [T, K],
+    W bf16 [N, K], dY2 bf16 [T, N] -> (Y [T, N], dX [T, K], dW [N, K]), the quantisers and GEMMs of
+    ``linear.linear_forward`` + ``linear.linear_backward`` enqueued from C with the same bits.
+    T, K, N multiples of 128.  ``out`` = (Y, dX, dW) to write into; ``workspace`` = a uint8 tensor of at least
+    :func:`linear_step_workspace_bytes` bytes (both allocated here when absent)."""
+    for t, name in ((X2, "X"), (W, "W"), (dY2, "dY")):
+        _check_bf16(t, name)
+        _need(t.dim() == 2, f"{name} must be 2-D")
+    T, K = X2.shape
+    N = W.shape[0]
+    _need(W.shape[1] == K and tuple(dY2.shape) == (T, N), f"shapes do not fit: X {tuple(X2.shape)}, W {tuple(W.shape)}, dY {tuple(dY2.shape)}")
+    need = linear_step_workspace_bytes(T, K, N, scheme)
+
+    def rows(t):
+        if t.stride(1) != 1 or t.stride(0) % 8 or t.data_ptr() % 16:
+            t = t.contiguous()
+        return t
+    X2, W, dY2 = rows(X2), rows(W), rows(dY2)
+    dev = X2.device
+    if out is None:
+        out = (torch.empty((T, N), dtype=torch.bfloat16, device=dev), torch.empty((T, K), dtype=torch.bfloat16, device=dev),
+               torch.empty((N, K), dtype=torch.bfloat16, device=dev))
+    else:
+        for o, shape in zip(out, ((T, N), (T, K), (N, K))):
+            _need(tuple(o.shape) == shape and o.dtype == torch.bfloat16 and o.stride(1) == 1 and _on_gpu(o), "bad `out` tensor")
+    if workspace is None:
+        workspace = torch.empty((need + 256,), dtype=torch.uint8, device=dev)
+        workspace = workspace[(-workspace.data_ptr()) % 256:][:need]    # device allocations are aligned already: a no-op there
+    else:
+        _need(workspace.dtype == torch.uint8 and workspace.is_contiguous() and workspace.numel() >= need and _on_gpu(workspace)
+              and workspace.data_ptr() % 256 == 0, f"`workspace` must be a contiguous, 256-byte aligned uint8 GPU tensor of at least {need} bytes")
+    Y, dX, dW = out
+    _lib.call("ti8_linear_fwd_bwd", X2.data_ptr(), X2.stride(0), W.data_ptr(), W.stride(0), dY2.data_ptr(), dY2.stride(0),
+              Y.data_ptr(), Y.stride(0), dX.data_ptr(), dX.stride(0), dW.data_ptr(), dW.stride(0), T, K, N, _STEP_SCHEMES[scheme],
+              {"auto": 0, "tiled": GEMM_TILED, "large": GEMM_LARGE_TILES}.get(GEMM_PATH, 0) | (0 if GEMM_PERSISTENT else GEMM_ONE_TILE),
+              workspace.data_ptr(), workspace.numel(), _stream())
+    return Y, dX, dW
