@@ -35,6 +35,10 @@ __device__ __forceinline__ float scale_at(const ScaleDesc& d, int64_t batch, int
     return d.p[idx::scale_index(d.mode, d.bs, d.rs, d.ks, batch, row, kb)];
 }
 
+#ifndef TI8_LOAD_AUX
+#define TI8_LOAD_AUX 0   // cache policy bits of the operand loads (0: default)
+#endif
+
 // One wave's share of a K tile: NI global->LDS instructions of 64 x 16 bytes; instruction i
 // fills the 1 KiB slab at lds + i*1024 (lane l lands at byte 16*l of the slab) from
 // base + i*stride8 (wave-uniform: 8 rows further per instruction) + voff[(t0 + i) & 1] (per lane).
@@ -49,7 +53,7 @@ __device__ __forceinline__ void issue_tile_loads(const int8_t* base, int64_t str
     asm volatile("" : "+v"(vo[0]), "+v"(vo[1]));
 #pragma unroll
     for (int i = 0; i < NI; ++i)
-        __builtin_amdgcn_global_load_lds(base + i * stride8 + vo[(t0 + i) & 1], lds + i * 1024, 16, 0, 0);   // = idx::gemm_load_offset_bytes
+        __builtin_amdgcn_global_load_lds(base + i * stride8 + vo[(t0 + i) & 1], lds + i * 1024, 16, 0, TI8_LOAD_AUX);   // = idx::gemm_load_offset_bytes
 #else
     (void)base; (void)stride8; (void)voff; (void)t0; (void)lds;
 #endif
