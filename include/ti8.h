@@ -332,9 +332,12 @@ int ti8_gemm_i8_nt_multi(const ti8_gemm_problem* problems, int count, int gemm_f
  *   TI8_SCHEME_BLOCK_CHANNEL   ti8_quant_block_multi(X, dY; q and qT) -> ti8_quant_row_col_t(W) ->
  *                              ti8_gemm_i8_nt_multi(Y, dX, dW)          (3 launches + W's absmax pass)
  *   TI8_SCHEME_DOUBLE_CHANNEL  ti8_quant_row_col_t on X, W, dY (TI8_INV_AMAX_DIV_127) -> three
- *                              ti8_gemm_i8_nt(acc_i32_full = 1, TI8_GEMM_TILED)
+ *                              ti8_gemm_i8_nt(acc_i32_full = 1)
  *   X bf16 [T][K] (ldx), W bf16 [N][K] (ldw), dY bf16 [T][N] (lddy)  ->  Y bf16 [T][N], dX bf16 [T][K], dW bf16 [N][K]
- *   T, K, N multiples of 128 (zero-pad the tokens: padded rows change no absmax and add nothing to dW).
+ *   T, K, N multiples of 128.  `tokens` (1 <= tokens <= T) = the rows of X and dY that hold data when the caller has
+ *   zero-padded them to T rows (padded rows change no absmax and add nothing to dW; pass tokens = T otherwise).  With
+ *   T <= 256 or N <= 256 the GEMMs are launched one by one, as ti8_gemm_i8_nt would launch them (few-rows kernel up to 256
+ *   rows), and Y and dX are computed for the first ceil(tokens / 32) * 32 rows only.
  *   workspace: ti8_linear_fwd_bwd_workspace(T, K, N, scheme) bytes of device memory, 256-byte aligned, contents
  *   undefined before and after (it holds the int8 operands, their transposes, scales and maxima; the call clears
  *   what it needs cleared itself, so the same buffer serves any sequence of calls in stream order).
@@ -348,7 +351,7 @@ enum ti8_scheme {
 int64_t ti8_linear_fwd_bwd_workspace(int64_t T, int64_t K, int64_t N, int scheme);
 int ti8_linear_fwd_bwd(const void* X, int64_t ldx, const void* W, int64_t ldw, const void* dY, int64_t lddy,
                        void* Y, int64_t ldy, void* dX, int64_t lddx, void* dW, int64_t lddw,
-                       int64_t T, int64_t K, int64_t N, int scheme, int gemm_flags,
+                       int64_t T, int64_t tokens, int64_t K, int64_t N, int scheme, int gemm_flags,
                        void* workspace, int64_t workspace_bytes, ti8_stream_t stream);
 
 /* Raw int32 accumulators of the same GEMM over the whole K, C int32 [batch][M][N]:

@@ -256,7 +256,9 @@ def test_one_call_step_matches_the_assembled_step(T, dev):
     from triton_int8_amd import linear, ops
     from triton_int8_amd._lib import KERNEL_ONE_TILE, KERNEL_PERSISTENT_CHAIN
     g = make_gen(31)
-    for (M, K, N) in ((640, 512, 384), (4096, 4096, 4096)):     # the second: 256 tiles of 256 x 256 per GEMM, the persistent kernel
+    # few and ragged token counts (the GEMMs launched one by one, few-rows kernel on the live rows), more than 256 tokens
+    # and features (one launch), and 256 tiles of 256 x 256 per GEMM (the persistent kernel)
+    for (M, K, N) in ((16, 512, 256), (100, 512, 384), (128, 4096, 4096), (300, 512, 256), (640, 512, 384), (4096, 4096, 4096)):
         X = config_operand(M, K, g, outlier_frac=0.01, outlier_mul=20.0).to(dev)
         W, dY = config_operand(N, K, g, std=0.02).to(dev), config_operand(M, N, g, std=1e-3).to(dev)
         for scheme in ("block_channel", "double_channel"):
@@ -268,6 +270,10 @@ def test_one_call_step_matches_the_assembled_step(T, dev):
             with T._lib.timed_launches() as rec:
                 got = T.linear_fwd_bwd(X, W, dY, scheme)
             assert list(rec) == ["ti8_linear_fwd_bwd"], list(rec)
+            for a, b in zip(got, want):
+                assert a.shape == b.shape and torch.equal(a, b), (scheme, M)
+            if M % 128:
+                continue
             if scheme == "block_channel" and M >= 4096:
                 assert T.last_gemm_kernel() == KERNEL_PERSISTENT_CHAIN
             for a, b in zip(got, want):

@@ -264,10 +264,10 @@ def test_one_call_step_workspace(recorded, scheme, M, K, N):
     Y, dX, dW = T.linear_fwd_bwd(X, W, dY, scheme)
     assert [c[0] for c in calls] == ["ti8_linear_fwd_bwd"]
     a = calls[0][1]
-    assert (a[12], a[13], a[14]) == (M, K, N) and (a[1], a[3], a[5], a[7], a[9], a[11]) == (K, K, N, N, K, K)
+    assert (a[12], a[13], a[14], a[15]) == (M, M, K, N) and (a[1], a[3], a[5], a[7], a[9], a[11]) == (K, K, N, N, K, K)
     for ptr, elems in ((a[0], M * K), (a[2], N * K), (a[4], M * N), (a[6], M * N), (a[8], M * K), (a[10], N * K)):
         assert allocs.room(ptr, 2) >= elems
-    ws_ptr, ws_bytes = a[17], a[18]
+    ws_ptr, ws_bytes = a[18], a[19]
     assert ws_ptr % 256 == 0 and allocs.room(ws_ptr, 1) >= ws_bytes == T.ops.linear_step_workspace_bytes(M, K, N, scheme)
     int8_bytes = 2 * (M * K + M * N + N * K)                     # q and qT of every operand
     if scheme == "block_channel":

@@ -45,7 +45,7 @@ PROTOTYPES = {
                        _i64, _i64, _i64, _i64, _int, _int, _f32, _f32, _int, _vp],
     "ti8_gemm_i8_nt_multi": [ctypes.POINTER(GemmProblem), _int, _int, _vp],
     "ti8_gemm_i8_nt_i32": [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp],
-    "ti8_linear_fwd_bwd": [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp, _i64, _vp],
+    "ti8_linear_fwd_bwd": [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp, _i64, _vp],
     "ti8_probe_mfma": [_vp, _i64, _vp, _int, _int, _int, _int, _vp],
 }
 EXPORTS = ["ti8_version", "ti8_last_error", "ti8_arch", "ti8_init", "ti8_last_gemm_kernel", "ti8_linear_fwd_bwd_workspace"] + list(PROTOTYPES)

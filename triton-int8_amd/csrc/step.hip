@@ -95,13 +95,14 @@ ti8_gemm_problem gemm2d(const int8_t* A, int64_t lda, const float* sA, int modeA
 }
 
 int check_step(const char* fn, const void* X, int64_t ldx, const void* W, int64_t ldw, const void* dY, int64_t lddy, const void* Y,
-               int64_t ldy, const void* dX, int64_t lddx, const void* dW, int64_t lddw, int64_t T, int64_t K, int64_t N, int scheme) {
+               int64_t ldy, const void* dX, int64_t lddx, const void* dW, int64_t lddw, int64_t T, int64_t tokens, int64_t K, int64_t N, int scheme) {
     if (scheme != TI8_SCHEME_BLOCK_CHANNEL && scheme != TI8_SCHEME_DOUBLE_CHANNEL)
         return fail(TI8_ERR_MODE, "%s: scheme must be TI8_SCHEME_BLOCK_CHANNEL or TI8_SCHEME_DOUBLE_CHANNEL, got %d", fn, scheme);
     if (!X || !W || !dY || !Y || !dX || !dW) return fail(TI8_ERR_NULL, "%s: X, W, dY, Y, dX and dW are required", fn);
     if (T <= 0 || K <= 0 || N <= 0 || T % 128 || K % 128 || N % 128 || T > 0x3fffffff || K > 0x3fffffff || N > 0x3fffffff)
         return fail(TI8_ERR_SHAPE, "%s: T, K and N must be positive multiples of 128 (zero-pad the tokens); got T=%lld K=%lld N=%lld", fn,
                     (long long)T, (long long)K, (long long)N);
+    if (tokens < 1 || tokens > T) return fail(TI8_ERR_SHAPE, "%s: tokens must be in [1, T]; got tokens=%lld T=%lld", fn, (long long)tokens, (long long)T);
     if (ldx < K || ldw < K || lddy < N || ldy < N || lddx < K || lddw < K) return fail(TI8_ERR_SHAPE, "%s: leading dimension smaller than the row length", fn);
     return TI8_OK;
 }
@@ -118,12 +119,21 @@ extern "C" int64_t ti8_linear_fwd_bwd_workspace(int64_t T, int64_t K, int64_t N,
     return -1;
 }
 
+// One GEMM of the step launched alone (what ti8_gemm_i8_nt selects for its shape: the few-rows kernel up to 256 rows).
+// `live` rows of A are multiplied: with few tokens the padding rows of the 128-row-quantised operand are zeros whose
+// products nobody reads.
+static int one_gemm(const ti8_gemm_problem& p, int64_t live, int gemm_flags, ti8_stream_t stream) {
+    return ti8_gemm_i8_nt(p.A, p.bsa, p.lda, p.B, p.bsb, p.ldb, p.C, p.bsc, p.ldc, p.sA, p.modeA, p.sa_bs, p.sa_rs, p.sa_ks,
+                          p.sB, p.modeB, p.sb_bs, p.sb_rs, p.sb_ks, 1, live, p.N, p.K, p.acc_i32_full, p.combine, p.out_scale, p.post_scale,
+                          gemm_flags, stream);
+}
+
 extern "C" int ti8_linear_fwd_bwd(const void* X, int64_t ldx, const void* W, int64_t ldw, const void* dY, int64_t lddy,
                                   void* Y, int64_t ldy, void* dX, int64_t lddx, void* dW, int64_t lddw,
-                                  int64_t T, int64_t K, int64_t N, int scheme, int gemm_flags,
+                                  int64_t T, int64_t tokens, int64_t K, int64_t N, int scheme, int gemm_flags,
                                   void* workspace, int64_t workspace_bytes, ti8_stream_t stream) {
     const char* fn = "ti8_linear_fwd_bwd";
-    if (int e = check_step(fn, X, ldx, W, ldw, dY, lddy, Y, ldy, dX, lddx, dW, lddw, T, K, N, scheme)) return e;
+    if (int e = check_step(fn, X, ldx, W, ldw, dY, lddy, Y, ldy, dX, lddx, dW, lddw, T, tokens, K, N, scheme)) return e;
     const int64_t need = ti8_linear_fwd_bwd_workspace(T, K, N, scheme);
     if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255) || workspace_bytes < need)
         return fail(TI8_ERR_SHAPE, "%s: the workspace must be 256-byte aligned and hold %lld bytes (ti8_linear_fwd_bwd_workspace); got %lld", fn,
@@ -131,6 +141,15 @@ extern "C" int ti8_linear_fwd_bwd(const void* X, int64_t ldx, const void* W, int
     if (gemm_flags & ~(TI8_GEMM_TILED | TI8_GEMM_LARGE_TILES | TI8_GEMM_ONE_TILE)) return fail(TI8_ERR_MODE, "%s: only TI8_GEMM_TILED, TI8_GEMM_LARGE_TILES and TI8_GEMM_ONE_TILE apply here", fn);
     char* base = static_cast<char*>(workspace);
     const int q = TI8_Q_CLAMP;
+    // rows of the token operands that Y and dX multiply: all of them, or with up to 256 (padded) tokens the real ones
+    // rounded up to 32, which the few-rows kernel takes
+    auto live_rows = [&](int64_t contraction) {
+        if (T > 256 || (gemm_flags & (TI8_GEMM_TILED | TI8_GEMM_LARGE_TILES)) || contraction > 32768) return T;
+        const int64_t r = (tokens + 31) / 32 * 32;
+        return r < T ? r : T;
+    };
+    // the three GEMMs go into one launch where none of them has so few rows that it would take the few-rows kernel
+    const bool one_launch = (T < N ? T : N) > 256;
 
     if (scheme == TI8_SCHEME_BLOCK_CHANNEL) {
         // triton/block_channel_fwd32.py:221-222 on (X, W) and on (dY, W^T), triton/block_channel_bwd33.py:153-154 on (dY^T, X^T):
@@ -148,7 +167,10 @@ extern "C" int ti8_linear_fwd_bwd(const void* X, int64_t ldx, const void* W, int
             gemm2d(L.x.q, K, L.x.s, TI8_SCALE_BLOCK128, K / 128, 1, L.w.q, K, L.w.s_row, TI8_SCALE_ROW, 1, 0, Y, ldy, T, N, K, 0),
             gemm2d(L.dy.q, N, L.dy.s, TI8_SCALE_BLOCK128, N / 128, 1, L.w.qT, N, L.w.s_col, TI8_SCALE_ROW, 1, 0, dX, lddx, T, K, N, 0),
             gemm2d(L.dy.qT, T, L.dy.s, TI8_SCALE_BLOCK128, 1, N / 128, L.x.qT, T, L.x.s, TI8_SCALE_BLOCK128, 1, K / 128, dW, lddw, N, K, T, 0)};
-        return ti8_gemm_i8_nt_multi(g, 3, gemm_flags, stream);
+        if (one_launch) return ti8_gemm_i8_nt_multi(g, 3, gemm_flags, stream);
+        if (int e = one_gemm(g[0], live_rows(K), gemm_flags, stream)) return e;
+        if (int e = one_gemm(g[1], live_rows(N), gemm_flags, stream)) return e;
+        return one_gemm(g[2], N, gemm_flags, stream);
     }
 
     // double-channel: every operand per row and per column (triton/double-channle_fwd32.py:277-278 on (X, W) and (dY, W^T),
@@ -165,11 +187,7 @@ extern "C" int ti8_linear_fwd_bwd(const void* X, int64_t ldx, const void* W, int
         gemm2d(L.dy.q, N, L.dy.s_row, TI8_SCALE_ROW, 1, 0, L.w.qT, N, L.w.s_col, TI8_SCALE_ROW, 1, 0, dX, lddx, T, K, N, 1),
         gemm2d(L.dy.qT, T, L.dy.s_col, TI8_SCALE_ROW, 1, 0, L.x.qT, T, L.x.s_col, TI8_SCALE_ROW, 1, 0, dW, lddw, N, K, T, 1)};
     // three launches: the int32 kernel gains nothing from one launch of all three
-    for (int i = 0; i < 3; ++i) {
-        const ti8_gemm_problem& p = g[i];
-        if (int e = ti8_gemm_i8_nt(p.A, p.bsa, p.lda, p.B, p.bsb, p.ldb, p.C, p.bsc, p.ldc, p.sA, p.modeA, p.sa_bs, p.sa_rs, p.sa_ks,
-                                   p.sB, p.modeB, p.sb_bs, p.sb_rs, p.sb_ks, 1, p.M, p.N, p.K, 1, p.combine, p.out_scale, p.post_scale,
-                                   gemm_flags | TI8_GEMM_TILED, stream)) return e;
-    }
-    return TI8_OK;
+    if (int e = one_gemm(g[0], live_rows(K), gemm_flags, stream)) return e;
+    if (int e = one_gemm(g[1], live_rows(N), gemm_flags, stream)) return e;
+    return one_gemm(g[2], N, gemm_flags, stream);
 }

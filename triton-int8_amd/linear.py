@@ -265,8 +265,7 @@ def _one_launch(scheme, hadamard, padded_tokens, out_features):
 
 
 # Schemes whose whole step is one library call (ops.linear_step: the same launches, queued from C) when nothing is
-# rotated and no GEMM of the step has so few rows that it would take the few-rows kernel.  False: the step is
-# assembled here from the separate entry points (same bits; the tests run both).
+# rotated.  False: the step is assembled here from the separate entry points (same bits; the tests run both).
 ONE_CALL_STEP = True
 ONE_CALL_SCHEMES = ("block_channel", "double_channel")
 
@@ -285,14 +284,13 @@ def linear_fwd_bwd(X, W, dY, scheme="block_channel", hadamard=None, out=None, wo
     if T == 0:   # nothing to multiply: empty Y and dX, a zero weight gradient (as torch.nn.functional.linear gives)
         return X.new_empty((*lead, N)), X.new_empty((*lead, K)), W.new_zeros((N, K))
     X2, dY2 = pad_tokens(X2), pad_tokens(dY2)
-    one_call = (ONE_CALL_STEP and scheme in ONE_CALL_SCHEMES and hadamard is None and min(X2.shape[0], N) > 256
-                and ops.GEMM_PATH in ("auto", "tiled", "large"))
+    one_call = ONE_CALL_STEP and scheme in ONE_CALL_SCHEMES and hadamard is None and ops.GEMM_PATH in ("auto", "tiled", "large")
     if out is not None or workspace is not None:
         if not one_call or X2.shape[0] != T:
             raise ValueError("`out` / `workspace` go with the one-call step: block_channel or double_channel without rotation, "
-                             "more than 256 tokens and output features, tokens a multiple of 128")
+                             "tokens a multiple of 128")
     if one_call:
-        Y, dX, dW = ops.linear_step(X2, W, dY2, scheme, out=out, workspace=workspace)
+        Y, dX, dW = ops.linear_step(X2, W, dY2, scheme, tokens=T, out=out, workspace=workspace)
         return Y[:T].reshape(*lead, N), dX[:T].reshape(*lead, K), dW
     gemms = [] if _one_launch(scheme, hadamard, X2.shape[0], N) else None
     pre = None

@@ -408,11 +408,12 @@ def linear_step_workspace_bytes(T, K, N, scheme):
     return n
 
 
-def linear_step(X2, W, dY2, scheme, *, out=None, workspace=None):
+def linear_step(X2, W, dY2, scheme, *, tokens=None, out=None, workspace=None):
     """A whole forward + backward of the layer in ONE library call (``ti8_linear_fwd_bwd``): X2 bf16 [T, K],
     W bf16 [N, K], dY2 bf16 [T, N] -> (Y [T, N], dX [T, K], dW [N, K]), the quantisers and GEMMs of
     ``linear.linear_forward`` + ``linear.linear_backward`` enqueued from C with the same bits.
-    T, K, N multiples of 128.  ``out`` = (Y, dX, dW) to write into; ``workspace`` = a uint8 tensor of at least
+    T, K, N multiples of 128; ``tokens`` = rows that hold data when the caller has zero-padded X2 and dY2 (with up to
+    256 rows Y and dX are then computed for the first ceil(tokens / 32) * 32 rows only).  ``out`` = (Y, dX, dW) to write into; ``workspace`` = a uint8 tensor of at least
     :func:`linear_step_workspace_bytes` bytes (both allocated here when absent)."""
     for t, name in ((X2, "X"), (W, "W"), (dY2, "dY")):
         _check_bf16(t, name)
@@ -442,7 +443,8 @@ def linear_step(X2, W, dY2, scheme, *, out=None, workspace=None):
               and workspace.data_ptr() % 256 == 0, f"`workspace` must be a contiguous, 256-byte aligned uint8 GPU tensor of at least {need} bytes")
     Y, dX, dW = out
     _lib.call("ti8_linear_fwd_bwd", X2.data_ptr(), X2.stride(0), W.data_ptr(), W.stride(0), dY2.data_ptr(), dY2.stride(0),
-              Y.data_ptr(), Y.stride(0), dX.data_ptr(), dX.stride(0), dW.data_ptr(), dW.stride(0), T, K, N, _STEP_SCHEMES[scheme],
+              Y.data_ptr(), Y.stride(0), dX.data_ptr(), dX.stride(0), dW.data_ptr(), dW.stride(0), T, T if tokens is None else tokens, K, N,
+              _STEP_SCHEMES[scheme],
               {"auto": 0, "tiled": GEMM_TILED, "large": GEMM_LARGE_TILES}.get(GEMM_PATH, 0) | (0 if GEMM_PERSISTENT else GEMM_ONE_TILE),
               workspace.data_ptr(), workspace.numel(), _stream())
     return Y, dX, dW
