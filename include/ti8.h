@@ -258,7 +258,9 @@ int ti8_quant_row_col_t_noalloc(const void* x, int64_t ldx, int8_t* q, int64_t l
  * 189-190,208-209).  bf16 in, fp32 butterflies (strides 1,2,4,...), times `scale`,
  * one rounding to bf16 out.  Transforms contiguous groups of n along each row:
  * n = cols is the reference's full-length rotation, n = 128 the block-diagonal one.
- * n a power of two, 128 <= n <= 32768, cols % n == 0.  x == y is allowed. */
+ * n a power of two, 128 <= n <= 32768, cols % n == 0.  x == y is allowed.
+ * A row whose length is no power of two (n / 2 < cols < n, cols % 16 == 0, n the next power of two) is transformed as
+ * the external library transforms it: zero-extended to n, multiplied by H_n, cut back to its first cols elements. */
 int ti8_fwht(const void* x, int64_t ldx, void* y, int64_t ldy,
              int64_t rows, int64_t cols, int64_t n, float scale, ti8_stream_t stream);
 

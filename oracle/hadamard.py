@@ -35,10 +35,16 @@ def fwht_f32(xf: torch.Tensor, n: int) -> torch.Tensor:
 def hadamard_transform(x: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
     """Full-length transform along the last dim; bf16 in -> bf16 out (one rounding).
 
-    The last dim must be a power of two (the external library zero-pads other
-    lengths to the next power of two and truncates; that case is not modelled)."""
-    n = x.shape[-1]
-    y = fwht_f32(widen(x), n)
+    A last dim that is no power of two is handled as the external library documents it
+    ("if dim is not a power of 2, we implicitly pad x with zero so that dim is the next
+    power of 2"; the result has the input's shape): zero-extended to the next power of two,
+    transformed, cut back to the first ``dim`` elements."""
+    dim = x.shape[-1]
+    n = 1 << (dim - 1).bit_length()
+    xf = widen(x)
+    if n != dim:
+        xf = torch.nn.functional.pad(xf, (0, n - dim))
+    y = fwht_f32(xf, n)[..., :dim]
     if scale != 1.0:
         y = y * torch.tensor(scale, dtype=F32)
     return y.to(x.dtype)

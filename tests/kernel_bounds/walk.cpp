@@ -55,12 +55,14 @@ int walk_fwht(int64_t ldx, int64_t ldy, int64_t rows, int64_t cols, int64_t n, i
     Report r{msg, msglen};
     const int64_t L = fwht_segment_len(cols, n);
     const int NT = fwht_threads(L);
-    const int64_t nblocks = rows * (cols / L);
+    const bool extended = cols < L;             // a zero-extended row per workgroup
+    const int valid = (int)(extended ? cols : L);
+    const int64_t nblocks = rows * (extended ? 1 : cols / L);
     const int64_t lds_words = fwht_lds_words(L);
     if (lds_words * 4 > lds_bytes_limit) r.fail("fwht: %lld bytes of LDS requested, limit %lld", (long long)(lds_words * 4), (long long)lds_bytes_limit);
     int logn = 0;
     while ((1LL << logn) < n) ++logn;
-    const int segs_per_row = (int)(cols / L);
+    const int segs_per_row = extended ? 1 : (int)(cols / L);
     // LDS indices do not depend on the workgroup: walk them once
     for (int tid = 0; tid < NT && !r.bad; ++tid) {
         for (int vt = tid; vt < (L >> 4); vt += NT)
@@ -88,10 +90,12 @@ int walk_fwht(int64_t ldx, int64_t ldy, int64_t rows, int64_t cols, int64_t n, i
         const int64_t yo = fwht_segment_offset(block, segs_per_row, ldy, (int)L);
         for (int tid = 0; tid < NT; ++tid) {
             for (int vt = tid; vt < (L >> 4); vt += NT) {   // two 16-byte loads: elements vt*16 .. +16
+                if (!fwht_chunk_valid(vt * 16, 16, valid)) continue;
                 r.access("fwht x", xo + vt * 16, 8, x_elems, block, tid, vt);
                 r.access("fwht x", xo + vt * 16 + 8, 8, x_elems, block, tid, vt);
             }
-            for (int c = tid; c < (L >> 3); c += NT) r.access("fwht y", yo + c * 8, 8, y_elems, block, tid, c);
+            for (int c = tid; c < (L >> 3); c += NT)
+                if (fwht_chunk_valid(c * 8, 8, valid)) r.access("fwht y", yo + c * 8, 8, y_elems, block, tid, c);
         }
     }
     *n_checked = r.checked;

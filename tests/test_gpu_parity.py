@@ -359,6 +359,25 @@ def test_row_and_col_quant_workspace_cache_is_bounded(T, dev):
     assert not errors, errors[0]
 
 
+@pytest.mark.parametrize("cols", [96, 144, 384, 1792, 3584, 14336, 24576])
+def test_fwht_of_a_length_that_is_no_power_of_two(T, dev, cols):
+    """Zero-extended to the next power of two, transformed, cut back (the external library's rule; 14336 is the Llama MLP
+    width the reference's pipeline would hand it): bit for bit against the oracle, also in place and from a strided
+    input; the double-channel pipeline built on it against its oracle."""
+    x = randn_bf16(make_gen(cols), 5, cols)
+    want = ohad.hadamard_transform(x)
+    assert bits_equal(T.ops.fwht(x.to(dev)), want)
+    assert bits_equal(T.double_channel_fwd32.hadamard_transform(x.to(dev), 0.25), ohad.hadamard_transform(x, 0.25))
+    wide = randn_bf16(make_gen(cols + 1), 5, cols + 64).to(dev)
+    assert bits_equal(T.ops.fwht(wide[:, :cols]), ohad.hadamard_transform(wide[:, :cols].cpu()))
+    if cols % 128 == 0 and cols >= 256:
+        xt = randn_bf16(make_gen(cols + 2), cols, 24)
+        assert bits_equal(T.ops.fwht_t(xt.to(dev)), ohad.hadamard_transform(xt.t().contiguous()))
+    if cols % 2048 == 0:
+        a, b = randn_bf16(make_gen(cols + 3), 1, 128, cols), randn_bf16(make_gen(cols + 4), 256, cols)
+        assert bits_equal(T.double_channel_fwd32.fwd_32(a.to(dev), b.to(dev)), odf.fwd_32(a, b))
+
+
 @pytest.mark.parametrize("n,cols", [(128, 384), (128, 4096), (256, 256), (512, 1536), (1024, 2048), (2048, 2048),
                                     (4096, 4096), (8192, 8192), (16384, 16384), (32768, 32768)])
 def test_fwht(T, dev, n, cols):

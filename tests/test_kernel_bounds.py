@@ -239,6 +239,21 @@ def test_transposed_hadamard_launches(walker, recorded, R, C):
     assert walker.walk_fwht_t(C, R, R, C, R * C, R * C - 8, LDS_LIMIT, ctypes.byref(n), msg, 512) == 1 and msg.value.split(b":")[0].endswith(b" y")
 
 
+@pytest.mark.parametrize("rows,cols", [(3, 96), (5, 1792), (4, 14336), (2, 24576)])
+def test_zero_extended_hadamard_launch(walker, recorded, rows, cols):
+    """ti8_fwht on a length that is no power of two: one zero-extended row per workgroup, nothing read or stored beyond
+    the row's own elements."""
+    T, allocs, calls = recorded
+    y = T.ops.fwht(torch.empty(rows, cols, dtype=torch.bfloat16))
+    assert tuple(y.shape) == (rows, cols) and [c[0] for c in calls] == ["ti8_fwht"]
+    assert calls[0][1][6] == 1 << (cols - 1).bit_length()
+    assert walk(walker, allocs, *calls[0]) >= rows * cols // 8
+    msg, n = ctypes.create_string_buffer(512), ctypes.c_int64(0)
+    nn = 1 << (cols - 1).bit_length()
+    assert walker.walk_fwht(cols, cols, rows, cols, nn, rows * cols - 8, rows * cols, LDS_LIMIT, ctypes.byref(n), msg, 512) == 1 and b"fwht x" in msg.value
+    assert walker.walk_fwht(cols, cols, rows, cols, nn, rows * cols, rows * cols - 8, LDS_LIMIT, ctypes.byref(n), msg, 512) == 1 and b"fwht y" in msg.value
+
+
 @pytest.mark.parametrize("M,K,N", [(1024, 512, 768), (8192, 4096, 4096)])
 def test_one_launch_step_is_in_bounds(walker, recorded, monkeypatch, M, K, N):
     """The three GEMMs of a block-channel step in one launch: each GEMM's accesses stay inside its operands, and the

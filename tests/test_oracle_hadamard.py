@@ -51,3 +51,27 @@ def test_bf16_interface_and_block_diagonal():
     assert float((yb.double() - refb).norm() / refb.norm()) < 4e-3
     # along another dim = transpose, transform, transpose back
     assert bits_equal(hadamard128(x.t().contiguous(), dim=0), hadamard128(x).t().contiguous())
+
+
+@pytest.mark.parametrize("dim", [96, 384, 1792])
+def test_a_length_that_is_no_power_of_two_is_zero_extended_and_cut_back(dim):
+    """The external library's documented rule for such a length (the reference hands it K = 14336 of the Llama MLP
+    unchanged, triton/double-channle_fwd32.py:299-300): pad with zeros to the next power of two, multiply by H, keep the
+    first `dim` outputs.  Against scipy's matrix on small integers (exact), and NOT an orthogonal map."""
+    n = 1 << (dim - 1).bit_length()
+    g = make_gen(dim)
+    x = torch.zeros(5, dim)
+    for r in range(5):      # 40 small integers per row: every output is an integer below 128 in magnitude, exact also in bf16
+        x[r, torch.randperm(dim, generator=g)[:40]] = torch.randint(1, 4, (40,), generator=g).float() * (torch.randint(0, 2, (40,), generator=g) * 2 - 1)
+    x = x.to(torch.bfloat16)
+    H = torch.from_numpy(scipy.linalg.hadamard(n).astype(np.float32))
+    want = (torch.nn.functional.pad(x.float(), (0, n - dim)) @ H)[:, :dim]
+    assert float(want.abs().max()) < 256                                      # representable in bf16
+    assert torch.equal(hadamard_transform(x).float(), want)
+    # = the first `dim` columns of the first `dim` rows of H_n: a one-hot gives that row of H, cut
+    e = torch.zeros(1, dim, dtype=torch.bfloat16)
+    e[0, dim - 1] = 1
+    assert torch.equal(hadamard_transform(e)[0].float(), H[dim - 1, :dim])
+    # power-of-two lengths are untouched by the rule
+    y = randn_bf16(g, 3, 256)
+    assert bits_equal(hadamard_transform(y), fwht_f32(y.float(), 256).to(torch.bfloat16))

@@ -71,14 +71,19 @@ __global__ __launch_bounds__(NT) void fwht_kernel(const uint16_t* __restrict__ x
                                                    int L, float scale) {
     extern __shared__ float lds[];
     const int tid = threadIdx.x;
-    const int segs_per_row = cols / L;
+    // cols < L: one zero-extended row per workgroup (a length that is no power of two, transformed as the next power of
+    // two and cut back): elements from `valid` on read as zero and are not stored
+    const int valid = cols < L ? cols : L;
+    const int segs_per_row = cols < L ? 1 : cols / L;
     const uint16_t* xr = x + idx::fwht_segment_offset(blockIdx.x, segs_per_row, ldx, L);
     uint16_t* yr = y + idx::fwht_segment_offset(blockIdx.x, segs_per_row, ldy, L);
 
     // pass over bits 0..3 (n >= 128, so all four stages belong to every group)
     for (int vt = tid; vt < (L >> 4); vt += NT) {
-        const uint4 v0 = *reinterpret_cast<const uint4*>(xr + vt * 16);
-        const uint4 v1 = *reinterpret_cast<const uint4*>(xr + vt * 16 + 8);
+        const bool in = idx::fwht_chunk_valid(vt * 16, 16, valid);   // valid is a multiple of 16: a chunk is inside or outside
+        const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
+        const uint4 v0 = in ? *reinterpret_cast<const uint4*>(xr + vt * 16) : zero4;
+        const uint4 v1 = in ? *reinterpret_cast<const uint4*>(xr + vt * 16 + 8) : zero4;
         float a[16] = {bf16_lo(v0.x), bf16_hi(v0.x), bf16_lo(v0.y), bf16_hi(v0.y), bf16_lo(v0.z), bf16_hi(v0.z),
                        bf16_lo(v0.w), bf16_hi(v0.w), bf16_lo(v1.x), bf16_hi(v1.x), bf16_lo(v1.y), bf16_hi(v1.y),
                        bf16_lo(v1.z), bf16_hi(v1.z), bf16_lo(v1.w), bf16_hi(v1.w)};
@@ -103,6 +108,7 @@ __global__ __launch_bounds__(NT) void fwht_kernel(const uint16_t* __restrict__ x
         }
     }
     for (int c = tid; c < (L >> 3); c += NT) {
+        if (!idx::fwht_chunk_valid(c * 8, 8, valid)) continue;
         const float* src = lds + padded(c * 8);   // 8 words of one 16-word run: contiguous
         float f[8];
 #pragma unroll
@@ -319,11 +325,15 @@ extern "C" int ti8_fwht(const void* x, int64_t ldx, void* y, int64_t ldy, int64_
                         float scale, ti8_stream_t stream) {
     if (!x || !y) return fail(TI8_ERR_NULL, "ti8_fwht: x and y are required");
     if (n < 128 || n > 32768 || (n & (n - 1))) return fail(TI8_ERR_SHAPE, "ti8_fwht: n must be a power of two in [128, 32768], got %lld", (long long)n);
-    if (rows <= 0 || cols <= 0 || cols % n) return fail(TI8_ERR_SHAPE, "ti8_fwht: need rows>0 and cols%%n==0; got rows=%lld cols=%lld n=%lld", (long long)rows, (long long)cols, (long long)n);
+    // cols a multiple of n, or a row shorter than n (n the next power of two: n / 2 < cols < n) that is transformed zero-extended
+    const bool extended = cols > n / 2 && cols < n;
+    if (rows <= 0 || cols <= 0 || (cols % n && !extended) || (extended && cols % 16))
+        return fail(TI8_ERR_SHAPE, "ti8_fwht: need rows>0 and cols%%n==0, or n/2 < cols < n with cols%%16==0; got rows=%lld cols=%lld n=%lld", (long long)rows, (long long)cols, (long long)n);
+    if (extended && x == y && ldx != ldy) return fail(TI8_ERR_MODE, "ti8_fwht: in place needs ldx == ldy");
     const int64_t L = idx::fwht_segment_len(cols, n);   // elements per workgroup
     if (ldx < cols || ldy < cols) return fail(TI8_ERR_SHAPE, "ti8_fwht: leading dimension smaller than cols");
     if (!aligned16(x) || !aligned16(y) || (ldx % 8) || (ldy % 8)) return fail(TI8_ERR_ALIGN, "ti8_fwht: pointers must be 16-byte aligned and strides multiples of 16 bytes");
-    const int64_t nblocks = rows * (cols / L);
+    const int64_t nblocks = rows * (extended ? 1 : cols / L);
     if (nblocks > 0x7fffffffLL) return fail(TI8_ERR_SHAPE, "ti8_fwht: too many segments");
     int logn = 0;
     while ((1LL << logn) < n) ++logn;

@@ -142,6 +142,9 @@ TI8_HD int64_t fwht_segment_offset(int64_t block, int segs_per_row, int64_t ld, 
     const int seg = (int)(block % segs_per_row);
     return row * ld + (int64_t)seg * L;
 }
+// whether the `len` elements from `first` of a segment exist in memory (`valid` elements do; the rest of a zero-extended
+// row reads as zero and is not stored); valid is a multiple of len
+TI8_HD bool fwht_chunk_valid(int first, int len, int valid) { return first + len <= valid; }
 // LDS words a workgroup needs for L elements
 TI8_HD int64_t fwht_lds_words(int64_t L) { return L + L / 16; }
 // base LDS index of the radix-2^rb group `vt` in the pass over index bits [p, p + rb)
@@ -225,7 +228,7 @@ TI8_HD QRowConfig qrow_config(int nchunk, bool group128) {
 // Walsh-Hadamard transform: elements per workgroup (a whole group of n when n >= 2048, else as
 // many groups as divide both the row and 2048) and threads per workgroup
 TI8_HD int64_t fwht_segment_len(int64_t cols, int64_t n) {
-    if (n >= 2048) return n;
+    if (n >= 2048 || cols < n) return n;    // cols < n: a zero-extended row of n elements per workgroup
     int64_t a = cols, b = 2048;
     while (b) {
         const int64_t t = a % b;

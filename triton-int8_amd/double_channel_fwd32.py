@@ -21,8 +21,11 @@ __all__ = ["hadamard_transform", "triton_per_row_quant_2d", "triton_per_row_quan
 def hadamard_transform(x: torch.Tensor, scale: float = 1.0):
     """Replacement of ``fast_hadamard_transform.hadamard_transform`` (the reference's
     external dependency, triton/double-channle_fwd32.py:8): ``x @ H_n * scale`` along
-    the last dim, Sylvester order, bf16 in -> bf16 out.  n must be a power of two in
-    [128, 32768] (the external library zero-pads other lengths; that is not offered)."""
+    the last dim, Sylvester order, bf16 in -> bf16 out, n a power of two in [128, 32768].
+    Other lengths (multiples of 16 up to 32768) are handled as the external library handles
+    them: zero-extended to the next power of two, transformed, cut back -- which is not an
+    orthogonal rotation any more, so the pipeline's result is only as good as the reference's
+    own at such a K (14336 of the Llama MLP)."""
     return ops.fwht(x, None, scale)
 
 

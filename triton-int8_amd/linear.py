@@ -214,8 +214,8 @@ def linear_backward(dY2, X2, W, scheme="block_channel", hadamard=None, saved=Non
     # double_channel
     if hadamard == "full":
         # the transposed operands are rotated along the rows of the tensors as they lie in memory (ops.fwht_t):
-        # no bf16 transpose of W, dY or X.  A token count that is not a power of two in [128, 32768] has no
-        # full-length rotation along the tokens (as in the reference, whose transform needs a power of two)
+        # no bf16 transpose of W, dY or X.  A length that is no power of two is rotated as the reference's external
+        # library rotates it (zero-extended to the next power of two and cut back, through a transposed copy)
         dq, ds = ops.quant_row(ops.fwht(dY2), clamp=True, inv_mode=INV_AMAX_DIV_127)
         wtq, wts = ops.quant_row(ops.fwht_t(W), clamp=True, inv_mode=INV_AMAX_DIV_127)
         dX = _gemm_dc(dq, ds, wtq, wts, 1.0 / N, tokens=tokens, gemms=gemms)

@@ -259,12 +259,15 @@ def _pingpong_workspace(device, stream, R, C):
 
 
 def fwht(x, n=None, scale=1.0):
-    """Un-normalised Walsh-Hadamard transform over groups of ``n`` (default: all) of the last dim."""
+    """Un-normalised Walsh-Hadamard transform over groups of ``n`` (default: all) of the last dim.
+    Without ``n``, a last dim that is no power of two is transformed as the reference's external library
+    transforms it: zero-extended to the next power of two, multiplied by H, cut back to its own length
+    (a multiple of 16 in (64, 32768))."""
     _check_bf16(x, "x")
     cols = x.shape[-1]
-    n = cols if n is None else n
+    n = (1 << max(cols - 1, 1).bit_length()) if n is None else n
     _need(n >= 128 and n <= 32768 and (n & (n - 1)) == 0, f"n must be a power of two in [128, 32768], got {n}")
-    _need(cols % n == 0, f"last dim {cols} is not a multiple of n={n}")
+    _need(cols % n == 0 or (n // 2 < cols < n and cols % 16 == 0), f"last dim {cols} is neither a multiple of n={n} nor a multiple of 16 in ({n // 2}, {n})")
     x2 = x.reshape(-1, cols)
     if x2.stride(1) != 1 or x2.stride(0) % 8 or x2.data_ptr() % 16:
         x2 = x2.contiguous()
@@ -279,7 +282,10 @@ def fwht_t(x, scale=1.0):
     _check_bf16(x, "x")
     _need(x.dim() == 2, "x must be [R, C]")
     R, C = x.shape
-    _need(R >= 128 and R <= 32768 and (R & (R - 1)) == 0, f"R must be a power of two in [128, 32768], got {R}")
+    if R & (R - 1) and R % 16 == 0 and 64 < R < 32768:
+        # a length that is no power of two: the zero-extended transform, on the transposed copy
+        return fwht(x.t().contiguous(), None, scale)
+    _need(R >= 128 and R <= 32768 and (R & (R - 1)) == 0, f"R must be a power of two in [128, 32768] or a multiple of 16 in (64, 32768), got {R}")
     _need(C > 0 and C % 8 == 0, f"C must be a positive multiple of 8, got {C}")
     if x.stride(1) != 1 or x.stride(0) % 8 or x.data_ptr() % 16:
         x = x.contiguous()
