@@ -271,21 +271,14 @@ def main():
         def step():
             return T.linear_fwd_bwd(X, W, dY, args.scheme)
 
-    # ---- the device leaves its idle clocks (settle), then the secondary figures FIRST: the activation quantiser against
-    # HBM, the bf16 GEMMs the reference times beside its int8 path (test.py:34-38), the device copy and the pure-MFMA
-    # probe.  They run before the steps, not after, so that the device is at its sustained clock when the warm-up starts:
+    # ---- the device leaves its idle clocks (settle), then secondary figures FIRST: the bf16 GEMMs the reference times
+    # beside its int8 path (test.py:34-38) and the pure-MFMA probe.  They run before the steps, not after, so that the
+    # device is at its sustained clock when the warm-up starts:
     # a GPU that has idled (process start, host-side set-up) takes some 20 ms of work to get back there -- steps of
     # 0.60 falling to 0.50 ms over the first twenty against 0.47 ms flat -- and a warm-up of a few steps would leave
     # that ramp inside the timed region
     settle(dev)
     side_reps = 30
-    q_ms = event_time_ms(lambda: ops.quant_block(X[None], clamp=True, with_transpose=True), side_reps)
-    q_bytes = 4.0 * M * K  # 2 B read + 1 B int8 + 1 B transposed int8 per element
-    q1_ms = event_time_ms(lambda: ops.quant_block(X[None], clamp=True), side_reps)
-    # a plain device copy of X (64 MiB read + 64 MiB write): the reachable HBM rate on this box,
-    # and the known-size kernel the rocprofv3 FETCH_SIZE / WRITE_SIZE counters are calibrated on
-    X.clone()
-    copy_ms = event_time_ms(lambda: X.clone(), side_reps)
     bf16_fns = (lambda: X @ W.t(), lambda: dY @ W, lambda: dY.t() @ X)
     for f in bf16_fns:
         f()
@@ -338,6 +331,18 @@ def main():
     ops_per_launch = gemms_per_launch * 2.0 * M * N * K
     achieved = ops_per_launch / (avg_ms * 1e-3) / 1e12
 
+    # ---- the activation quantiser and a plain device copy against HBM, behind the steps (memory-bound kernels need the
+    # memory side of the device awake as well, which the steps' own quantisers have seen to)
+    q_bytes = 4.0 * M * K  # 2 B read + 1 B int8 + 1 B transposed int8 per element
+    for _ in range(5):
+        ops.quant_block(X[None], clamp=True, with_transpose=True)
+    q_ms = event_time_ms(lambda: ops.quant_block(X[None], clamp=True, with_transpose=True), side_reps)
+    q1_ms = event_time_ms(lambda: ops.quant_block(X[None], clamp=True), side_reps)
+    # a plain device copy of X (64 MiB read + 64 MiB write): the reachable HBM rate on this box,
+    # and the known-size kernel the rocprofv3 FETCH_SIZE / WRITE_SIZE counters are calibrated on
+    X.clone()
+    copy_ms = event_time_ms(lambda: X.clone(), side_reps)
+
     # HBM-side bytes per GEMM launch: NOT measured by this run.  They come from two rocprofv3 --pmc runs of this
     # command (FETCH_SIZE, WRITE_SIZE), scaled on the device copy above, whose summary is the file named in
     # `traffic_source`; measured for these two schemes
@@ -375,6 +380,7 @@ def main():
         "quant_roofline": {"bound": "hbm", "kernel": "quant_block_kernel<1,true,true>",
                            "achieved": round(q_bytes / (q_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                            "frac": round(q_bytes / (q_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "launch_ms": round(q_ms, 4),
+                           "frac_of_device_copy": round(q_bytes / q_ms / (2.0 * X.numel() * 2 / copy_ms), 4),
                            "bytes_per_launch": int(q_bytes),
                            "note": "launched back to back on X; `in_step` is the same kernel where it runs inside a step (X and dY, behind a GEMM)",
                            "in_step": in_step,
@@ -384,8 +390,8 @@ def main():
         "bf16_matmul_tflops": round(6.0 * M * N * K / (bf16_ms * 1e-3) / 1e12, 1),
         "entry_point_ms_per_step": {k: round(v, 4) for k, v in sorted(per_entry_ms.items())},
         "between_launches_ms_per_step": round(dt * 1e3 - sum(per_entry_ms.values()), 4),
-        "order": f"{SETTLE_MS:.0f} ms of untimed bf16 GEMMs take the device out of its idle clocks, then the secondary measurements (quantiser, "
-                 "bf16 GEMMs, copy, MFMA probe: about 60 ms of GPU work), then the warm-up and the timed steps, then the per-kernel event pass",
+        "order": f"{SETTLE_MS:.0f} ms of untimed bf16 GEMMs take the device out of its idle clocks, then the bf16 GEMMs of the step's shapes and the "
+                 "MFMA probe (about 50 ms of GPU work), then the warm-up and the timed steps, then the per-kernel event pass, the quantiser and the copy",
         "step_issue": "one ti8_linear_fwd_bwd call per step on outputs and a workspace allocated once" if one_call else "entry point by entry point",
         "gemm_kernel_id": gemm_kernel_id, "init_note": init_note,
     }
