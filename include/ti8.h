@@ -333,8 +333,8 @@ int ti8_gemm_i8_nt_multi(const ti8_gemm_problem* problems, int count, int gemm_f
  * its own allocations).  Same kernels on the same operands as the separate entry points, so the same bits:
  *   TI8_SCHEME_BLOCK_CHANNEL   ti8_quant_block_multi(X, dY; q and qT) -> ti8_quant_row_col_t(W) ->
  *                              ti8_gemm_i8_nt_multi(Y, dX, dW)          (3 launches + W's absmax pass)
- *   TI8_SCHEME_DOUBLE_CHANNEL  ti8_quant_row_col_t on X, W, dY (TI8_INV_AMAX_DIV_127) -> three
- *                              ti8_gemm_i8_nt(acc_i32_full = 1)
+ *   TI8_SCHEME_DOUBLE_CHANNEL  ti8_quant_row_col_t on X, W, dY (TI8_INV_AMAX_DIV_127) ->
+ *                              ti8_gemm_i8_nt_multi(Y, dX, dW; acc_i32_full = 1)
  *   X bf16 [T][K] (ldx), W bf16 [N][K] (ldw), dY bf16 [T][N] (lddy)  ->  Y bf16 [T][N], dX bf16 [T][K], dW bf16 [N][K]
  *   T, K, N multiples of 128.  `tokens` (1 <= tokens <= T) = the rows of X and dY that hold data when the caller has
  *   zero-padded them to T rows (padded rows change no absmax and add nothing to dW; pass tokens = T otherwise).  With

@@ -36,7 +36,7 @@ __device__ __forceinline__ float scale_at(const ScaleDesc& d, int64_t batch, int
 }
 
 #ifndef TI8_LOAD_AUX
-#define TI8_LOAD_AUX 0   // cache policy bits of the operand loads (0: default)
+#define TI8_LOAD_AUX 0   // cache policy bits of the operand loads (0: default; sc0, sc1 measured no different, nt slower)
 #endif
 
 // One wave's share of a K tile: NI global->LDS instructions of 64 x 16 bytes; instruction i

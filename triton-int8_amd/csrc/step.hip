@@ -186,7 +186,7 @@ extern "C" int ti8_linear_fwd_bwd(const void* X, int64_t ldx, const void* W, int
         gemm2d(L.x.q, K, L.x.s_row, TI8_SCALE_ROW, 1, 0, L.w.q, K, L.w.s_row, TI8_SCALE_ROW, 1, 0, Y, ldy, T, N, K, 1),
         gemm2d(L.dy.q, N, L.dy.s_row, TI8_SCALE_ROW, 1, 0, L.w.qT, N, L.w.s_col, TI8_SCALE_ROW, 1, 0, dX, lddx, T, K, N, 1),
         gemm2d(L.dy.qT, T, L.dy.s_col, TI8_SCALE_ROW, 1, 0, L.x.qT, T, L.x.s_col, TI8_SCALE_ROW, 1, 0, dW, lddw, N, K, T, 1)};
-    // three launches: the int32 kernel gains nothing from one launch of all three
+    if (one_launch) return ti8_gemm_i8_nt_multi(g, 3, gemm_flags, stream);
     if (int e = one_gemm(g[0], live_rows(K), gemm_flags, stream)) return e;
     if (int e = one_gemm(g[1], live_rows(N), gemm_flags, stream)) return e;
     return one_gemm(g[2], N, gemm_flags, stream);

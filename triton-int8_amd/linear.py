@@ -253,9 +253,8 @@ def pad_tokens(x2, multiple=128):
 
 # Schemes whose whole step (linear_fwd_bwd with more than 256 tokens and output features) runs its three GEMMs as
 # one launch (ops.gemm_i8_nt_multi; same kernels on the same operands, so the same bits as linear_forward +
-# linear_backward).  Measured at 8192 tokens, K = N = 4096: block_channel 0.497 -> 0.482 ms per step; double_channel,
-# which the launch also serves, gains nothing (0.445 -> 0.448) and stays on three launches.
-ONE_LAUNCH_SCHEMES = ("block_channel", "row_block")
+# linear_backward): one launch of persistent workgroups walks the tiles of all three.
+ONE_LAUNCH_SCHEMES = ("block_channel", "row_block", "double_channel")
 
 
 def _one_launch(scheme, hadamard, padded_tokens, out_features):
