@@ -219,6 +219,43 @@ def test_persistent_kernel_wait_variants(T, dev, M, N, K):
         check_sampled_tiles(got[0], Ad[0], sa_blk[0], olin.BLOCK, Bd, sB, oB, g, f"persistent {M}x{N}x{K} B:{oB}", tile=tile)
 
 
+def test_persistent_kernel_on_seeded_random_shapes(T, dev):
+    """Twelve seeded shapes (tile counts below, at and above the CU count, 2 to 68 K tiles, single GEMMs and three of different
+    shapes in one launch): the persistent kernel against one workgroup per tile, bit for bit over NaN-filled outputs."""
+    import random
+    from triton_int8_amd import ops
+    from triton_int8_amd._lib import KERNEL_ONE_TILE, KERNEL_ONE_TILE_MULTI, KERNEL_PERSISTENT_CHAIN, SCALE_BLOCK128, SCALE_ROW
+    rng, g = random.Random(7), make_gen(7)
+
+    def operands(M, N, K, modeB):
+        sB = scales(g, N) if modeB == SCALE_ROW else scales(g, N // 128, K // 128)
+        return dict(A=torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8).to(dev),
+                    B=torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8).to(dev),
+                    sA=scales(g, M // 128, K // 128).to(dev), modeA=SCALE_BLOCK128, sB=sB.to(dev), modeB=modeB)
+
+    ops.GEMM_PATH = "large"
+    try:
+        for it in range(12):
+            M, N = 128 * rng.randint(2, 40), 128 * rng.randint(2, 40)
+            K = 256 * rng.choice([1, 2, 3, 5, 8, 16, 33, 34])
+            if M * N * K > 1.5e11:
+                K = 512
+            ps = [operands(M, N, K, rng.choice([SCALE_ROW, SCALE_BLOCK128]))]
+            if it % 2:
+                ps += [operands(128 * rng.randint(2, 24), 128 * rng.randint(2, 24), 256 * rng.choice([1, 4, 9]), SCALE_ROW),
+                       operands(128 * rng.randint(2, 24), 128 * rng.randint(2, 24), 256 * rng.choice([2, 6, 34]), SCALE_BLOCK128)]
+            outs = {}
+            for persistent in (True, False):
+                ops.GEMM_PERSISTENT = persistent
+                nan = [torch.full((p["A"].shape[0], p["B"].shape[0]), float("nan"), dtype=torch.bfloat16, device=dev) for p in ps]
+                outs[persistent] = ops.gemm_i8_nt_multi([dict(p, out=o) for p, o in zip(ps, nan)])
+                assert T.last_gemm_kernel() in ((KERNEL_PERSISTENT_CHAIN,) if persistent else (KERNEL_ONE_TILE, KERNEL_ONE_TILE_MULTI)), it
+            for a, b, p in zip(outs[True], outs[False], ps):
+                assert torch.equal(a, b) and torch.isfinite(a).all(), (it, tuple(p["A"].shape), tuple(p["B"].shape))
+    finally:
+        ops.GEMM_PATH, ops.GEMM_PERSISTENT = "auto", True
+
+
 def test_config5_skinny_shapes_at_their_own_size(T, dev):
     """Config 5's decode shapes as worded: M = 16 and M = 128 tokens at K = N = 4096, seed 4, every scheme, the whole
     layer step (Y, dX, dW) and the forward-only module against the oracle -- per element for the promoted
