@@ -423,6 +423,12 @@ def test_fused_hadamard_quantisers(T, dev):
     q, s = T.ops.quant_row(xw.to(dev), clamp=True, hadamard128=True)
     qo, so = obf.token_quant(ohad.hadamard128(xw), True)
     assert bits_equal(q, qo) and bits_equal(s, so.flatten())
+    # one scale per row and 128 columns, behind the rotation (every launch shape of the grouped row quantiser)
+    for rows, cols in ((130, 1024), (7, 4096), (3, 16384)):
+        xg = randn_bf16(make_gen(23 + cols), rows, cols)
+        q, s = T.ops.quant_row(xg.to(dev), clamp=False, group=128, eps_add=True, inv_mode=3, hadamard128=True)
+        qo, so = off.tile_quant_additive_eps(ohad.hadamard128(xg)[None], 1)
+        assert bits_equal(q, qo[0]) and bits_equal(s, so[0]), (rows, cols)
 
 
 @pytest.mark.parametrize("R,C", [(128, 128), (384, 256), (1024, 512)])

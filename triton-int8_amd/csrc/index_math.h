@@ -177,6 +177,11 @@ TI8_HD int64_t fwht_t_colblock(int64_t id, int64_t nblocks, int W) {
 TI8_HD int64_t qrow_row(int64_t block, int wave, bool wg_row) { return wg_row ? block : block * 4 + wave; }
 // 16-byte chunk index of load i of thread t (T threads per row)
 TI8_HD int qrow_chunk(int t, int i, int T) { return t + i * T; }
+// The quantisers that rotate 128-element segments first (H128 across 16 lanes x 8 elements) give chunk
+// c ^ (c & 4 ? 3 : 0) of a segment to the lane that would otherwise hold chunk c: a permutation within
+// every aligned group of 16 chunks (its own inverse), under which the partners of all four cross-lane
+// stages are one DPP pattern away.
+TI8_HD int had_chunk(int c) { return c ^ ((c & 4) ? 3 : 0); }
 
 // ---- 128 x 128 tile quantisers (quant.hip) ---------------------------------------------------
 struct TileId {

@@ -132,20 +132,53 @@ __device__ __forceinline__ float absmax8(const uint4& v, float m) {
 
 
 // Value of `v` in another lane of the same row of 16 lanes (DPP: no LDS traffic, and the move
-// folds into the add that consumes it).  CTRL: 0xB1 / 0x4E = quad_perm lane^1 / lane^2,
-// 0x104 / 0x114 = row_shl:4 / row_shr:4 (lane+4 / lane-4), 0x128 = row_ror:8 (lane^8).
+// folds into the instruction that consumes it).  CTRL: 0xB1 / 0x4E = quad_perm lane^1 / lane^2,
+// 0x141 = row_half_mirror (lane^7), 0x128 = row_ror:8 (lane^8).
 template <int CTRL>
 __device__ __forceinline__ float dpp_f32(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
 }
 
 // 128-point Walsh-Hadamard transform of a row segment held as 8 consecutive bf16 per lane by 16
-// consecutive lanes (lane%16 = chunk index): butterflies in the fixed order stride 1, 2, 4 (in
-// registers), 8, 16, 32, 64 (lane xor 1, 2, 4, 8), fp32, un-normalised; one rounding to bf16.
-// A cross-lane stage is (a, b) -> (a + b, a - b) with a in the lane whose bit is clear: the lower
-// lane computes a + partner, the upper one partner - a = partner + (-a), so flipping the sign of
-// the own value in upper lanes (one xor) makes both a single add with a DPP operand.
-__device__ __forceinline__ uint4 fwht128_bf16(const uint4& v, int lane) {
+// consecutive lanes: butterflies in the fixed order stride 1, 2, 4 (in registers), 8, 16, 32, 64
+// (across lanes), fp32, un-normalised; one rounding to bf16.
+//
+// Which lane holds which 16-byte chunk is chosen so that every cross-lane stage is ONE instruction.
+// Lane l (of its row of 16) holds chunk idx::had_chunk(l) = l ^ (l & 4 ? 3 : 0); then the partners
+// of the four stages (chunk ^ 1, ^ 2, ^ 4, ^ 8) sit in lanes l ^ 1, l ^ 2, l ^ 7, l ^ 8, each a single
+// DPP pattern (two quad_perms, row_half_mirror, row_ror:8; there is none for l ^ 4).  A stage is
+// (a, b) -> (a + b, a - b) with a in the lane whose chunk bit is clear; here every lane computes
+// own + sigma * partner with sigma = +1 / -1 for a clear / set chunk bit (an fma with a DPP operand:
+// the product with +-1 is exact, so the one rounding is that of the add or subtract).  The upper
+// lane thereby gets b - a, the NEGATIVE of its result; as both partners of a later stage carry the
+// same number of such flips, the stages stay as they are and a lane ends with all its values
+// multiplied by had_sign(lane) = -1 if its chunk index has an odd number of bits set.  The callers
+// quantise with the scale multiplied by the same sign (exact; absmax does not see signs).
+struct HadLane {
+    float sigma[4];   // per stage: -1 where the lane's chunk has that bit set
+    float sign;       // what the lane's results are multiplied by
+};
+__device__ __forceinline__ HadLane had_lane(int lane) {
+    const int c = idx::had_chunk(lane & 15);
+    HadLane h;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) h.sigma[k] = ((c >> k) & 1) ? -1.0f : 1.0f;
+    h.sign = (__builtin_popcount(c) & 1) ? -1.0f : 1.0f;
+    return h;
+}
+// One cross-lane stage for the 8 values of a lane: A[e] += partner's A[e] * SIGMA, the partner chosen by
+// the DPP pattern.  Written out because the compiler keeps a separate v_mov_b32_dpp in front of an fma.
+// A DPP operand must not be read within two instructions of the vector instruction that wrote it: inside
+// a stage the eight chains are independent (each register was written eight instructions earlier), and
+// the s_nop covers whatever the compiler placed in front of the stage.  All 64 lanes are active here.
+#define TI8_HAD_FMAC(N, PATTERN) "v_fmac_f32_dpp %" #N ", %" #N ", %8 " PATTERN " row_mask:0xf bank_mask:0xf\n\t"
+#define TI8_HAD_STAGE(A, SIGMA, PATTERN)                                                                                     \
+    asm("s_nop 1\n\t" TI8_HAD_FMAC(0, PATTERN) TI8_HAD_FMAC(1, PATTERN) TI8_HAD_FMAC(2, PATTERN) TI8_HAD_FMAC(3, PATTERN)     \
+        TI8_HAD_FMAC(4, PATTERN) TI8_HAD_FMAC(5, PATTERN) TI8_HAD_FMAC(6, PATTERN) TI8_HAD_FMAC(7, PATTERN)                  \
+        : "+v"(A[0]), "+v"(A[1]), "+v"(A[2]), "+v"(A[3]), "+v"(A[4]), "+v"(A[5]), "+v"(A[6]), "+v"(A[7])                     \
+        : "v"(SIGMA))
+
+__device__ __forceinline__ uint4 fwht128_bf16_signed(const uint4& v, const HadLane& hl) {
     float a[8] = {bf16_lo(v.x), bf16_hi(v.x), bf16_lo(v.y), bf16_hi(v.y), bf16_lo(v.z), bf16_hi(v.z), bf16_lo(v.w), bf16_hi(v.w)};
 #pragma unroll
     for (int h = 1; h < 8; h <<= 1)
@@ -156,20 +189,10 @@ __device__ __forceinline__ uint4 fwht128_bf16(const uint4& v, int lane) {
                 a[e] = u + w;
                 a[e + h] = u - w;
             }
-    const uint32_t s1 = (lane & 1) ? 0x80000000u : 0u, s2 = (lane & 2) ? 0x80000000u : 0u;
-    const uint32_t s8 = (lane & 8) ? 0x80000000u : 0u;
-    const bool up4 = (lane & 4) != 0;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        float x = a[e];
-        x = dpp_f32<0xB1>(x) + __uint_as_float(__float_as_uint(x) ^ s1);
-        x = dpp_f32<0x4E>(x) + __uint_as_float(__float_as_uint(x) ^ s2);
-        const float lo = x + dpp_f32<0x104>(x);   // lanes with bit 2 clear: own + lane+4
-        const float hi = dpp_f32<0x114>(x) - x;   // lanes with bit 2 set: lane-4 - own
-        x = up4 ? hi : lo;
-        x = dpp_f32<0x128>(x) + __uint_as_float(__float_as_uint(x) ^ s8);
-        a[e] = x;
-    }
+    TI8_HAD_STAGE(a, hl.sigma[0], "quad_perm:[1,0,3,2]");
+    TI8_HAD_STAGE(a, hl.sigma[1], "quad_perm:[2,3,0,1]");
+    TI8_HAD_STAGE(a, hl.sigma[2], "row_half_mirror");
+    TI8_HAD_STAGE(a, hl.sigma[3], "row_ror:8");
     uint4 o;
     o.x = pack_bf16x2(a[0], a[1]);
     o.y = pack_bf16x2(a[2], a[3]);
@@ -373,7 +396,9 @@ __global__ __launch_bounds__(256) void quant_block_had_kernel(
     const int rb = t % nrb;
     const int b = t / nrb;
     const int tid = threadIdx.x;
-    const int cc = tid & 15, rg = tid >> 4;
+    // chunk of 8 elements along the rotated direction that this lane holds (see fwht128_bf16_signed)
+    const int cc = idx::had_chunk(tid & 15), rg = tid >> 4;
+    const int lc = ALONG_ROWS ? (tid & 15) : cc;   // chunk of the row that this lane loads
 
     const uint16_t* xt = x + b * bsx + (int64_t)rb * 128 * ldx + (int64_t)cb * 128;
     uint4 v[2][4];
@@ -381,7 +406,7 @@ __global__ __launch_bounds__(256) void quant_block_had_kernel(
     for (int h = 0; h < 2; ++h)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-            v[h][j] = *reinterpret_cast<const uint4*>(xt + (int64_t)(h * 64 + rg * 4 + j) * ldx + cc * 8);
+            v[h][j] = *reinterpret_cast<const uint4*>(xt + (int64_t)(h * 64 + rg * 4 + j) * ldx + lc * 8);
 
     if (ALONG_ROWS) {
         // tile[row][chunk ^ (row >> 3)]: the 16 lanes that later read one column from 16 different
@@ -391,7 +416,7 @@ __global__ __launch_bounds__(256) void quant_block_had_kernel(
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const int row = h * 64 + rg * 4 + j;
-                *reinterpret_cast<uint4*>(tile + row * 128 + ((cc ^ (row >> 3)) & 15) * 8) = v[h][j];
+                *reinterpret_cast<uint4*>(tile + row * 128 + ((lc ^ (row >> 3)) & 15) * 8) = v[h][j];
             }
         __syncthreads();
         // now this thread is (transposed row = original column h*64 + rg*4 + j, transposed columns = original rows 8cc..8cc+7)
@@ -409,7 +434,7 @@ __global__ __launch_bounds__(256) void quant_block_had_kernel(
                 v[h][j] = make_uint4(e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16));
             }
     }
-    const int lane = tid & 63;
+    const HadLane hl = had_lane(tid);
     if (SCALE != HAD_BLOCK) {
         // this thread holds, per (h, j), 8 consecutive rows of column h*64 + rg*4 + j of the tile;
         // the 16 lanes with the same rg hold the other rows of that column
@@ -419,7 +444,7 @@ __global__ __launch_bounds__(256) void quant_block_had_kernel(
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const int col = cb * 128 + h * 64 + rg * 4 + j;
-                const uint4 r = fwht128_bf16(v[h][j], lane);
+                const uint4 r = fwht128_bf16_signed(v[h][j], hl);
                 if (SCALE == HAD_COLMAX) {
                     const float m = row16_max(absmax8(r, 0.0f));
                     if (cc == 0) atomicMax(ws + col, __float_as_uint(m));
@@ -427,7 +452,7 @@ __global__ __launch_bounds__(256) void quant_block_had_kernel(
                     const float amax = amax_floor(__uint_as_float(ws[col]), mode.eps_add);
                     const float scale = 127.0f / amax;
                     if (rb == 0 && cc == 0) s[col] = stored_scale(amax, scale, mode);
-                    *reinterpret_cast<uint2*>(qcol + (int64_t)(h * 64 + rg * 4 + j) * ldq) = quant8(r, scale);
+                    *reinterpret_cast<uint2*>(qcol + (int64_t)(h * 64 + rg * 4 + j) * ldq) = quant8(r, scale * hl.sign);
                 }
             }
         return;
@@ -437,13 +462,14 @@ __global__ __launch_bounds__(256) void quant_block_had_kernel(
     for (int h = 0; h < 2; ++h)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            v[h][j] = fwht128_bf16(v[h][j], lane);
+            v[h][j] = fwht128_bf16_signed(v[h][j], hl);
             amax = absmax8(v[h][j], amax);
         }
     amax = block_max_256(amax, red4);
     amax = amax_floor(amax, mode.eps_add);
     const float scale = 127.0f / amax;
     if (tid == 0) s[b * ssb + rb * ssr + cb * ssc] = stored_scale(amax, scale, mode);
+    const float lane_scale = scale * hl.sign;
     // output tile origin: same orientation as x, or transposed
     int8_t* qt = ALONG_ROWS ? q + b * bsq + (int64_t)cb * 128 * ldq + (int64_t)rb * 128
                             : q + b * bsq + (int64_t)rb * 128 * ldq + (int64_t)cb * 128;
@@ -451,7 +477,7 @@ __global__ __launch_bounds__(256) void quant_block_had_kernel(
     for (int h = 0; h < 2; ++h)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-            *reinterpret_cast<uint2*>(qt + (int64_t)(h * 64 + rg * 4 + j) * ldq + cc * 8) = quant8(v[h][j], scale);
+            *reinterpret_cast<uint2*>(qt + (int64_t)(h * 64 + rg * 4 + j) * ldq + cc * 8) = quant8(v[h][j], lane_scale);
 }
 
 // ---------------------------------------------------------------------------------
@@ -473,23 +499,28 @@ __global__ __launch_bounds__(256) void quant_row_kernel(const uint16_t* __restri
     const uint16_t* xr = x + row * ldx;
 
     uint4 v[NLOAD];
+    HadLane hl;
+    if (HAD) hl = had_lane(threadIdx.x);
+    const float lane_sign = HAD ? hl.sign : 1.0f;
 #pragma unroll
     for (int i = 0; i < NLOAD; ++i) {
-        const int c = idx::qrow_chunk(t, i, T);
+        // the 16 chunks of a 128-column group sit in 16 consecutive lanes (T % 16 == 0), with the
+        // rotation in the order that fwht128_bf16_signed wants (cols % 128 == 0 then: the permuted
+        // chunk is inside the row whenever the plain one is)
+        const int c = HAD ? idx::had_chunk(idx::qrow_chunk(t, i, T)) : idx::qrow_chunk(t, i, T);
         v[i] = (c < nchunk) ? *reinterpret_cast<const uint4*>(xr + c * 8) : make_uint4(0, 0, 0, 0);
-        // chunks c, c^1, ... c^15 of a 128-column group sit in 16 consecutive lanes (T % 16 == 0)
-        if (HAD) v[i] = fwht128_bf16(v[i], threadIdx.x & 63);
+        if (HAD) v[i] = fwht128_bf16_signed(v[i], hl);
     }
     int8_t* qr = q + row * ldq;
     if (GROUP16) {
         const int ngrp = cols >> 7;
 #pragma unroll
         for (int i = 0; i < NLOAD; ++i) {
-            const int c = t + i * T;
+            const int c = HAD ? idx::had_chunk(idx::qrow_chunk(t, i, T)) : idx::qrow_chunk(t, i, T);
             const float amax = amax_floor(row16_max(absmax8(v[i], 0.0f)), mode.eps_add);
             const float scale = 127.0f / amax;
             if (c < nchunk) {
-                *reinterpret_cast<uint2*>(qr + c * 8) = quant8(v[i], scale);
+                *reinterpret_cast<uint2*>(qr + c * 8) = quant8(v[i], scale * lane_sign);
                 if ((c & 15) == 0) s[row * ngrp + (c >> 4)] = stored_scale(amax, scale, mode);
             }
         }
@@ -507,8 +538,8 @@ __global__ __launch_bounds__(256) void quant_row_kernel(const uint16_t* __restri
     if (t == 0) s[row] = stored_scale_arith<ARITH>(amax, scale, mode);
 #pragma unroll
     for (int i = 0; i < NLOAD; ++i) {
-        const int c = idx::qrow_chunk(t, i, T);
-        if (c < nchunk) *reinterpret_cast<uint2*>(qr + c * 8) = quant8<ARITH>(v[i], scale);
+        const int c = HAD ? idx::had_chunk(idx::qrow_chunk(t, i, T)) : idx::qrow_chunk(t, i, T);
+        if (c < nchunk) *reinterpret_cast<uint2*>(qr + c * 8) = quant8<ARITH>(v[i], scale * lane_sign);
     }
 }
 
