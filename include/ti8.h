@@ -336,6 +336,7 @@ int ti8_gemm_i8_nt_multi(const ti8_gemm_problem* problems, int count, int gemm_f
  *   TI8_SCHEME_DOUBLE_CHANNEL  ti8_quant_row_col_t on X, W, dY (TI8_INV_AMAX_DIV_127) ->
  *                              ti8_gemm_i8_nt_multi(Y, dX, dW; acc_i32_full = 1)
  *   X bf16 [T][K] (ldx), W bf16 [N][K] (ldw), dY bf16 [T][N] (lddy)  ->  Y bf16 [T][N], dX bf16 [T][K], dW bf16 [N][K]
+ *   All six 16-byte aligned, leading dimensions multiples of 8 elements; every argument is checked before the first launch.
  *   T, K, N multiples of 128.  `tokens` (1 <= tokens <= T) = the rows of X and dY that hold data when the caller has
  *   zero-padded them to T rows (padded rows change no absmax and add nothing to dW; pass tokens = T otherwise).  With
  *   T <= 256 or N <= 256 the GEMMs are launched one by one, as ti8_gemm_i8_nt would launch them (few-rows kernel up to 256

@@ -139,6 +139,33 @@ def test_latency_harness_shape_rules():
     assert torch.equal(T._common.bf16_reference_nt(a, b), torch.matmul(a, b.transpose(-2, -1)))
 
 
+def test_linear_step_validation(lib):
+    """ti8_linear_fwd_bwd rejects bad arguments before it launches anything (no GPU here: a launch would fail differently)."""
+    T_, K, N = 256, 128, 384
+    need = lib.ti8_linear_fwd_bwd_workspace(T_, K, N, 0)
+    assert need > 0 and need % 256 == 0
+    ws = 0x100000   # 256-byte aligned, never dereferenced
+    good = dict(X=FAKE, ldx=K, W=FAKE, ldw=K, dY=FAKE, lddy=N, Y=FAKE, ldy=N, dX=FAKE, lddx=K, dW=FAKE, lddw=K, T=T_, tokens=T_, K=K, N=N,
+                scheme=0, gemm_flags=0, workspace=ws, workspace_bytes=need, stream=None)
+    cases = [(dict(scheme=1), 4, "scheme must be"), (dict(scheme=7), 4, "scheme must be"),
+             (dict(X=None), 1, "required"), (dict(dW=None), 1, "required"),
+             (dict(T=200, tokens=200), 2, "multiples of 128"), (dict(K=100, ldx=128, ldw=128, lddx=128, lddw=128), 2, "multiples of 128"),
+             (dict(N=0), 2, "multiples of 128"),
+             (dict(tokens=0), 2, "tokens must be"), (dict(tokens=T_ + 1), 2, "tokens must be"),
+             (dict(ldx=K - 8), 2, "leading dimension"), (dict(ldy=N - 8), 2, "leading dimension"),
+             (dict(X=FAKE + 8), 3, "16-byte aligned"), (dict(dW=FAKE + 4), 3, "16-byte aligned"), (dict(lddy=N + 4), 3, "16-byte aligned"),
+             (dict(workspace=None), 2, "workspace"), (dict(workspace=ws + 16), 2, "workspace"), (dict(workspace_bytes=need - 1), 2, "workspace"),
+             (dict(gemm_flags=1), 4, "apply here"), (dict(gemm_flags=4), 4, "apply here")]     # TI8_GEMM_STRICT, TI8_GEMM_SKINNY
+    for change, code, msg in cases:
+        a = {**good, **change}
+        rc = lib.ti8_linear_fwd_bwd(*a.values())
+        assert rc == code and msg in lib.ti8_last_error().decode(), (change, rc, lib.ti8_last_error())
+    for scheme in (0, 2):
+        assert lib.ti8_linear_fwd_bwd_workspace(T_, K, N, scheme) > 0
+    for bad in ((T_ + 1, K, N, 0), (T_, 0, N, 0), (T_, K, N, 1), (T_, K, N, -1)):
+        assert lib.ti8_linear_fwd_bwd_workspace(*bad) == -1
+
+
 def test_quant_block_multi_validation(lib):
     """ti8_quant_block_multi takes a host array of operand descriptors; bad ones are rejected before any launch."""
     import triton_int8_amd

@@ -204,6 +204,33 @@ def test_persistent_workgroups_match_one_tile_kernel(T, dev, M, N, K, batch):
             assert_promoted_close(got[b], want, mag, K, f"persistent {M}x{N}x{K} batch {b} modes {mA}/{mB}")
 
 
+def test_output_that_is_only_8_byte_aligned_leaves_the_persistent_kernel(T, dev):
+    """The persistent kernel stores 16 bytes per lane and row; an output that starts 8 bytes off, or whose rows are an odd
+    number of 8-byte units apart, goes to the one-tile kernel (8-byte stores) and gets the same bits."""
+    from triton_int8_amd import ops
+    from triton_int8_amd._lib import KERNEL_ONE_TILE, KERNEL_PERSISTENT_CHAIN, SCALE_BLOCK128, SCALE_ROW
+    M, N, K = 512, 768, 512
+    g = make_gen(4321)
+    A = torch.randint(-127, 128, (1, M, K), generator=g, dtype=torch.int8).to(dev)
+    B = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8).to(dev)
+    sa = (torch.rand(1, M // 128, K // 128, generator=g) * 1e-2 + 1e-4).to(dev)
+    sb = (torch.rand(N, generator=g) * 1e-2 + 1e-4).to(dev)
+    ops.GEMM_PATH = "large"
+    try:
+        want = ops.gemm_i8_nt(A, B, sa, SCALE_BLOCK128, sb, SCALE_ROW)
+        assert T.last_gemm_kernel() == KERNEL_PERSISTENT_CHAIN
+        flat = torch.zeros(M * (N + 4) + 8, dtype=torch.bfloat16, device=dev)
+        shifted = flat[4:4 + M * N].view(1, M, N)                        # 8 bytes off a 16-byte boundary
+        odd_rows = flat[:M * (N + 4)].view(1, M, N + 4)[:, :, :N]        # rows 8 * odd bytes apart
+        for out in (shifted, odd_rows):
+            flat.zero_()
+            got = ops.gemm_i8_nt(A, B, sa, SCALE_BLOCK128, sb, SCALE_ROW, out=out)
+            assert T.last_gemm_kernel() == KERNEL_ONE_TILE
+            assert got.data_ptr() == out.data_ptr() and torch.equal(got, want)
+    finally:
+        ops.GEMM_PATH = "auto"
+
+
 def test_block_quant_of_several_operands_in_one_launch(T, dev):
     """ti8_quant_block_multi = separate ti8_quant_block calls, bit for bit: operands of different shapes,
     with and without the transposed copy, and the layer step that uses it for X and dY."""

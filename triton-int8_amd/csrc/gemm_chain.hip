@@ -499,6 +499,8 @@ bool chain_persistent_supported(const GemmMulti& m) {
         const int nk = m.g[i].K >> 7;
         if (nk < 2 || nk > 256 || (nk & 1) || m.g[i].strict) return false;
         if (m.g[i].sa.mode == TI8_SCALE_ROW_K128 || m.g[i].sb.mode == TI8_SCALE_ROW_K128) return false;
+        // the epilogue stores 16 bytes per lane and row (the one-tile kernels store 8)
+        if ((reinterpret_cast<uintptr_t>(m.g[i].C) & 15) || (m.g[i].ldc % 8) || (m.g[i].bsc % 8)) return false;
         // per-lane offsets into the scale arrays are kept in 32 bits: 64 K blocks x stride, 64 columns x stride
         const int64_t lim = (int64_t)1 << 24;
         if (m.g[i].sa.ks < 0 || m.g[i].sa.ks >= lim || m.g[i].sb.ks < 0 || m.g[i].sb.ks >= lim || m.g[i].sb.rs < 0 || m.g[i].sb.rs >= lim) return false;

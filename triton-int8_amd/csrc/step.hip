@@ -104,6 +104,10 @@ int check_step(const char* fn, const void* X, int64_t ldx, const void* W, int64_
                     (long long)T, (long long)K, (long long)N);
     if (tokens < 1 || tokens > T) return fail(TI8_ERR_SHAPE, "%s: tokens must be in [1, T]; got tokens=%lld T=%lld", fn, (long long)tokens, (long long)T);
     if (ldx < K || ldw < K || lddy < N || ldy < N || lddx < K || lddw < K) return fail(TI8_ERR_SHAPE, "%s: leading dimension smaller than the row length", fn);
+    // what the quantisers (inputs) and the GEMM epilogues (outputs) need, checked here so that nothing is launched before a rejection
+    if (!aligned16(X) || !aligned16(W) || !aligned16(dY) || !aligned16(Y) || !aligned16(dX) || !aligned16(dW) || (ldx % 8) || (ldw % 8) ||
+        (lddy % 8) || (ldy % 8) || (lddx % 8) || (lddw % 8))
+        return fail(TI8_ERR_ALIGN, "%s: X, W, dY, Y, dX and dW must be 16-byte aligned with leading dimensions multiples of 8 elements", fn);
     return TI8_OK;
 }
 
