@@ -1,9 +1,10 @@
 """Oracle of triton/fused_triton_bwd33.py (quantise-inside-the-GEMM, 3-D x 3-D).
 
-TEST INFRASTRUCTURE.  The reference autotunes its tile shapes (:10-23), and
-BLOCK_K in {64, 128} changes the quantisation groups, so its result depends on
-the tuner's pick; this oracle fixes the 128x128x128 configuration that
-``fused_int8_gemm`` names as its intent (:65-67).
+TEST INFRASTRUCTURE.  The reference lists nine tile shapes for its tuner (:10-23), and
+BLOCK_K in {64, 128} would change the quantisation groups; but the host wrapper launches
+ceildiv(M, 128) x ceildiv(N, 128) programs whatever the pick (:66-75), so only the picks with
+BLOCK_M = BLOCK_N = 128 cover the output exactly once, and both have BLOCK_K = 128.  This oracle
+therefore restates the 128x128x128 configuration that ``fused_int8_gemm`` names (:66-68).
 """
 import torch
 
