@@ -296,9 +296,14 @@ def main():
     dt = (time.perf_counter() - t0) / args.steps
     tops = 6.0 * M * N * K / dt / 1e12
 
+    # which GEMM kernel the timed steps ran, read back from the library: `roofline.kernel` is built from it, and for the
+    # block-channel scheme anything but the persistent kernel is a fallback that the line must show
     gemm_kernel_id = T.last_gemm_kernel()
-    if args.scheme == "block_channel":   # the figure below is quoted on the persistent kernel: make sure it is the one that ran
-        assert gemm_kernel_id == _lib.KERNEL_PERSISTENT_CHAIN, f"the persistent GEMM kernel did not run (kernel id {gemm_kernel_id}; {init_note})"
+    kernel = _lib.describe_gemm_kernel()
+    kernel_check = "ok"
+    if args.scheme == "block_channel" and gemm_kernel_id != _lib.KERNEL_PERSISTENT_CHAIN:
+        kernel_check = f"FALLBACK: the persistent GEMM kernel did not run ({init_note}; last error: {_lib.lib().ti8_last_error().decode()!r})"
+        print("bench.py: " + kernel_check, file=sys.stderr, flush=True)
 
     # ---- dominant kernel: the GEMM launches of a step (Y, dX, dW), bracketed by HIP events on the launch stream while
     # whole steps run, in a second pass of K steps (so the events do not sit in the region `value` is timed on).  The
@@ -321,12 +326,10 @@ def main():
         g = [a.elapsed_time(b) for a, b in rec["ti8_gemm_i8_nt_multi"]]
         assert len(g) == ev_steps
         gemm_ms, gemms_per_launch = [sum(g) / ev_steps], 3
-        kernel = "gemm_i8_chain_kernel (persistent workgroups, 256x256 tiles, chained block-channel promotion)"
     else:
         g = [a.elapsed_time(b) for a, b in rec["ti8_gemm_i8_nt"]]
         assert len(g) == 3 * ev_steps
         gemm_ms, gemms_per_launch = [sum(g[i::3]) / ev_steps for i in range(3)], 1
-        kernel = "gemm_i8_kernel<256,256,2,4,EPI_ROWS>" if args.scheme == "double_channel" else "gemm_i8_chain_kernel (persistent workgroups, 256x256 tiles, chained block-channel promotion)"
     avg_ms = sum(gemm_ms) / len(gemm_ms)
     ops_per_launch = gemms_per_launch * 2.0 * M * N * K
     achieved = ops_per_launch / (avg_ms * 1e-3) / 1e12
@@ -393,7 +396,7 @@ def main():
         "order": f"{SETTLE_MS:.0f} ms of untimed bf16 GEMMs take the device out of its idle clocks, then the bf16 GEMMs of the step's shapes and the "
                  "MFMA probe (about 50 ms of GPU work), then the warm-up and the timed steps, then the per-kernel event pass, the quantiser and the copy",
         "step_issue": "one ti8_linear_fwd_bwd call per step on outputs and a workspace allocated once" if one_call else "entry point by entry point",
-        "gemm_kernel_id": gemm_kernel_id, "init_note": init_note,
+        "gemm_kernel_id": gemm_kernel_id, "gemm_kernel_check": kernel_check, "init_note": init_note,
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.scheme)

@@ -139,6 +139,20 @@ def test_latency_harness_shape_rules():
     assert torch.equal(T._common.bf16_reference_nt(a, b), torch.matmul(a, b.transpose(-2, -1)))
 
 
+def test_gemm_kernel_id_text():
+    """The text for a value of ti8_last_gemm_kernel (kind | epilogue << 8 | rows / 64 << 16 | columns / 64 << 20)."""
+    import triton_int8_amd
+    L = triton_int8_amd._lib
+    t = L.describe_gemm_kernel(L.KERNEL_PERSISTENT_CHAIN | 5 << 8 | 4 << 16 | 4 << 20)
+    assert "gemm_i8_chain_kernel" in t and "256x256" in t and "chained" in t
+    t = L.describe_gemm_kernel(L.KERNEL_ONE_TILE_MULTI | 1 << 8 | 4 << 16 | 4 << 20)
+    assert "gemm_i8_multi_kernel" in t and "256x256" in t and "int32 over the whole K" in t
+    t = L.describe_gemm_kernel(L.KERNEL_ONE_TILE | 2 << 8 | 4 << 16 | 2 << 20)
+    assert "gemm_i8_kernel" in t and "256x128" in t
+    assert L.describe_gemm_kernel(L.KERNEL_FEW_ROWS) == "gemm_i8_wavering_kernel (few rows)"
+    assert L.describe_gemm_kernel(0) == "none"
+
+
 def test_linear_step_validation(lib):
     """ti8_linear_fwd_bwd rejects bad arguments before it launches anything (no GPU here: a launch would fail differently)."""
     T_, K, N = 256, 128, 384

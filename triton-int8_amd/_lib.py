@@ -147,6 +147,25 @@ def init():
     return l.ti8_last_error().decode()
 
 
+_EPILOGUES = ("int32 out", "per-row scales, int32 over the whole K", "promotion per K tile", "literal arithmetic",
+              "promotion per K tile, per-lane factors", "chained promotion per K tile")
+_KINDS = {KERNEL_NONE: "none", KERNEL_ONE_TILE: "gemm_i8_kernel (one workgroup per tile)",
+          KERNEL_ONE_TILE_MULTI: "gemm_i8_multi_kernel (one workgroup per tile, several GEMMs per launch)",
+          KERNEL_PERSISTENT_CHAIN: "gemm_i8_chain_kernel (persistent workgroups)",
+          KERNEL_FEW_ROWS: "gemm_i8_wavering_kernel (few rows)"}
+
+
+def describe_gemm_kernel(kernel_id=None):
+    """Text for a value of ``ti8_last_gemm_kernel`` (default: the current one): kernel, tile, epilogue."""
+    if kernel_id is None:
+        kernel_id = lib().ti8_last_gemm_kernel()
+    kind, epi, bm, bn = kernel_id & 0xff, (kernel_id >> 8) & 0xff, ((kernel_id >> 16) & 0xf) * 64, ((kernel_id >> 20) & 0xf) * 64
+    name = _KINDS.get(kind, f"kernel kind {kind}")
+    if kind in (KERNEL_NONE, KERNEL_FEW_ROWS):
+        return name
+    return f"{name}, {bm}x{bn} tiles, {_EPILOGUES[epi] if epi < len(_EPILOGUES) else epi}"
+
+
 def last_gemm_kernel():
     """Kind of the GEMM kernel that the last GEMM entry point called from this thread launched
     (``KERNEL_*``): kernels of one family give the same bits, so this is how a caller tells which ran."""
