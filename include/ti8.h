@@ -273,6 +273,20 @@ int ti8_fwht(const void* x, int64_t ldx, void* y, int64_t ldy,
 int ti8_fwht_t(const void* x, int64_t ldx, void* y, int64_t ldy,
                int64_t R, int64_t C, float scale, ti8_stream_t stream);
 
+/* The full-length rotation and the per-row quantiser behind it in one pass: replaces the pair
+ *   a = hadamard_transform(a); a_q, a_s = triton_per_row_quant_2d/3d(a)
+ * of triton/double-channle_fwd32.py:273-278 and triton/double_channel_bwd33.py:189-194 (there a bf16 tensor written
+ * by one kernel and read back by two more).  Same arithmetic on the same bf16-rounded rotated values, so q and s are
+ * bit-identical to ti8_fwht(scale = 1) followed by ti8_quant_row; the rotated row stays in the workgroup's LDS and
+ * registers, i.e. 3 bytes of HBM traffic per element instead of 7.
+ *   x bf16 [rows][cols] (ldx) -> q int8 [rows][cols] (ldq), s fp32 [rows]
+ *   n = the transform length: cols itself (a power of two, 128 <= n <= 32768), or the next power of two above a
+ *   row that is none (n / 2 < cols < n, zero-extended as in ti8_fwht); cols % 16 == 0.
+ *   qflags: TI8_Q_CLAMP, TI8_Q_EPS_ADD; inv_mode as in ti8_quant_row (the reference's pipelines use
+ *   TI8_INV_AMAX_DIV_127). */
+int ti8_fwht_quant_row(const void* x, int64_t ldx, int8_t* q, int64_t ldq, float* s,
+                       int64_t rows, int64_t cols, int64_t n, int qflags, int inv_mode, ti8_stream_t stream);
+
 /* ---------------------------------------------------------------------------------
  * INT8 NT GEMM with fused dequantising epilogue, C[b] = dequant(A[b] * B[b]^T):
  * replaces triton_gemm + int8_gemm_kernel of every scheme

@@ -49,11 +49,14 @@ struct Report {
 
 extern "C" {
 
-// ti8_fwht -> fwht_kernel<NT> (fwht.hip): bf16 x [rows][cols] (ldx) -> y (ldy)
-int walk_fwht(int64_t ldx, int64_t ldy, int64_t rows, int64_t cols, int64_t n, int64_t x_elems, int64_t y_elems,
-              int64_t lds_bytes_limit, int64_t* n_checked, char* msg, int msglen) {
+// ti8_fwht -> fwht_kernel<NT, false> (fwht.hip): bf16 x [rows][cols] (ldx) -> y (ldy).
+// quant: ti8_fwht_quant_row -> fwht_kernel<NT, true>: one workgroup per row (L = n), int8 q [rows][cols] (ldy = ldq, y_elems
+// = bytes of q) and one fp32 scale per row (s_elems) instead of y
+static int walk_fwht_impl(bool quant, int64_t ldx, int64_t ldy, int64_t rows, int64_t cols, int64_t n, int64_t x_elems, int64_t y_elems,
+                          int64_t s_elems, int64_t lds_bytes_limit, int64_t* n_checked, char* msg, int msglen) {
     Report r{msg, msglen};
-    const int64_t L = fwht_segment_len(cols, n);
+    const int64_t L = quant ? n : fwht_segment_len(cols, n);
+    if (quant && cols > n) r.fail("fwht_quant_row: %lld columns exceed the transform length %lld", (long long)cols, (long long)n);
     const int NT = fwht_threads(L);
     const bool extended = cols < L;             // a zero-extended row per workgroup
     const int valid = (int)(extended ? cols : L);
@@ -83,8 +86,15 @@ int walk_fwht(int64_t ldx, int64_t ldy, int64_t rows, int64_t cols, int64_t n, i
             rem -= rb2;
             if (rem > 0) pass(8 + rb2, rem);
         }
-        for (int c = tid; c < (L >> 3); c += NT) r.access("fwht lds read-back", fwht_padded(c * 8), 8, lds_words, tid, c);
+        if (quant) {   // at most 4 chunks per thread are kept in registers; the first words of LDS then hold one maximum per wave
+            for (int k = 0; k < 4; ++k)
+                if (tid + k * NT < (L >> 3)) r.access("fwht lds read-back", fwht_padded((tid + k * NT) * 8), 8, lds_words, tid, k);
+            r.access("fwht lds wave maxima", tid >> 6, 1, lds_words, tid);
+        } else {
+            for (int c = tid; c < (L >> 3); c += NT) r.access("fwht lds read-back", fwht_padded(c * 8), 8, lds_words, tid, c);
+        }
     }
+    if (quant && (L >> 3) > 4 * NT) r.fail("fwht_quant_row: %lld chunks do not fit 4 per thread on %d threads", (long long)(L >> 3), NT);
     for (int64_t block = 0; block < nblocks && !r.bad; ++block) {
         const int64_t xo = fwht_segment_offset(block, segs_per_row, ldx, (int)L);
         const int64_t yo = fwht_segment_offset(block, segs_per_row, ldy, (int)L);
@@ -95,11 +105,20 @@ int walk_fwht(int64_t ldx, int64_t ldy, int64_t rows, int64_t cols, int64_t n, i
                 r.access("fwht x", xo + vt * 16 + 8, 8, x_elems, block, tid, vt);
             }
             for (int c = tid; c < (L >> 3); c += NT)
-                if (fwht_chunk_valid(c * 8, 8, valid)) r.access("fwht y", yo + c * 8, 8, y_elems, block, tid, c);
+                if (fwht_chunk_valid(c * 8, 8, valid)) r.access(quant ? "fwht q" : "fwht y", yo + c * 8, 8, y_elems, block, tid, c);
+            if (quant && tid == 0) r.access("fwht s", block, 1, s_elems, block);
         }
     }
     *n_checked = r.checked;
     return r.bad;
+}
+int walk_fwht(int64_t ldx, int64_t ldy, int64_t rows, int64_t cols, int64_t n, int64_t x_elems, int64_t y_elems,
+              int64_t lds_bytes_limit, int64_t* n_checked, char* msg, int msglen) {
+    return walk_fwht_impl(false, ldx, ldy, rows, cols, n, x_elems, y_elems, 0, lds_bytes_limit, n_checked, msg, msglen);
+}
+int walk_fwht_quant_row(int64_t ldx, int64_t ldq, int64_t rows, int64_t cols, int64_t n, int64_t x_elems, int64_t q_elems, int64_t s_elems,
+                        int64_t lds_bytes_limit, int64_t* n_checked, char* msg, int msglen) {
+    return walk_fwht_impl(true, ldx, ldq, rows, cols, n, x_elems, q_elems, s_elems, lds_bytes_limit, n_checked, msg, msglen);
 }
 
 // ti8_fwht_t -> fwht_t_kernel<NT, W> (fwht.hip): x bf16 [R][C] (ldx) -> y bf16 [C][R] (ldy)

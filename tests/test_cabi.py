@@ -68,6 +68,17 @@ FAKE = 0x10000  # a 16-byte aligned non-null "device pointer"; validation never 
     (("ti8_quant_row", FAKE, 4096, FAKE, 4096, FAKE, 4, 65536, 0, 0, 0, None), 2, "cols<=32768"),
     (("ti8_quant_row", FAKE, 4096, FAKE, 4096, FAKE, 4, 4096, 64, 0, 0, None), 4, "group"),
     (("ti8_quant_row", FAKE, 4096, FAKE, 4096, FAKE, 4, 4096, 0, 0, 7, None), 4, "inv_mode"),
+    (("ti8_fwht_quant_row", FAKE, 4096, None, 4096, FAKE, 4, 4096, 4096, 1, 1, None), 1, "required"),
+    (("ti8_fwht_quant_row", FAKE, 4096, FAKE, 4096, FAKE, 4, 4096, 3000, 1, 1, None), 2, "power of two"),
+    (("ti8_fwht_quant_row", FAKE, 8192, FAKE, 8192, FAKE, 4, 8192, 4096, 1, 1, None), 2, "cols==n"),       # several transforms per row
+    (("ti8_fwht_quant_row", FAKE, 2048, FAKE, 2048, FAKE, 4, 2048, 4096, 1, 1, None), 2, "cols==n"),       # cols = n / 2: not zero-extended
+    (("ti8_fwht_quant_row", FAKE, 3000, FAKE, 3008, FAKE, 4, 3000, 4096, 1, 1, None), 2, "cols%16"),
+    (("ti8_fwht_quant_row", FAKE, 4096, FAKE, 4096, FAKE, 0, 4096, 4096, 1, 1, None), 2, "rows>0"),
+    (("ti8_fwht_quant_row", FAKE, 4096, FAKE, 4000, FAKE, 4, 4096, 4096, 1, 1, None), 2, "leading dimension"),
+    (("ti8_fwht_quant_row", FAKE + 8, 4096, FAKE, 4096, FAKE, 4, 4096, 4096, 1, 1, None), 3, "aligned"),
+    (("ti8_fwht_quant_row", FAKE, 4096, FAKE, 4096, FAKE, 4, 4096, 4096, 8, 1, None), 4, "apply here"),     # TI8_Q_HAD128
+    (("ti8_fwht_quant_row", FAKE, 4096, FAKE, 4096, FAKE, 4, 4096, 4096, 4, 1, None), 4, "apply here"),     # TI8_Q_SCALE_BF16
+    (("ti8_fwht_quant_row", FAKE, 4096, FAKE, 4096, FAKE, 4, 4096, 4096, 1, 9, None), 4, "inv_mode"),
     (("ti8_quant_col_t", FAKE, 256, FAKE, 128, FAKE, None, 128, 256, 0, 0, None), 1, "required"),
     (("ti8_quant_col_t", FAKE, 256, FAKE, 128, FAKE, FAKE, 100, 256, 0, 0, None), 2, "R%128"),
     (("ti8_quant_row_col_t", FAKE, 256, FAKE, 256, FAKE, FAKE, 128, FAKE, None, 128, 256, 0, 0, None), 1, "required"),

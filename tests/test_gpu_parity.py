@@ -433,6 +433,32 @@ def test_fwht_of_the_transpose(T, dev, R, C):
     assert torch.equal(T.ops.fwht_t(wide[:, 8:8 + C]), y)
 
 
+@pytest.mark.parametrize("cols", [128, 256, 1024, 2048, 4096, 8192, 16384, 32768, 1536, 14336, 28672])
+def test_rotation_and_row_quantiser_in_one_pass(T, dev, cols):
+    """ti8_fwht_quant_row = ti8_fwht followed by ti8_quant_row, bit for bit (the rotated bf16 row never leaves the
+    workgroup), and equal to the oracle's rotate, round to bf16, quantise; powers of two and zero-extended lengths,
+    every scale form, an all-zero row, a row with one huge element."""
+    from triton_int8_amd._lib import INV_AMAX_DIV_127, INV_RCP_OF_SCALE
+    x = randn_bf16(make_gen(900 + cols), 7, cols)
+    x[2] = 0
+    x[4, cols // 3] = 3.0e4
+    xd = x.to(dev)
+    for kw in (dict(clamp=True, inv_mode=INV_AMAX_DIV_127), dict(clamp=True, inv_mode=INV_RCP_OF_SCALE), dict(clamp=False, eps_add=True, inv_mode=INV_RCP_OF_SCALE)):
+        q, s = T.ops.fwht_quant_row(xd, **kw)
+        q2, s2 = T.ops.quant_row(T.ops.fwht(xd), **kw)
+        assert torch.equal(q, q2) and bits_equal(s, s2.cpu()), (cols, kw)
+    q, s = T.ops.fwht_quant_row(xd, clamp=True, inv_mode=INV_AMAX_DIV_127)
+    qo, so = odf.triton_per_row_quant_2d(ohad.hadamard_transform(x), BLOCK_N=128)
+    assert bits_equal(q, qo) and bits_equal(s, so)
+    x3 = xd.reshape(1, 7, cols).expand(2, 7, cols).contiguous()
+    q3, s3 = T.ops.fwht_quant_row(x3, clamp=True, inv_mode=INV_AMAX_DIV_127)
+    assert q3.shape == (2, 7, cols) and s3.shape == (2, 7) and torch.equal(q3[1], q) and torch.equal(s3[0], s)
+    wide = torch.zeros(7, cols + 64, dtype=torch.bfloat16, device=dev)     # a strided view
+    wide[:, 16:16 + cols] = xd
+    qw, sw = T.ops.fwht_quant_row(wide[:, 16:16 + cols], clamp=True, inv_mode=INV_AMAX_DIV_127)
+    assert torch.equal(qw, q) and torch.equal(sw, s)
+
+
 def test_fused_hadamard_quantisers(T, dev):
     """H_128 fused into the quantisers equals the un-fused oracle (rotate, round to bf16, quantise)."""
     x = planted(20, 2, 256, 384)

@@ -37,6 +37,7 @@ def walker(tmp_path_factory):
     i64, ci, cp = ctypes.c_int64, ctypes.c_int, ctypes.c_char_p
     p64 = ctypes.POINTER(ctypes.c_int64)
     lib.walk_fwht.argtypes = [i64] * 8 + [p64, cp, ci]
+    lib.walk_fwht_quant_row.argtypes = [i64] * 9 + [p64, cp, ci]
     lib.walk_fwht_t.argtypes = [i64] * 7 + [p64, cp, ci]
     lib.walk_quant_row.argtypes = [i64] * 4 + [ci] + [i64] * 3 + [p64, cp, ci]
     lib.walk_quant_block.argtypes = [i64, i64, ci, i64, i64, ci, i64, i64, i64, i64, i64, i64, i64, i64, ci, i64, i64, i64, i64, p64, cp, ci]
@@ -92,6 +93,10 @@ def walk(lib, allocs, name, a):
     if name == "ti8_fwht":
         x, ldx, y, ldy, rows, cols, nn = a[:7]
         rc = lib.walk_fwht(ldx, ldy, rows, cols, nn, allocs.room(x, 2), allocs.room(y, 2), LDS_LIMIT, ctypes.byref(n), msg, 512)
+    elif name == "ti8_fwht_quant_row":
+        x, ldx, q, ldq, sc, rows, cols, nn = a[:8]
+        rc = lib.walk_fwht_quant_row(ldx, ldq, rows, cols, nn, allocs.room(x, 2), allocs.room(q, 1), allocs.room(sc, 4), LDS_LIMIT,
+                                     ctypes.byref(n), msg, 512)
     elif name == "ti8_fwht_t":
         x, ldx, y, ldy, R, C = a[:6]
         rc = lib.walk_fwht_t(ldx, ldy, R, C, allocs.room(x, 2), allocs.room(y, 2), LDS_LIMIT, ctypes.byref(n), msg, 512)
@@ -237,6 +242,24 @@ def test_transposed_hadamard_launches(walker, recorded, R, C):
     n = ctypes.c_int64(0)
     assert walker.walk_fwht_t(C, R, R, C, R * C - 1, R * C, LDS_LIMIT, ctypes.byref(n), msg, 512) == 1 and msg.value.split(b":")[0].endswith(b" x")
     assert walker.walk_fwht_t(C, R, R, C, R * C, R * C - 8, LDS_LIMIT, ctypes.byref(n), msg, 512) == 1 and msg.value.split(b":")[0].endswith(b" y")
+
+
+@pytest.mark.parametrize("rows,cols", [(5, 128), (3, 2048), (2, 8192), (2, 14336), (1, 16384), (1, 32768), (2, 28672)])
+def test_rotate_and_quantise_launch(walker, recorded, rows, cols):
+    """ti8_fwht_quant_row as the wrapper launches it: every global and LDS access in bounds, every chunk of a row kept by
+    one thread; and the walker notices an allocation that is too small."""
+    T, allocs, calls = recorded
+    q, s = T.ops.fwht_quant_row(torch.empty(rows, cols, dtype=torch.bfloat16))
+    assert tuple(q.shape) == (rows, cols) and tuple(s.shape) == (rows,) and [c[0] for c in calls] == ["ti8_fwht_quant_row"]
+    nn = 1 << (cols - 1).bit_length()
+    assert calls[0][1][7] == nn
+    assert walk(walker, allocs, *calls[0]) >= rows * cols // 8
+    msg, n = ctypes.create_string_buffer(512), ctypes.c_int64(0)
+    args = lambda x_el, q_el, s_el: (cols, cols, rows, cols, nn, x_el, q_el, s_el, LDS_LIMIT, ctypes.byref(n), msg, 512)
+    assert walker.walk_fwht_quant_row(*args(rows * cols, rows * cols, rows)) == 0
+    assert walker.walk_fwht_quant_row(*args(rows * cols - 8, rows * cols, rows)) == 1 and b"fwht x" in msg.value
+    assert walker.walk_fwht_quant_row(*args(rows * cols, rows * cols - 8, rows)) == 1 and b"fwht q" in msg.value
+    assert walker.walk_fwht_quant_row(*args(rows * cols, rows * cols, rows - 1)) == 1 and b"fwht s" in msg.value
 
 
 @pytest.mark.parametrize("rows,cols", [(3, 96), (5, 1792), (4, 14336), (2, 24576)])

@@ -18,6 +18,7 @@
 // butterfly).
 #include "ti8_common.h"
 #include "index_math.h"
+#include "quant_math.h"
 
 namespace ti8 {
 
@@ -64,11 +65,16 @@ __device__ __forceinline__ void pass_dispatch(float* lds, int L, int p, int rb, 
 }
 
 // NT threads per workgroup: 256, or 1024 for segments of 16384 elements and more (their LDS
-// footprint allows only one or two workgroups per CU, which 256 threads would leave idle)
-template <int NT>
+// footprint allows only one or two workgroups per CU, which 256 threads would leave idle).
+// QUANT: the workgroup's segment is a whole row (L >= cols), and instead of the rotated bf16 row the
+// kernel writes what the per-row quantiser makes of it -- int8 q[row][cols] and the row's scale --
+// with the quantiser's own arithmetic on the same bf16-rounded values: the rotated operand never
+// goes to HBM (3 bytes per element instead of 4 + 3).
+template <int NT, bool QUANT>
 __global__ __launch_bounds__(NT) void fwht_kernel(const uint16_t* __restrict__ x, int64_t ldx,
                                                    uint16_t* __restrict__ y, int64_t ldy, int cols, int logn,
-                                                   int L, float scale) {
+                                                   int L, float scale, int8_t* __restrict__ q, int64_t ldq,
+                                                   float* __restrict__ s, QMode mode) {
     extern __shared__ float lds[];
     const int tid = threadIdx.x;
     // cols < L: one zero-extended row per workgroup (a length that is no power of two, transformed as the next power of
@@ -106,6 +112,47 @@ __global__ __launch_bounds__(NT) void fwht_kernel(const uint16_t* __restrict__ x
             pass_dispatch<NT>(lds, L, 8 + rb2, rem, tid);
             __syncthreads();
         }
+    }
+    if (QUANT) {
+        // a thread's chunks stay in registers (bf16, as they would have been stored) while the row's absmax is reduced
+        constexpr int MAXC = 4;          // L / 8 / NT: 8192 elements on 256 threads, 32768 on 1024
+        uint4 o[MAXC];
+        float amax = 0.0f;
+#pragma unroll
+        for (int k = 0; k < MAXC; ++k) {
+            const int c = tid + k * NT;
+            o[k] = make_uint4(0u, 0u, 0u, 0u);
+            if (c < (L >> 3) && idx::fwht_chunk_valid(c * 8, 8, valid)) {
+                const float* src = lds + padded(c * 8);
+                float f[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) f[e] = src[e];
+                if (scale != 1.0f) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) f[e] = f[e] * scale;
+                }
+                o[k] = make_uint4(pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]), pack_bf16x2(f[6], f[7]));
+                amax = absmax8(o[k], amax);
+            }
+        }
+        __syncthreads();                 // everybody has taken its values out of LDS: its first words now serve the reduction
+        amax = wave_max(amax);
+        if ((tid & 63) == 0) lds[tid >> 6] = amax;
+        __syncthreads();
+        amax = lds[0];
+#pragma unroll
+        for (int w = 1; w < NT / 64; ++w) amax = fmaxf(amax, lds[w]);
+        amax = amax_floor(amax, mode.eps_add);
+        const float mult = 127.0f / amax;
+        const int64_t row = blockIdx.x;
+        if (tid == 0) s[row] = stored_scale(amax, mult, mode);
+        int8_t* qr = q + row * ldq;
+#pragma unroll
+        for (int k = 0; k < MAXC; ++k) {
+            const int c = tid + k * NT;
+            if (c < (L >> 3) && idx::fwht_chunk_valid(c * 8, 8, valid)) *reinterpret_cast<uint2*>(qr + c * 8) = quant8(o[k], mult);
+        }
+        return;
     }
     for (int c = tid; c < (L >> 3); c += NT) {
         if (!idx::fwht_chunk_valid(c * 8, 8, valid)) continue;
@@ -265,8 +312,9 @@ static int prepare_fwht_t() {
 }
 
 static int prepare_fwht() {
-    static OncePerDevice once;
-    const hipError_t e = raise_lds_limit(once, reinterpret_cast<const void*>(fwht_kernel<1024>), FWHT_LDS_LIMIT);
+    static OncePerDevice once, once_quant;
+    hipError_t e = raise_lds_limit(once, reinterpret_cast<const void*>(fwht_kernel<1024, false>), FWHT_LDS_LIMIT);
+    if (e == hipSuccess) e = raise_lds_limit(once_quant, reinterpret_cast<const void*>(fwht_kernel<1024, true>), FWHT_LDS_LIMIT);
     if (e != hipSuccess) return fail(TI8_ERR_HIP, "ti8_fwht: cannot raise the LDS limit: %s", hipGetErrorString(e));
     return TI8_OK;
 }
@@ -339,11 +387,43 @@ extern "C" int ti8_fwht(const void* x, int64_t ldx, void* y, int64_t ldy, int64_
     while ((1LL << logn) < n) ++logn;
     const size_t shmem = (size_t)idx::fwht_lds_words(L) * sizeof(float);
     if (int e = prepare_fwht()) return e;
+    const QMode none = {0, 0, 0, 0};
     if (idx::fwht_threads(L) == 1024)
-        hipLaunchKernelGGL(fwht_kernel<1024>, dim3((unsigned)nblocks), dim3(1024), shmem, static_cast<hipStream_t>(stream),
-                           static_cast<const uint16_t*>(x), ldx, static_cast<uint16_t*>(y), ldy, (int)cols, logn, (int)L, scale);
+        hipLaunchKernelGGL((fwht_kernel<1024, false>), dim3((unsigned)nblocks), dim3(1024), shmem, static_cast<hipStream_t>(stream),
+                           static_cast<const uint16_t*>(x), ldx, static_cast<uint16_t*>(y), ldy, (int)cols, logn, (int)L, scale,
+                           (int8_t*)nullptr, (int64_t)0, (float*)nullptr, none);
     else
-        hipLaunchKernelGGL(fwht_kernel<256>, dim3((unsigned)nblocks), dim3(256), shmem, static_cast<hipStream_t>(stream),
-                           static_cast<const uint16_t*>(x), ldx, static_cast<uint16_t*>(y), ldy, (int)cols, logn, (int)L, scale);
+        hipLaunchKernelGGL((fwht_kernel<256, false>), dim3((unsigned)nblocks), dim3(256), shmem, static_cast<hipStream_t>(stream),
+                           static_cast<const uint16_t*>(x), ldx, static_cast<uint16_t*>(y), ldy, (int)cols, logn, (int)L, scale,
+                           (int8_t*)nullptr, (int64_t)0, (float*)nullptr, none);
     return check_launch("ti8_fwht");
+}
+
+extern "C" int ti8_fwht_quant_row(const void* x, int64_t ldx, int8_t* q, int64_t ldq, float* s, int64_t rows, int64_t cols, int64_t n,
+                                  int qflags, int inv_mode, ti8_stream_t stream) {
+    const char* fn = "ti8_fwht_quant_row";
+    if (!x || !q || !s) return fail(TI8_ERR_NULL, "%s: x, q and s are required", fn);
+    if (n < 128 || n > 32768 || (n & (n - 1))) return fail(TI8_ERR_SHAPE, "%s: n must be a power of two in [128, 32768], got %lld", fn, (long long)n);
+    // the rotation runs over the whole row: cols = n, or a row shorter than n (n / 2 < cols < n) that is transformed zero-extended
+    const bool extended = cols > n / 2 && cols < n;
+    if (rows <= 0 || rows > 0x7fffffffLL || (cols != n && !extended) || cols % 16)
+        return fail(TI8_ERR_SHAPE, "%s: need rows>0 and cols==n, or n/2 < cols < n, with cols%%16==0; got rows=%lld cols=%lld n=%lld", fn, (long long)rows,
+                    (long long)cols, (long long)n);
+    QMode mode;
+    if (int e = parse_mode(qflags, inv_mode, &mode)) return e;
+    if (qflags & (TI8_Q_HAD128 | TI8_Q_SCALE_BF16)) return fail(TI8_ERR_MODE, "%s: only TI8_Q_CLAMP and TI8_Q_EPS_ADD apply here", fn);
+    if (ldx < cols || ldq < cols) return fail(TI8_ERR_SHAPE, "%s: leading dimension smaller than cols", fn);
+    if (!aligned16(x) || !aligned16(q) || (ldx % 8) || (ldq % 16)) return fail(TI8_ERR_ALIGN, "%s: pointers must be 16-byte aligned and strides multiples of 16 bytes", fn);
+    int logn = 0;
+    while ((1LL << logn) < n) ++logn;
+    const int64_t L = n;   // one workgroup per row
+    const size_t shmem = (size_t)idx::fwht_lds_words(L) * sizeof(float);
+    if (int e = prepare_fwht()) return e;
+    if (idx::fwht_threads(L) == 1024)
+        hipLaunchKernelGGL((fwht_kernel<1024, true>), dim3((unsigned)rows), dim3(1024), shmem, static_cast<hipStream_t>(stream),
+                           static_cast<const uint16_t*>(x), ldx, (uint16_t*)nullptr, (int64_t)0, (int)cols, logn, (int)L, 1.0f, q, ldq, s, mode);
+    else
+        hipLaunchKernelGGL((fwht_kernel<256, true>), dim3((unsigned)rows), dim3(256), shmem, static_cast<hipStream_t>(stream),
+                           static_cast<const uint16_t*>(x), ldx, (uint16_t*)nullptr, (int64_t)0, (int)cols, logn, (int)L, 1.0f, q, ldq, s, mode);
+    return check_launch(fn);
 }

@@ -4,7 +4,7 @@ import torch
 from . import ops
 from ._common import calc_diff, need_bf16_out
 from ._lib import SCALE_ROW
-from .double_channel_fwd32 import _row_quant, hadamard_transform
+from .double_channel_fwd32 import _row_quant, hadamard_transform, rotate_and_row_quant
 
 __all__ = ["hadamard_transform", "triton_per_row_quant_3d", "triton_gemm", "int8_gemm_pipeline", "bwd_33",
            "calc_diff"]
@@ -31,12 +31,14 @@ def int8_gemm_pipeline(A_bf, B_bf, out_dtype=torch.bfloat16, hadamard=True):
     """triton/double_channel_bwd33.py:186-201."""
     torch.cuda.set_device(A_bf.device)
     inv_K = 1.0 / A_bf.shape[-1]
-    if hadamard:
-        A_bf = hadamard_transform(A_bf)
-        B_bf = hadamard_transform(B_bf)
-    bn = 2048 if hadamard else 128
-    A_int8, A_scale = triton_per_row_quant_3d(A_bf, BLOCK_N=bn)
-    B_int8, B_scale = triton_per_row_quant_3d(B_bf, BLOCK_N=bn)
+    if A_bf.dim() != 3 or B_bf.dim() != 3:
+        raise ValueError("A_bf must be [B, M, K] and B_bf [B, N, K]")
+    if hadamard:   # rotation + quantiser fused: one read of each operand
+        A_int8, A_scale = rotate_and_row_quant(A_bf)
+        B_int8, B_scale = rotate_and_row_quant(B_bf)
+    else:
+        A_int8, A_scale = triton_per_row_quant_3d(A_bf, BLOCK_N=128)
+        B_int8, B_scale = triton_per_row_quant_3d(B_bf, BLOCK_N=128)
     return triton_gemm(A_int8, B_int8, A_scale, B_scale, out_dtype=out_dtype,
                        post_scale=inv_K if hadamard else 0.0)
 

@@ -14,7 +14,7 @@ from . import ops
 from ._common import calc_diff, need_bf16_out
 from ._lib import INV_AMAX_DIV_127, SCALE_ROW
 
-__all__ = ["hadamard_transform", "triton_per_row_quant_2d", "triton_per_row_quant_3d", "triton_gemm",
+__all__ = ["hadamard_transform", "rotate_and_row_quant", "triton_per_row_quant_2d", "triton_per_row_quant_3d", "triton_gemm",
            "int8_gemm_pipeline", "fwd_32", "calc_diff"]
 
 
@@ -35,6 +35,14 @@ def _row_quant(x, BLOCK_N):
     if x.shape[-1] % int(BLOCK_N) != 0:
         raise ValueError(f"last dim {x.shape[-1]} is not a multiple of BLOCK_N={BLOCK_N}")
     return ops.quant_row(x, clamp=True, inv_mode=INV_AMAX_DIV_127)
+
+
+def rotate_and_row_quant(x, BLOCK_N=2048):
+    """``triton_per_row_quant_2d/3d(hadamard_transform(x))`` (triton/double-channle_fwd32.py:273-278) in one pass over
+    ``x``: the rotated bf16 tensor, which the reference writes once and reads twice, stays on chip.  Same bits."""
+    if x.shape[-1] % int(BLOCK_N) != 0:
+        raise ValueError(f"last dim {x.shape[-1]} is not a multiple of BLOCK_N={BLOCK_N}")
+    return ops.fwht_quant_row(x, clamp=True, inv_mode=INV_AMAX_DIV_127)
 
 
 def triton_per_row_quant_2d(x: torch.Tensor, BLOCK_N: int = 2048):
@@ -65,11 +73,14 @@ def int8_gemm_pipeline(A_bf, B_bf, out_dtype=torch.bfloat16, hadamard=True):
     its 1/K factor (needed when K is not a power of two)."""
     torch.cuda.set_device(A_bf.device)
     inv_K = 1.0 / A_bf.shape[-1]
-    if hadamard:
-        A_bf = hadamard_transform(A_bf)
-        B_bf = hadamard_transform(B_bf)
-    A_int8, A_scale = triton_per_row_quant_3d(A_bf, BLOCK_N=2048 if hadamard else 128)
-    B_int8, B_scale = triton_per_row_quant_2d(B_bf, BLOCK_N=2048 if hadamard else 128)
+    if A_bf.dim() != 3 or B_bf.dim() != 2:
+        raise ValueError("A_bf must be [B, M, K] and B_bf [N, K]")
+    if hadamard:   # rotation + quantiser fused: one read of each operand
+        A_int8, A_scale = rotate_and_row_quant(A_bf)
+        B_int8, B_scale = rotate_and_row_quant(B_bf)
+    else:
+        A_int8, A_scale = triton_per_row_quant_3d(A_bf, BLOCK_N=128)
+        B_int8, B_scale = triton_per_row_quant_2d(B_bf, BLOCK_N=128)
     return triton_gemm(A_int8, B_int8, A_scale, B_scale, out_dtype=out_dtype,
                        post_scale=inv_K if hadamard else 0.0)
 

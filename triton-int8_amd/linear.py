@@ -102,6 +102,14 @@ def _row_col(x, **kw):
     return q, s, qT, sT
 
 
+def _rotated_row_quant(x, hadamard):
+    """The double-channel scheme's per-row quantiser, behind the full-length rotation when ``hadamard`` is "full" (one
+    pass: the rotated bf16 tensor is not written)."""
+    if hadamard == "full":
+        return ops.fwht_quant_row(x, clamp=True, inv_mode=INV_AMAX_DIV_127)
+    return ops.quant_row(x, clamp=True, inv_mode=INV_AMAX_DIV_127)
+
+
 def quantize_weight(W, scheme="block_channel", hadamard=None):
     """The forward GEMM's view of W [N, K]: ``(Wq int8 [N, K], scales)`` in the scheme's layout (per
     output channel, or 128x128 blocks for "row_block"; rotated first when ``hadamard`` asks).
@@ -113,7 +121,7 @@ def quantize_weight(W, scheme="block_channel", hadamard=None):
     if scheme == "row_block":
         wq, ws = ops.quant_block_had128(W[None], clamp=True) if hadamard == 128 else ops.quant_block(W[None], clamp=True)
         return wq[0], ws[0]
-    return ops.quant_row(ops.fwht(W) if hadamard == "full" else W, clamp=True, inv_mode=INV_AMAX_DIV_127)
+    return _rotated_row_quant(W, hadamard)
 
 
 def linear_forward(X2, W, scheme="block_channel", hadamard=None, need_backward=True, wq=None, tokens=None, xq=None, gemms=None):
@@ -153,7 +161,7 @@ def linear_forward(X2, W, scheme="block_channel", hadamard=None, need_backward=T
     # double_channel
     K = X2.shape[1]
     if hadamard == "full" or not need_backward:
-        q, s = ops.quant_row(ops.fwht(X2) if hadamard == "full" else X2, clamp=True, inv_mode=INV_AMAX_DIV_127)
+        q, s = _rotated_row_quant(X2, hadamard)
         wq, ws = wq if wq is not None else quantize_weight(W, scheme, hadamard)
         return _gemm_dc(q, s, wq, ws, 1.0 / K if hadamard == "full" else 0.0, tokens=tokens, gemms=gemms), saved
     q, s, saved["XtQ"], saved["Xts"] = _row_col(X2, clamp=True, inv_mode=INV_AMAX_DIV_127)
@@ -216,7 +224,7 @@ def linear_backward(dY2, X2, W, scheme="block_channel", hadamard=None, saved=Non
         # the transposed operands are rotated along the rows of the tensors as they lie in memory (ops.fwht_t):
         # no bf16 transpose of W, dY or X.  A length that is no power of two is rotated as the reference's external
         # library rotates it (zero-extended to the next power of two and cut back, through a transposed copy)
-        dq, ds = ops.quant_row(ops.fwht(dY2), clamp=True, inv_mode=INV_AMAX_DIV_127)
+        dq, ds = _rotated_row_quant(dY2, "full")
         wtq, wts = ops.quant_row(ops.fwht_t(W), clamp=True, inv_mode=INV_AMAX_DIV_127)
         dX = _gemm_dc(dq, ds, wtq, wts, 1.0 / N, tokens=tokens, gemms=gemms)
         dytq, dyts = ops.quant_row(ops.fwht_t(dY2), clamp=True, inv_mode=INV_AMAX_DIV_127)

@@ -276,6 +276,26 @@ def fwht(x, n=None, scale=1.0):
     return y.reshape(x.shape)
 
 
+def fwht_quant_row(x, *, clamp=True, eps_add=False, inv_mode=INV_RCP_OF_SCALE):
+    """``quant_row(fwht(x))`` in one pass over ``x`` (bf16 [..., cols], the rotation over the whole last dim, zero-extended
+    when ``cols`` is no power of two): the rotated bf16 tensor is never written.  Returns ``(q, s)``, the same bits."""
+    _check_bf16(x, "x")
+    _need(x.dim() >= 1 and x.numel() > 0, "x must be a non-empty tensor")
+    cols = x.shape[-1]
+    n = 1 << max(cols - 1, 1).bit_length()
+    _need(128 <= n <= 32768 and cols % 128 == 0, f"the last dim must be a multiple of 128 in (64, 32768], got {cols}")
+    x2 = x.reshape(-1, cols)
+    if x2.stride(1) != 1 or x2.stride(0) % 8 or x2.data_ptr() % 16:
+        x2 = x2.contiguous()
+    rows = x2.shape[0]
+    q = torch.empty((rows, cols), dtype=torch.int8, device=x.device)
+    s = torch.empty((rows,), dtype=torch.float32, device=x.device)
+    _lib.call("ti8_fwht_quant_row", x2.data_ptr(), x2.stride(0), q.data_ptr(), cols, s.data_ptr(), rows, cols, n,
+              _qflags(clamp, eps_add, False), inv_mode, _stream())
+    lead = x.shape[:-1]
+    return q.reshape(*lead, cols), s.reshape(*lead)
+
+
 def fwht_t(x, scale=1.0):
     """Walsh-Hadamard transform of ``x.T`` along its rows, i.e. along the ROWS of ``x`` [R, C], without
     the bf16 transpose: returns y [C, R] = ``fwht(x.T.contiguous())``, bit for bit."""
