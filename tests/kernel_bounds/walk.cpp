@@ -67,9 +67,15 @@ static int walk_fwht_impl(bool quant, int64_t ldx, int64_t ldy, int64_t rows, in
     while ((1LL << logn) < n) ++logn;
     const int segs_per_row = extended ? 1 : (int)(cols / L);
     // LDS indices do not depend on the workgroup: walk them once
+    // segments of 1024 elements and more run bits 4..9 across the lanes of a wave (lane l of a row of 16 takes chunk
+    // had_chunk(l)); that needs whole waves of chunks
+    const bool by_lanes = L >= 1024;
+    if (by_lanes && ((L >> 4) % 64)) r.fail("fwht: %lld chunks are not whole waves", (long long)(L >> 4));
     for (int tid = 0; tid < NT && !r.bad; ++tid) {
-        for (int vt = tid; vt < (L >> 4); vt += NT)
+        for (int v0 = tid; v0 < (L >> 4); v0 += NT) {
+            const int vt = by_lanes ? ((v0 & ~15) | had_chunk(v0 & 15)) : v0;
             for (int e = 0; e < 16; ++e) r.access("fwht lds first pass", vt * 17 + e, 1, lds_words, tid, vt, e);
+        }
         auto pass = [&](int p, int rb) {   // pass_in_lds<RB, NT>
             const int ngroups = (int)(L >> rb);
             for (int vt = tid; vt < ngroups; vt += NT) {
@@ -77,14 +83,18 @@ static int walk_fwht_impl(bool quant, int64_t ldx, int64_t ldy, int64_t rows, in
                 for (int e = 0; e < (1 << rb); ++e) r.access("fwht lds pass", fwht_padded(base + (e << p)), 1, lds_words, tid, vt, e, p);
             }
         };
-        const int rb1 = imin(4, logn - 4);
-        pass(4, rb1);
-        int rem = logn - 8;
-        if (rem > 0) {
-            const int rb2 = rem <= 5 ? rem : (rem + 1) / 2;
-            pass(8, rb2);
-            rem -= rb2;
-            if (rem > 0) pass(8 + rb2, rem);
+        if (by_lanes) {
+            if (logn - 10 > 0) pass(10, logn - 10);
+        } else {
+            const int rb1 = imin(4, logn - 4);
+            pass(4, rb1);
+            int rem = logn - 8;
+            if (rem > 0) {
+                const int rb2 = rem <= 5 ? rem : (rem + 1) / 2;
+                pass(8, rb2);
+                rem -= rb2;
+                if (rem > 0) pass(8 + rb2, rem);
+            }
         }
         if (quant) {   // at most 4 chunks per thread are kept in registers; the first words of LDS then hold one maximum per wave
             for (int k = 0; k < 4; ++k)
@@ -99,7 +109,8 @@ static int walk_fwht_impl(bool quant, int64_t ldx, int64_t ldy, int64_t rows, in
         const int64_t xo = fwht_segment_offset(block, segs_per_row, ldx, (int)L);
         const int64_t yo = fwht_segment_offset(block, segs_per_row, ldy, (int)L);
         for (int tid = 0; tid < NT; ++tid) {
-            for (int vt = tid; vt < (L >> 4); vt += NT) {   // two 16-byte loads: elements vt*16 .. +16
+            for (int v0 = tid; v0 < (L >> 4); v0 += NT) {   // two 16-byte loads: elements vt*16 .. +16
+                const int vt = by_lanes ? ((v0 & ~15) | had_chunk(v0 & 15)) : v0;
                 if (!fwht_chunk_valid(vt * 16, 16, valid)) continue;
                 r.access("fwht x", xo + vt * 16, 8, x_elems, block, tid, vt);
                 r.access("fwht x", xo + vt * 16 + 8, 8, x_elems, block, tid, vt);

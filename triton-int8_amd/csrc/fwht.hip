@@ -7,8 +7,12 @@
 // passes: in a pass over index bits [p, p+r) a thread gathers the 2^r elements that
 // differ only in those bits, does the butterflies in registers and hands them on through
 // LDS (fp32).  The first pass (bits 0..3) takes its 16 consecutive elements straight from
-// global memory; the passes are bits 0..3, 4..7 and then the remaining bits in one pass
-// (up to 5 bits) or two.
+// global memory.  Segments of 1024 elements and more then run bits 4..9 across the 64 lanes of
+// a wave (DPP and lane-swap instructions, no LDS) and what is left (up to 5 bits) in one pass
+// through LDS: two LDS round trips and three barriers per row instead of three or four and
+// four or five.  Shorter segments go through LDS after bits 0..3: bits 4..7, then the rest.
+// The kernel is bound by the vector unit, not by HBM: 13 butterfly stages at n = 8192 are 13
+// fp32 adds per element before any conversion or addressing (packed fp32 is not used).
 //
 // LDS index i lives at word i + i/16.  With that padding a wave's 64 accesses of one
 // instruction fall into 64 different banks in every pass: stride 17 in the first pass,
@@ -64,6 +68,69 @@ __device__ __forceinline__ void pass_dispatch(float* lds, int L, int p, int rb, 
     }
 }
 
+// ---- stages over index bits 4..9 without LDS: the 16-element chunks of 1024 consecutive elements sit in the 64 lanes
+// of a wave.  Bits 4..7 pair lanes of one row of 16: with chunk idx::had_chunk(l) in lane l of its row the partners are
+// lanes l ^ 1, l ^ 2, l ^ 7, l ^ 8, one DPP pattern each, and a stage is own + sigma * partner (sigma = -1 where the
+// chunk has the bit set: an fma whose product is exact, rounded once like the add or subtract it stands for).  That
+// leaves the upper lane of a pair with the negative of its result; both partners of every later stage carry the same
+// number of such flips, so nothing else changes and the lane multiplies by its sign (-1 for an odd number of set bits
+// among the stages that ran) at the end.  Bits 8 and 9 pair lanes 16 and 32 apart: v_permlane16_swap / v_permlane32_swap
+// of a register with its copy hand every lane the lower lane's value in one register and the upper lane's in the other,
+// so both lanes compute lower + sigma * upper, with the true sign.
+struct LaneStages {
+    float sigma[6];   // per stage: -1 in lanes whose chunk has the stage's bit set
+    float sign;       // what the DPP stages that ran have multiplied the lane's values by
+};
+__device__ __forceinline__ LaneStages lane_stages(int lane, int nstages) {
+    const int c = idx::had_chunk(lane & 15) | (lane & 48);
+    LaneStages st;
+#pragma unroll
+    for (int k = 0; k < 6; ++k) st.sigma[k] = ((c >> k) & 1) ? -1.0f : 1.0f;
+    const int ran = c & 15 & ((1 << (nstages < 4 ? nstages : 4)) - 1);
+    st.sign = (__builtin_popcount(ran) & 1) ? -1.0f : 1.0f;
+    return st;
+}
+// A[e] += (A[e] of the partner lane) * SIGMA for 16 registers.  A DPP operand must not be read within two instructions of
+// the vector instruction that wrote it: inside the block every register was written 16 instructions earlier, and the
+// s_nop covers whatever the compiler placed in front.  All 64 lanes are active where this is used.
+#define TI8_FWHT_FMAC(N, PATTERN) "v_fmac_f32_dpp %" #N ", %" #N ", %16 " PATTERN " row_mask:0xf bank_mask:0xf\n\t"
+#define TI8_FWHT_DPP_STAGE(A, SIGMA, PATTERN)                                                                                   \
+    asm("s_nop 1\n\t" TI8_FWHT_FMAC(0, PATTERN) TI8_FWHT_FMAC(1, PATTERN) TI8_FWHT_FMAC(2, PATTERN) TI8_FWHT_FMAC(3, PATTERN)    \
+        TI8_FWHT_FMAC(4, PATTERN) TI8_FWHT_FMAC(5, PATTERN) TI8_FWHT_FMAC(6, PATTERN) TI8_FWHT_FMAC(7, PATTERN)                 \
+        TI8_FWHT_FMAC(8, PATTERN) TI8_FWHT_FMAC(9, PATTERN) TI8_FWHT_FMAC(10, PATTERN) TI8_FWHT_FMAC(11, PATTERN)               \
+        TI8_FWHT_FMAC(12, PATTERN) TI8_FWHT_FMAC(13, PATTERN) TI8_FWHT_FMAC(14, PATTERN) TI8_FWHT_FMAC(15, PATTERN)             \
+        : "+v"(A[0]), "+v"(A[1]), "+v"(A[2]), "+v"(A[3]), "+v"(A[4]), "+v"(A[5]), "+v"(A[6]), "+v"(A[7]), "+v"(A[8]),           \
+          "+v"(A[9]), "+v"(A[10]), "+v"(A[11]), "+v"(A[12]), "+v"(A[13]), "+v"(A[14]), "+v"(A[15])                              \
+        : "v"(SIGMA))
+
+// the stages over bits 4 .. 4 + nstages - 1 (nstages <= 6) on the 16 elements of this lane's chunk
+__device__ __forceinline__ void lane_butterflies(float (&a)[16], const LaneStages& st, int nstages) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    if (nstages > 0) TI8_FWHT_DPP_STAGE(a, st.sigma[0], "quad_perm:[1,0,3,2]");
+    if (nstages > 1) TI8_FWHT_DPP_STAGE(a, st.sigma[1], "quad_perm:[2,3,0,1]");
+    if (nstages > 2) TI8_FWHT_DPP_STAGE(a, st.sigma[2], "row_half_mirror");
+    if (nstages > 3) TI8_FWHT_DPP_STAGE(a, st.sigma[3], "row_ror:8");
+#pragma unroll
+    for (int e = 0; e < 16; ++e) a[e] = a[e] * st.sign;
+    if (nstages > 4) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const int v = __float_as_int(a[e]);
+            const auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+            a[e] = __builtin_fmaf(__int_as_float(r[1]), st.sigma[4], __int_as_float(r[0]));
+        }
+    }
+    if (nstages > 5) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const int v = __float_as_int(a[e]);
+            const auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+            a[e] = __builtin_fmaf(__int_as_float(r[1]), st.sigma[5], __int_as_float(r[0]));
+        }
+    }
+#endif
+}
+
 // NT threads per workgroup: 256, or 1024 for segments of 16384 elements and more (their LDS
 // footprint allows only one or two workgroups per CU, which 256 threads would leave idle).
 // QUANT: the workgroup's segment is a whole row (L >= cols), and instead of the rotated bf16 row the
@@ -84,8 +151,35 @@ __global__ __launch_bounds__(NT) void fwht_kernel(const uint16_t* __restrict__ x
     const uint16_t* xr = x + idx::fwht_segment_offset(blockIdx.x, segs_per_row, ldx, L);
     uint16_t* yr = y + idx::fwht_segment_offset(blockIdx.x, segs_per_row, ldy, L);
 
+    // Segments of 1024 elements and more: bits 0..3 in registers and bits 4..9 across the lanes of a wave, whose 64 lanes
+    // hold 64 consecutive chunks (in the order lane_stages wants), then one pass through LDS for what is left.
+    const bool by_lanes = L >= 1024;
+    if (by_lanes) {
+        const int nstages = min(6, logn - 4);
+        const LaneStages st = lane_stages(tid & 63, nstages);
+        for (int v0 = tid; v0 < (L >> 4); v0 += NT) {   // L / 16 is a multiple of 64: whole waves
+            const int vt = (v0 & ~15) | idx::had_chunk(v0 & 15);
+            const bool in = idx::fwht_chunk_valid(vt * 16, 16, valid);
+            const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
+            const uint4 v0q = in ? *reinterpret_cast<const uint4*>(xr + vt * 16) : zero4;
+            const uint4 v1q = in ? *reinterpret_cast<const uint4*>(xr + vt * 16 + 8) : zero4;
+            float a[16] = {bf16_lo(v0q.x), bf16_hi(v0q.x), bf16_lo(v0q.y), bf16_hi(v0q.y), bf16_lo(v0q.z), bf16_hi(v0q.z),
+                           bf16_lo(v0q.w), bf16_hi(v0q.w), bf16_lo(v1q.x), bf16_hi(v1q.x), bf16_lo(v1q.y), bf16_hi(v1q.y),
+                           bf16_lo(v1q.z), bf16_hi(v1q.z), bf16_lo(v1q.w), bf16_hi(v1q.w)};
+            butterflies<4>(a);
+            lane_butterflies(a, st, nstages);
+#pragma unroll
+            for (int e = 0; e < 16; ++e) lds[vt * 17 + e] = a[e];   // = padded(16 vt + e)
+        }
+        __syncthreads();
+        const int rem = logn - 10;
+        if (rem > 0) {
+            pass_dispatch<NT>(lds, L, 10, rem, tid);
+            __syncthreads();
+        }
+    }
     // pass over bits 0..3 (n >= 128, so all four stages belong to every group)
-    for (int vt = tid; vt < (L >> 4); vt += NT) {
+    for (int vt = tid; vt < (by_lanes ? 0 : (L >> 4)); vt += NT) {
         const bool in = idx::fwht_chunk_valid(vt * 16, 16, valid);   // valid is a multiple of 16: a chunk is inside or outside
         const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
         const uint4 v0 = in ? *reinterpret_cast<const uint4*>(xr + vt * 16) : zero4;
@@ -97,12 +191,14 @@ __global__ __launch_bounds__(NT) void fwht_kernel(const uint16_t* __restrict__ x
 #pragma unroll
         for (int e = 0; e < 16; ++e) lds[vt * 17 + e] = a[e];   // = padded(16 vt + e)
     }
-    __syncthreads();
+    if (!by_lanes) __syncthreads();
     // bits 4..7 (4..6 when n = 128)
     const int rb1 = min(4, logn - 4);
-    pass_dispatch<NT>(lds, L, 4, rb1, tid);
-    __syncthreads();
-    int rem = logn - 8;
+    if (!by_lanes) {
+        pass_dispatch<NT>(lds, L, 4, rb1, tid);
+        __syncthreads();
+    }
+    int rem = by_lanes ? 0 : logn - 8;
     if (rem > 0) {
         const int rb2 = rem <= 5 ? rem : (rem + 1) / 2;
         pass_dispatch<NT>(lds, L, 8, rb2, tid);
