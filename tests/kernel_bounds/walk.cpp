@@ -290,7 +290,7 @@ int walk_gemm(int64_t bsa, int64_t lda, int64_t bsb, int64_t ldb, int64_t bsc, i
     const int BM = cfg.bm, BN = cfg.bn, WM = cfg.wm, WN = cfg.wn, EPI = cfg.epi;
     const int NW = WM * WN, TM = BM / WM / 32, TN = BN / WN / 32, A_INSTR = BM / 8 / NW, B_INSTR = BN / 8 / NW;
     const int A_BYTES = BM * 128, B_BYTES = BN * 128;
-    const bool CHAIN = EPI == 5, LANEB = EPI == 4, FAST = EPI == 2 || EPI == 4 || EPI == 5;
+    const bool CHAIN = EPI == 5 || EPI == 6, LANEB = EPI == 4 || EPI == 6, FAST = EPI == 2 || EPI == 4 || CHAIN;
     const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
     const int nk = (int)(K >> 7), klast = (nk - 1) * 128;
     const int WCOLS = TN * 32, LPR = WCOLS / 8, RPI = 64 / LPR, NRR = 32 / RPI;

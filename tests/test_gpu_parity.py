@@ -204,6 +204,47 @@ def test_persistent_workgroups_match_one_tile_kernel(T, dev, M, N, K, batch):
             assert_promoted_close(got[b], want, mag, K, f"persistent {M}x{N}x{K} batch {b} modes {mA}/{mB}")
 
 
+@pytest.mark.parametrize("M,N,K,batch", [(256, 256, 256, 1), (512, 768, 1024, 2), (384, 640, 8192, 1), (256, 512, 16640, 1)])
+def test_per_column_factors_on_large_tiles(T, dev, M, N, K, batch):
+    """Operand B scaled per (row, 128-wide K group), the fused forward's layout: the 256 x 256-tile kernel with the chained
+    promotion (this lane's column factor fetched one K tile ahead) against the 256 x 128-tile kernel bit for bit, both ways
+    of combining the scales, and against the oracle per element; tiles that hang over M and N, 2 to 130 K tiles."""
+    from triton_int8_amd import ops
+    from triton_int8_amd._lib import COMBINE_DIV_PROD, COMBINE_MUL_PROD, KERNEL_ONE_TILE, SCALE_BLOCK128, SCALE_ROW_K128
+    g = make_gen(M * 3 + N + K)
+    A = torch.randint(-127, 128, (batch, M, K), generator=g, dtype=torch.int8)
+    B = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+    sa = torch.rand(batch, M // 128, K // 128, generator=g) * 1e-2 + 1e-4
+    sb = torch.rand(N, K // 128, generator=g) * 1e-2 + 1e-4
+    args = (A.to(dev), B.to(dev), sa.to(dev), SCALE_BLOCK128, sb.to(dev), SCALE_ROW_K128)
+
+    def run(path, **kw):
+        ops.GEMM_PATH = path
+        try:
+            out = ops.gemm_i8_nt(*args, **kw)
+            ident = T._lib.lib().ti8_last_gemm_kernel()
+            assert ident & 0xff == KERNEL_ONE_TILE
+            return out, (ident >> 8) & 0xff, ((ident >> 16) & 0xf) * 64, ((ident >> 20) & 0xf) * 64
+        finally:
+            ops.GEMM_PATH = "auto"
+
+    for combine in (COMBINE_MUL_PROD, COMBINE_DIV_PROD):
+        big, epi, bm, bn = run("large", combine=combine)
+        assert (epi, bm, bn) == (6, 256, 256)
+        small, epi, bm, bn = run("tiled", combine=combine)
+        assert (epi, bm, bn) == (4, 256, 128)
+        assert torch.equal(big, small), (M, N, K, combine)
+    got, _, _, _ = run("large", combine=COMBINE_DIV_PROD)
+    want = off.fused_gemm_from_quant(A, sa, B[None], sb[None], 1)        # acc += f32(dot) / (sa * sb) per K group
+    assert rel_err(got, want) <= FAST_TOL
+    for b in (0, batch - 1):
+        mag = torch.zeros(M, N, dtype=torch.float64)                      # sum over the K groups of |term|
+        for kb in range(K // 128):
+            d = A[b, :, kb * 128:(kb + 1) * 128].double() @ B[:, kb * 128:(kb + 1) * 128].double().t()
+            mag += d.abs() / (sa[b, :, kb].double().repeat_interleave(128)[:, None] * sb[:, kb].double()[None, :])
+        assert_promoted_close(got[b], want[b], mag.float(), K, f"per-column factors {M}x{N}x{K} batch {b}")
+
+
 def test_output_that_is_only_8_byte_aligned_leaves_the_persistent_kernel(T, dev):
     """The persistent kernel stores 16 bytes per lane and row; an output that starts 8 bytes off, or whose rows are an odd
     number of 8-byte units apart, goes to the one-tile kernel (8-byte stores) and gets the same bits."""

@@ -55,9 +55,9 @@ __device__ __forceinline__ void gemm_i8_tile(const GemmArgs& g, const int block_
     constexpr int A_INSTR = BM / 8 / NW;  // global->LDS wave instructions per K tile per wave
     constexpr int B_INSTR = BN / 8 / NW;
     constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128;
-    constexpr bool CHAIN = (EPI == EPI_PROMOTE_CHAIN);
+    constexpr bool CHAIN = (EPI == EPI_PROMOTE_CHAIN || EPI == EPI_PROMOTE_CHAIN_LANE);
     constexpr bool FAST = (EPI == EPI_PROMOTE || EPI == EPI_PROMOTE_LANE || CHAIN);
-    constexpr bool LANEB = (EPI == EPI_PROMOTE_LANE);
+    constexpr bool LANEB = (EPI == EPI_PROMOTE_LANE || EPI == EPI_PROMOTE_CHAIN_LANE);
     constexpr bool PROMOTE = (FAST || EPI == EPI_STRICT);
     static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "tile/wave mismatch");
 
@@ -195,7 +195,7 @@ __device__ __forceinline__ void gemm_i8_tile(const GemmArgs& g, const int block_
             const float v3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fvec[3]), l));
             f_cur = c == 0 ? v0 : (c == 1 ? v1 : (c == 2 ? v2 : v3));
         }
-        if (LANEB) {  // issued before this tile's loads; consumed after its barrier (which waits for them)
+        if (LANEB && !CHAIN) {  // issued before this tile's loads; consumed after its barrier (which waits for them)
 #pragma unroll
             for (int j = 0; j < TN; ++j) fb[j] = pfb[j][(int64_t)kt * g.sb.ks];
         }
@@ -279,12 +279,41 @@ __device__ __forceinline__ void gemm_i8_tile(const GemmArgs& g, const int block_
 #pragma unroll
             for (int j = 0; j < TN; ++j) fbv[j][ks] = *reinterpret_cast<const v4i*>(stage_b + b_row_off + j * 4096 + choff[ks]);
         };
+        // factors of the K tile being folded, per block column: the wave-uniform one, or with operand B scaled per
+        // (column, K tile) this lane's column's (fb[] holds tile kt's values, fbn[] tile kt + 1's, requested one tile
+        // ahead so that the wait in front of the barrier has long covered them)
+        float f0 = 1.0f, f1 = 1.0f;
+        float fbn[TN];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fbn[j] = 1.0f;
+        auto tile_factors = [&](int kt) {
+            load_factors(kt);   // f_cur (and nothing else: the per-lane values are handled here)
+            if (LANEB) {
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    fb[j] = fbn[j];
+                    fbn[j] = pfb[j][(int64_t)min(kt + 1, nk - 1) * g.sb.ks];
+                }
+                f0 = f_cur * fb[0];
+                f1 = f_cur * fb[1];
+                if (divide) {
+                    f0 = 1.0f / f0;
+                    f1 = 1.0f / f1;
+                }
+            } else {
+                f0 = f1 = f_cur;
+            }
+        };
         auto fold = [&](int i, const v16i& d0, const v16i& d1) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) accf[PROMOTE ? i : 0][0][r] = __builtin_fmaf(static_cast<float>(d0[r]), f_cur, accf[PROMOTE ? i : 0][0][r]);
+            for (int r = 0; r < 16; ++r) accf[PROMOTE ? i : 0][0][r] = __builtin_fmaf(static_cast<float>(d0[r]), f0, accf[PROMOTE ? i : 0][0][r]);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) accf[PROMOTE ? i : 0][PROMOTE ? 1 : 0][r] = __builtin_fmaf(static_cast<float>(d1[r]), f_cur, accf[PROMOTE ? i : 0][PROMOTE ? 1 : 0][r]);
+            for (int r = 0; r < 16; ++r) accf[PROMOTE ? i : 0][PROMOTE ? 1 : 0][r] = __builtin_fmaf(static_cast<float>(d1[r]), f1, accf[PROMOTE ? i : 0][PROMOTE ? 1 : 0][r]);
         };
+        if (LANEB) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j) fbn[j] = pfb[j][0];
+        }
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) read_b(ldsB, ks);
         read_a(0, ldsA, 0);
@@ -293,7 +322,7 @@ __device__ __forceinline__ void gemm_i8_tile(const GemmArgs& g, const int block_
             const int8_t* stA = ldsA + cur * A_BYTES;
             const int8_t* stAn = ldsA + (cur ^ 1) * A_BYTES;
             const int8_t* stBn = ldsB + (cur ^ 1) * B_BYTES;
-            load_factors(kt);
+            tile_factors(kt);
             issue_tile_loads<B_INSTR>(baseB + idx::gemm_k_offset(kt + 1, klast), strideB8, voffB, tB0, wB + (cur ^ 1) * B_BYTES);
 #pragma unroll
             for (int i = 0; i < TM - 1; ++i) {
@@ -660,6 +689,7 @@ int init_gemm_kernels() {
     TI8_GEMM_CASE(256, 256, 2, 4, EPI_I32);
     TI8_GEMM_CASE(256, 128, 4, 2, EPI_PROMOTE_LANE);
     TI8_GEMM_CASE(256, 256, 2, 4, EPI_PROMOTE_CHAIN);
+    TI8_GEMM_CASE(256, 256, 2, 4, EPI_PROMOTE_CHAIN_LANE);
     TI8_GEMM_CASE(256, 128, 4, 2, EPI_PROMOTE);
 #undef TI8_GEMM_CASE
 #define TI8_GEMM_CASE(BM, BN, WM, WN, EPI) \
@@ -703,6 +733,7 @@ static int launch_tiled(const char* fn, const GemmArgs& a, int64_t batch, const 
     TI8_GEMM_CASE(128, 128, 2, 2, EPI_STRICT);
     TI8_GEMM_CASE(256, 128, 4, 2, EPI_PROMOTE_LANE);
     TI8_GEMM_CASE(256, 256, 2, 4, EPI_PROMOTE_CHAIN);
+    TI8_GEMM_CASE(256, 256, 2, 4, EPI_PROMOTE_CHAIN_LANE);
     TI8_GEMM_CASE(256, 128, 4, 2, EPI_PROMOTE);
     TI8_GEMM_CASE(128, 128, 2, 2, EPI_PROMOTE);
 #undef TI8_GEMM_CASE
@@ -754,7 +785,7 @@ extern "C" int ti8_gemm_i8_nt_multi(const ti8_gemm_problem* problems, int count,
                                 (gemm_flags & TI8_GEMM_LARGE_TILES) != 0, device_cu_count());
         one_launch = one_launch && c[i].bm == c[0].bm && c[i].bn == c[0].bn && c[i].epi == c[0].epi;
     }
-    one_launch = one_launch && c[0].epi != EPI_STRICT && c[0].epi != EPI_PROMOTE_LANE;
+    one_launch = one_launch && c[0].epi != EPI_STRICT && c[0].epi != EPI_PROMOTE_LANE && c[0].epi != EPI_PROMOTE_CHAIN_LANE;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool persistent = !(gemm_flags & TI8_GEMM_ONE_TILE);
     if (one_launch && c[0].epi == EPI_PROMOTE_CHAIN && persistent) {

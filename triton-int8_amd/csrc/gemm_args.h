@@ -27,7 +27,8 @@ struct GemmArgs {
 // EPI_PROMOTE: the per-K-tile factor is uniform over a wave's tile (block or per-row scales
 // on both operands); EPI_PROMOTE_LANE: operand B carries one scale per (column, K tile).
 // EPI_PROMOTE_CHAIN: EPI_PROMOTE without int32 accumulators that live across K tiles (see gemm.hip).
-enum { EPI_I32 = 0, EPI_ROWS = 1, EPI_PROMOTE = 2, EPI_STRICT = 3, EPI_PROMOTE_LANE = 4, EPI_PROMOTE_CHAIN = 5 };
+// EPI_PROMOTE_CHAIN_LANE: EPI_PROMOTE_CHAIN with operand B's factors per (column, K tile) as in EPI_PROMOTE_LANE.
+enum { EPI_I32 = 0, EPI_ROWS = 1, EPI_PROMOTE = 2, EPI_STRICT = 3, EPI_PROMOTE_LANE = 4, EPI_PROMOTE_CHAIN = 5, EPI_PROMOTE_CHAIN_LANE = 6 };
 
 
 // scale of operand row `row` at K block kb

@@ -262,7 +262,8 @@ TI8_HD GemmConfig gemm_config(int64_t M, int64_t N, int64_t K, int64_t batch, bo
     // the fast promotion keeps at most 256 per-K-tile factors in registers and cannot apply a
     // factor that varies per row of A inside the loop: those cases take the literal kernel
     if (strict || modeA == 2 || K > 256 * 128) return GemmConfig{128, 128, 2, 2, 3};
-    if (modeB == 2) return GemmConfig{256, 128, 4, 2, 4};
+    // operand B scaled per (row, K block): 256 x 256 tiles with the chained promotion where they fill the machine
+    if (modeB == 2) return (large || tiles_256x256 >= num_cu) ? GemmConfig{256, 256, 2, 4, 6} : GemmConfig{256, 128, 4, 2, 4};
     // 256 x 256 tiles (128 x 64 per wave, float accumulators only) where they fill the machine, else
     // 256 x 128 (64 x 64 per wave, int32 + float accumulators), else 128 x 128
     if (large || tiles_256x256 >= num_cu) return GemmConfig{256, 256, 2, 4, 5};
