@@ -287,6 +287,17 @@ int ti8_fwht_t(const void* x, int64_t ldx, void* y, int64_t ldy,
 int ti8_fwht_quant_row(const void* x, int64_t ldx, int8_t* q, int64_t ldq, float* s,
                        int64_t rows, int64_t cols, int64_t n, int qflags, int inv_mode, ti8_stream_t stream);
 
+/* The same for a transposed operand: q, s = ti8_quant_row(ti8_fwht_t(x)), bit for bit, i.e. the rotation along the ROWS of
+ * x [R][C] and the per-row quantiser of the rotated x^T -- what dX = fwd_32(dY, W^T) and dW = bwd_33(dY^T, X^T) need of
+ * W, dY and X when the scheme rotates along the contraction dim (triton/double-channle_fwd32.py:299-304 applied to the
+ * transposed operands).  Two launches: a tiled bf16 transposition into `scratch` (16-byte accesses both ways), then
+ * ti8_fwht_quant_row on it: 7 bytes of HBM traffic per element against 4 (2-to-16-byte strided reads) + 3 for the pair.
+ *   x bf16 [R][C] (ldx) -> q int8 [C][R] (ldq), s fp32 [C];  scratch: C * R bf16 elements, 16-byte aligned, contents
+ *   undefined afterwards.  R a power of two in [128, 32768] or a multiple of 64 that is zero-extended (n / 2 < R < n);
+ *   C % 64 == 0.  qflags, inv_mode as in ti8_fwht_quant_row. */
+int ti8_fwht_t_quant_row(const void* x, int64_t ldx, void* scratch, int8_t* q, int64_t ldq, float* s,
+                         int64_t R, int64_t C, int qflags, int inv_mode, ti8_stream_t stream);
+
 /* ---------------------------------------------------------------------------------
  * INT8 NT GEMM with fused dequantising epilogue, C[b] = dequant(A[b] * B[b]^T):
  * replaces triton_gemm + int8_gemm_kernel of every scheme

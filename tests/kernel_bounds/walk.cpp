@@ -132,6 +132,27 @@ int walk_fwht_quant_row(int64_t ldx, int64_t ldq, int64_t rows, int64_t cols, in
     return walk_fwht_impl(true, ldx, ldq, rows, cols, n, x_elems, q_elems, s_elems, lds_bytes_limit, n_checked, msg, msglen);
 }
 
+// transpose_bf16_kernel (fwht.hip): x bf16 [R][C] (ldx) -> y bf16 [C][R] (ldy), 64 x 64 tiles
+static void walk_transpose_tiles(Report& r, int64_t ldx, int64_t ldy, int64_t R, int64_t C, int64_t x_elems, int64_t y_elems) {
+    if (R % 64 || C % 64) { r.fail("transpose: %lld x %lld is not made of 64 x 64 tiles", (long long)R, (long long)C); return; }
+    const int tiles_c = (int)(C / 64);
+    for (int64_t block = 0; block < (R / 64) * (C / 64) && !r.bad; ++block) {
+        const int64_t tc = block % tiles_c, tr = block / tiles_c;
+        for (int tid = 0; tid < 256; ++tid)
+            for (int h = 0; h < 2; ++h) {
+                const int a = (tid >> 3) + 32 * h, b = (tid & 7) * 8;
+                r.access("fwht_t transpose x", (tr * 64 + a) * ldx + tc * 64 + b, 8, x_elems, block, tid, h);
+                r.access("fwht_t transpose y", (tc * 64 + a) * ldy + tr * 64 + b, 8, y_elems, block, tid, h);
+            }
+    }
+}
+int walk_transpose_bf16(int64_t ldx, int64_t ldy, int64_t R, int64_t C, int64_t x_elems, int64_t y_elems, int64_t* n_checked, char* msg, int msglen) {
+    Report r{msg, msglen};
+    walk_transpose_tiles(r, ldx, ldy, R, C, x_elems, y_elems);
+    *n_checked = r.checked;
+    return r.bad;
+}
+
 // ti8_fwht_t -> fwht_t_kernel<NT, W> (fwht.hip): x bf16 [R][C] (ldx) -> y bf16 [C][R] (ldy)
 int walk_fwht_t(int64_t ldx, int64_t ldy, int64_t R, int64_t C, int64_t x_elems, int64_t y_elems, int64_t lds_bytes_limit,
                 int64_t* n_checked, char* msg, int msglen) {
@@ -139,16 +160,7 @@ int walk_fwht_t(int64_t ldx, int64_t ldy, int64_t R, int64_t C, int64_t x_elems,
     if (!fwht_t_direct(R, C)) {
         // transpose_bf16_kernel: 64 x 64 tiles, thread t reads 8 columns of rows t/8 and t/8 + 32 and writes 8 rows
         // of columns t/8 and t/8 + 32; then fwht_kernel in place on y [C][R]
-        const int tiles_c = (int)(C / 64);
-        for (int64_t block = 0; block < (R / 64) * (C / 64) && !r.bad; ++block) {
-            const int64_t tc = block % tiles_c, tr = block / tiles_c;
-            for (int tid = 0; tid < 256; ++tid)
-                for (int h = 0; h < 2; ++h) {
-                    const int a = (tid >> 3) + 32 * h, b = (tid & 7) * 8;
-                    r.access("fwht_t transpose x", (tr * 64 + a) * ldx + tc * 64 + b, 8, x_elems, block, tid, h);
-                    r.access("fwht_t transpose y", (tc * 64 + a) * ldy + tr * 64 + b, 8, y_elems, block, tid, h);
-                }
-        }
+        walk_transpose_tiles(r, ldx, ldy, R, C, x_elems, y_elems);
         int64_t n2 = 0;
         const int bad = r.bad ? 1 : walk_fwht(ldy, ldy, C, R, R, y_elems, y_elems, lds_bytes_limit, &n2, msg, msglen);
         *n_checked = r.checked + n2;

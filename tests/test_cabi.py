@@ -79,6 +79,13 @@ FAKE = 0x10000  # a 16-byte aligned non-null "device pointer"; validation never 
     (("ti8_fwht_quant_row", FAKE, 4096, FAKE, 4096, FAKE, 4, 4096, 4096, 8, 1, None), 4, "apply here"),     # TI8_Q_HAD128
     (("ti8_fwht_quant_row", FAKE, 4096, FAKE, 4096, FAKE, 4, 4096, 4096, 4, 1, None), 4, "apply here"),     # TI8_Q_SCALE_BF16
     (("ti8_fwht_quant_row", FAKE, 4096, FAKE, 4096, FAKE, 4, 4096, 4096, 1, 9, None), 4, "inv_mode"),
+    (("ti8_fwht_t_quant_row", FAKE, 256, None, FAKE, 4096, FAKE, 4096, 256, 1, 1, None), 1, "required"),
+    (("ti8_fwht_t_quant_row", FAKE, 256, FAKE + 4096, FAKE, 4096, FAKE, 4096, 200, 1, 1, None), 2, "C % 64"),
+    (("ti8_fwht_t_quant_row", FAKE, 256, FAKE + 4096, FAKE, 4096, FAKE, 65536, 256, 1, 1, None), 2, "R <= 32768"),
+    (("ti8_fwht_t_quant_row", FAKE, 256, FAKE + 4096, FAKE, 2048, FAKE, 2048 + 64, 256, 1, 1, None), 2, "leading dimension of q"),
+    (("ti8_fwht_t_quant_row", FAKE, 200, FAKE + 4096, FAKE, 4096, FAKE, 4096, 256, 1, 1, None), 2, "leading dimension"),
+    (("ti8_fwht_t_quant_row", FAKE, 256, FAKE, FAKE, 4096, FAKE, 4096, 256, 1, 1, None), 4, "must not be the input"),
+    (("ti8_fwht_t_quant_row", FAKE, 256, FAKE + 4096, FAKE, 4096, FAKE, 4096, 256, 8, 1, None), 4, "apply here"),
     (("ti8_quant_col_t", FAKE, 256, FAKE, 128, FAKE, None, 128, 256, 0, 0, None), 1, "required"),
     (("ti8_quant_col_t", FAKE, 256, FAKE, 128, FAKE, FAKE, 100, 256, 0, 0, None), 2, "R%128"),
     (("ti8_quant_row_col_t", FAKE, 256, FAKE, 256, FAKE, FAKE, 128, FAKE, None, 128, 256, 0, 0, None), 1, "required"),

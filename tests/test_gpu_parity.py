@@ -500,6 +500,26 @@ def test_rotation_and_row_quantiser_in_one_pass(T, dev, cols):
     assert torch.equal(qw, q) and torch.equal(sw, s)
 
 
+@pytest.mark.parametrize("R,C", [(128, 64), (256, 512), (1024, 192), (4096, 512), (8192, 128), (16384, 64), (1536, 128), (14336, 64)])
+def test_rotation_and_row_quantiser_of_the_transpose(T, dev, R, C):
+    """ti8_fwht_t_quant_row = ti8_quant_row of ti8_fwht_t, bit for bit (powers of two and zero-extended row counts, a strided
+    view), and equal to the oracle: rotate the transposed operand, round to bf16, quantise per row."""
+    from triton_int8_amd._lib import INV_AMAX_DIV_127
+    x = randn_bf16(make_gen(R * 5 + C), R, C)
+    x[:, 3] = 0
+    x[R // 2, 7] = 2.0e4
+    xd = x.to(dev)
+    q, s = T.ops.fwht_t_quant_row(xd, clamp=True, inv_mode=INV_AMAX_DIV_127)
+    q2, s2 = T.ops.quant_row(T.ops.fwht_t(xd), clamp=True, inv_mode=INV_AMAX_DIV_127)
+    assert q.shape == (C, R) and torch.equal(q, q2) and torch.equal(s, s2)
+    qo, so = odf.triton_per_row_quant_2d(ohad.hadamard_transform(x.t().contiguous()), BLOCK_N=128)
+    assert bits_equal(q, qo) and bits_equal(s, so)
+    wide = torch.zeros(R, C + 24, dtype=torch.bfloat16, device=dev)
+    wide[:, 8:8 + C] = xd
+    qw, sw = T.ops.fwht_t_quant_row(wide[:, 8:8 + C], clamp=True, inv_mode=INV_AMAX_DIV_127)
+    assert torch.equal(qw, q) and torch.equal(sw, s)
+
+
 def test_fused_hadamard_quantisers(T, dev):
     """H_128 fused into the quantisers equals the un-fused oracle (rotate, round to bf16, quantise)."""
     x = planted(20, 2, 256, 384)

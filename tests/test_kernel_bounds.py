@@ -38,6 +38,7 @@ def walker(tmp_path_factory):
     p64 = ctypes.POINTER(ctypes.c_int64)
     lib.walk_fwht.argtypes = [i64] * 8 + [p64, cp, ci]
     lib.walk_fwht_quant_row.argtypes = [i64] * 9 + [p64, cp, ci]
+    lib.walk_transpose_bf16.argtypes = [i64] * 6 + [p64, cp, ci]
     lib.walk_fwht_t.argtypes = [i64] * 7 + [p64, cp, ci]
     lib.walk_quant_row.argtypes = [i64] * 4 + [ci] + [i64] * 3 + [p64, cp, ci]
     lib.walk_quant_block.argtypes = [i64, i64, ci, i64, i64, ci, i64, i64, i64, i64, i64, i64, i64, i64, ci, i64, i64, i64, i64, p64, cp, ci]
@@ -97,6 +98,16 @@ def walk(lib, allocs, name, a):
         x, ldx, q, ldq, sc, rows, cols, nn = a[:8]
         rc = lib.walk_fwht_quant_row(ldx, ldq, rows, cols, nn, allocs.room(x, 2), allocs.room(q, 1), allocs.room(sc, 4), LDS_LIMIT,
                                      ctypes.byref(n), msg, 512)
+    elif name == "ti8_fwht_t_quant_row":
+        # the transposition into the scratch buffer (the long-column path of ti8_fwht_t), then ti8_fwht_quant_row on it
+        x, ldx, scratch, q, ldq, sc, R, C = a[:8]
+        nn = 1 << (R - 1).bit_length()
+        rc = lib.walk_transpose_bf16(ldx, R, R, C, allocs.room(x, 2), allocs.room(scratch, 2), ctypes.byref(n), msg, 512)
+        assert rc == 0, f"{name} (transposition): {msg.value.decode()}"
+        first = n.value
+        rc = lib.walk_fwht_quant_row(R, ldq, C, R, nn, allocs.room(scratch, 2), allocs.room(q, 1), allocs.room(sc, 4), LDS_LIMIT,
+                                     ctypes.byref(n), msg, 512)
+        n.value += first
     elif name == "ti8_fwht_t":
         x, ldx, y, ldy, R, C = a[:6]
         rc = lib.walk_fwht_t(ldx, ldy, R, C, allocs.room(x, 2), allocs.room(y, 2), LDS_LIMIT, ctypes.byref(n), msg, 512)
@@ -242,6 +253,16 @@ def test_transposed_hadamard_launches(walker, recorded, R, C):
     n = ctypes.c_int64(0)
     assert walker.walk_fwht_t(C, R, R, C, R * C - 1, R * C, LDS_LIMIT, ctypes.byref(n), msg, 512) == 1 and msg.value.split(b":")[0].endswith(b" x")
     assert walker.walk_fwht_t(C, R, R, C, R * C, R * C - 8, LDS_LIMIT, ctypes.byref(n), msg, 512) == 1 and msg.value.split(b":")[0].endswith(b" y")
+
+
+@pytest.mark.parametrize("R,C", [(128, 64), (4096, 192), (8192, 128), (14336, 64), (32768, 64)])
+def test_rotate_and_quantise_of_the_transpose(walker, recorded, R, C):
+    """ti8_fwht_t_quant_row as the wrapper launches it (scratch tensor included): the transposition and the fused kernel
+    behind it stay inside their buffers."""
+    T, allocs, calls = recorded
+    q, s = T.ops.fwht_t_quant_row(torch.empty(R, C, dtype=torch.bfloat16))
+    assert tuple(q.shape) == (C, R) and tuple(s.shape) == (C,) and [c[0] for c in calls] == ["ti8_fwht_t_quant_row"]
+    assert walk(walker, allocs, *calls[0]) >= R * C // 4
 
 
 @pytest.mark.parametrize("rows,cols", [(5, 128), (3, 2048), (2, 8192), (2, 14336), (1, 16384), (1, 32768), (2, 28672)])

@@ -41,6 +41,7 @@ PROTOTYPES = {
     "ti8_fwht": [_vp, _i64, _vp, _i64, _i64, _i64, _i64, _f32, _vp],
     "ti8_fwht_t": [_vp, _i64, _vp, _i64, _i64, _i64, _f32, _vp],
     "ti8_fwht_quant_row": [_vp, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _int, _int, _vp],
+    "ti8_fwht_t_quant_row": [_vp, _i64, _vp, _vp, _i64, _vp, _i64, _i64, _int, _int, _vp],
     "ti8_gemm_i8_nt": [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64,
                        _vp, _int, _i64, _i64, _i64, _vp, _int, _i64, _i64, _i64,
                        _i64, _i64, _i64, _i64, _int, _int, _f32, _f32, _int, _vp],

@@ -523,3 +523,28 @@ extern "C" int ti8_fwht_quant_row(const void* x, int64_t ldx, int8_t* q, int64_t
                            static_cast<const uint16_t*>(x), ldx, (uint16_t*)nullptr, (int64_t)0, (int)cols, logn, (int)L, 1.0f, q, ldq, s, mode);
     return check_launch(fn);
 }
+
+extern "C" int ti8_fwht_t_quant_row(const void* x, int64_t ldx, void* scratch, int8_t* q, int64_t ldq, float* s, int64_t R, int64_t C,
+                                    int qflags, int inv_mode, ti8_stream_t stream) {
+    const char* fn = "ti8_fwht_t_quant_row";
+    if (!x || !scratch || !q || !s) return fail(TI8_ERR_NULL, "%s: x, scratch, q and s are required", fn);
+    if (R < 128 || R > 32768 || R % 64 || C <= 0 || C % 64)
+        return fail(TI8_ERR_SHAPE, "%s: need 128 <= R <= 32768, R %% 64 == 0 and C %% 64 == 0; got R=%lld C=%lld", fn, (long long)R, (long long)C);
+    if ((R / 64) * (C / 64) > 0x7fffffffLL) return fail(TI8_ERR_SHAPE, "%s: too many tiles", fn);
+    if (ldx < C) return fail(TI8_ERR_SHAPE, "%s: leading dimension smaller than the row length", fn);
+    if (!aligned16(x) || !aligned16(scratch) || (ldx % 8)) return fail(TI8_ERR_ALIGN, "%s: pointers must be 16-byte aligned and strides multiples of 16 bytes", fn);
+    if (x == scratch) return fail(TI8_ERR_MODE, "%s: the scratch buffer must not be the input", fn);
+    int64_t n = 128;
+    while (n < R) n <<= 1;
+    // n = the next power of two: R itself, or R is transformed zero-extended (n / 2 < R < n, R % 16 == 0 holds).
+    // The other checks of the second launch, made before the first one is queued:
+    if (ldq < R) return fail(TI8_ERR_SHAPE, "%s: leading dimension of q smaller than R", fn);
+    if (!aligned16(q) || (ldq % 16)) return fail(TI8_ERR_ALIGN, "%s: q must be 16-byte aligned with a stride that is a multiple of 16", fn);
+    QMode mode;
+    if (int e = parse_mode(qflags, inv_mode, &mode)) return e;
+    if (qflags & (TI8_Q_HAD128 | TI8_Q_SCALE_BF16)) return fail(TI8_ERR_MODE, "%s: only TI8_Q_CLAMP and TI8_Q_EPS_ADD apply here", fn);
+    hipLaunchKernelGGL(transpose_bf16_kernel, dim3((unsigned)((R / 64) * (C / 64))), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint16_t*>(x), ldx, static_cast<uint16_t*>(scratch), R, (int)(C / 64));
+    if (int e = check_launch(fn)) return e;
+    return ti8_fwht_quant_row(scratch, R, q, ldq, s, C, R, n, qflags, inv_mode, stream);
+}

@@ -221,14 +221,15 @@ def linear_backward(dY2, X2, W, scheme="block_channel", hadamard=None, saved=Non
         return dX, dW
     # double_channel
     if hadamard == "full":
-        # the transposed operands are rotated along the rows of the tensors as they lie in memory (ops.fwht_t):
-        # no bf16 transpose of W, dY or X.  A length that is no power of two is rotated as the reference's external
-        # library rotates it (zero-extended to the next power of two and cut back, through a transposed copy)
+        # the transposed operands are rotated along the rows of the tensors as they lie in memory and quantised per row
+        # of the transpose (ops.fwht_t_quant_row: a tiled int16 transposition + the one-pass rotate-and-quantise kernel;
+        # the same bits as quant_row(fwht_t(.))).  A length that is no power of two is rotated as the reference's external
+        # library rotates it (zero-extended to the next power of two and cut back)
         dq, ds = _rotated_row_quant(dY2, "full")
-        wtq, wts = ops.quant_row(ops.fwht_t(W), clamp=True, inv_mode=INV_AMAX_DIV_127)
+        wtq, wts = ops.fwht_t_quant_row(W, clamp=True, inv_mode=INV_AMAX_DIV_127)
         dX = _gemm_dc(dq, ds, wtq, wts, 1.0 / N, tokens=tokens, gemms=gemms)
-        dytq, dyts = ops.quant_row(ops.fwht_t(dY2), clamp=True, inv_mode=INV_AMAX_DIV_127)
-        xtq, xts = ops.quant_row(ops.fwht_t(X2), clamp=True, inv_mode=INV_AMAX_DIV_127)
+        dytq, dyts = ops.fwht_t_quant_row(dY2, clamp=True, inv_mode=INV_AMAX_DIV_127)
+        xtq, xts = ops.fwht_t_quant_row(X2, clamp=True, inv_mode=INV_AMAX_DIV_127)
         dW = _gemm_dc(dytq, dyts, xtq, xts, 1.0 / T, gemms=gemms)
         return dX, dW
     dq, ds, dytq, dyts = _row_col(dY2, clamp=True, inv_mode=INV_AMAX_DIV_127)

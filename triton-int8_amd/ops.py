@@ -296,6 +296,24 @@ def fwht_quant_row(x, *, clamp=True, eps_add=False, inv_mode=INV_RCP_OF_SCALE):
     return q.reshape(*lead, cols), s.reshape(*lead)
 
 
+def fwht_t_quant_row(x, *, clamp=True, eps_add=False, inv_mode=INV_RCP_OF_SCALE):
+    """``quant_row(fwht_t(x))`` for x bf16 [R, C]: the rotation along the rows of ``x`` and the per-row quantiser of the
+    rotated transpose, ``(q int8 [C, R], s fp32 [C])``, the same bits; a tiled transposition into a scratch tensor and the
+    one-pass rotate + quantise kernel on it."""
+    _check_bf16(x, "x")
+    _need(x.dim() == 2, "x must be [R, C]")
+    R, C = x.shape
+    _need(128 <= R <= 32768 and R % 128 == 0 and C > 0 and C % 64 == 0, f"need R a multiple of 128 in [128, 32768] and C % 64 == 0, got {R} x {C}")
+    if x.stride(1) != 1 or x.stride(0) % 8 or x.data_ptr() % 16:
+        x = x.contiguous()
+    scratch = torch.empty((C, R), dtype=torch.bfloat16, device=x.device)
+    q = torch.empty((C, R), dtype=torch.int8, device=x.device)
+    s = torch.empty((C,), dtype=torch.float32, device=x.device)
+    _lib.call("ti8_fwht_t_quant_row", x.data_ptr(), x.stride(0), scratch.data_ptr(), q.data_ptr(), R, s.data_ptr(), R, C,
+              _qflags(clamp, eps_add, False), inv_mode, _stream())
+    return q, s
+
+
 def fwht_t(x, scale=1.0):
     """Walsh-Hadamard transform of ``x.T`` along its rows, i.e. along the ROWS of ``x`` [R, C], without
     the bf16 transpose: returns y [C, R] = ``fwht(x.T.contiguous())``, bit for bit."""
