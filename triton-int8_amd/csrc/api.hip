@@ -27,7 +27,7 @@ int device_cu_count() {
 }
 }  // namespace ti8
 
-extern "C" int ti8_version(void) { return 200; }
+extern "C" int ti8_version(void) { return 300; }
 extern "C" const char* ti8_last_error(void) { return ti8::err_buf(); }
 extern "C" const char* ti8_arch(void) { return "gfx950"; }
 extern "C" int ti8_last_gemm_kernel(void) { return ti8::last_gemm_kernel; }
