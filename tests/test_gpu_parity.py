@@ -446,7 +446,7 @@ def test_fwht_of_a_length_that_is_no_power_of_two(T, dev, cols):
         assert bits_equal(T.double_channel_fwd32.fwd_32(a.to(dev), b.to(dev)), odf.fwd_32(a, b))
 
 
-@pytest.mark.parametrize("n,cols", [(128, 384), (128, 4096), (256, 256), (512, 1536), (1024, 2048), (2048, 2048),
+@pytest.mark.parametrize("n,cols", [(128, 384), (128, 4096), (256, 256), (256, 2048), (512, 1536), (512, 4096), (1024, 1024), (1024, 2048), (1024, 3072), (2048, 2048),
                                     (4096, 4096), (8192, 8192), (16384, 16384), (32768, 32768)])
 def test_fwht(T, dev, n, cols):
     x = randn_bf16(make_gen(n + cols), 9, cols)
