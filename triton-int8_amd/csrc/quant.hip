@@ -12,14 +12,6 @@
 
 namespace ti8 {
 
-// Value of `v` in another lane of the same row of 16 lanes (DPP: no LDS traffic, and the move
-// folds into the instruction that consumes it).  CTRL: 0xB1 / 0x4E = quad_perm lane^1 / lane^2,
-// 0x141 = row_half_mirror (lane^7), 0x128 = row_ror:8 (lane^8).
-template <int CTRL>
-__device__ __forceinline__ float dpp_f32(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
-}
-
 // 128-point Walsh-Hadamard transform of a row segment held as 8 consecutive bf16 per lane by 16
 // consecutive lanes: butterflies in the fixed order stride 1, 2, 4 (in registers), 8, 16, 32, 64
 // (across lanes), fp32, un-normalised; one rounding to bf16.
