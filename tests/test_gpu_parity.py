@@ -450,6 +450,12 @@ def test_fwht_of_a_length_that_is_no_power_of_two(T, dev, cols):
                                     (4096, 4096), (8192, 8192), (16384, 16384), (32768, 32768)])
 def test_fwht(T, dev, n, cols):
     x = randn_bf16(make_gen(n + cols), 9, cols)
+    # results that are exactly zero keep the sign the plain butterflies give them: an all-zero row (zero-padded tokens), a
+    # constant row (every difference is zero), rows of negative zeros and of zeros of both signs
+    x[0] = 0.0
+    x[1] = 1.5
+    x[2] = -0.0
+    x[3] = torch.where(torch.arange(cols) % 3 == 0, -0.0, 0.0).to(torch.bfloat16)
     y = T.ops.fwht(x.to(dev), n)
     assert bits_equal(y, ohad.fwht_f32(x.float(), n).to(torch.bfloat16))
     if n == cols:

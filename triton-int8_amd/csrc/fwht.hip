@@ -103,15 +103,39 @@ __device__ __forceinline__ LaneStages lane_stages(int lane, int nstages) {
           "+v"(A[9]), "+v"(A[10]), "+v"(A[11]), "+v"(A[12]), "+v"(A[13]), "+v"(A[14]), "+v"(A[15])                              \
         : "v"(SIGMA))
 
-// the stages over bits 4 .. 4 + nstages - 1 (nstages <= 6) on the 16 elements of this lane's chunk
+// One DPP stage with the sign of every zero as the plain butterfly leaves it: own + sigma * partner computes b - a in the
+// upper lane, and where a == b that is +0 although it stands for -(a - b) = -0, so a result that is exactly zero could
+// come out as -0 at the end.  Nothing that is quantised afterwards can tell, but the bf16 output of the transform itself
+// is compared bit for bit (zero-padded rows are all-zero rows).  Here the upper lane negates its own value first (exact)
+// and adds: partner + (-own) = a - b, the lower lane partner + own; two instructions per element instead of one.
+template <int CTRL>
+__device__ __forceinline__ void exact_dpp_stage(float (&a)[16], float sigma) {
+    const uint32_t flip = __float_as_uint(sigma) & 0x80000000u;   // sign bit set in the upper lane
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        const float own = __uint_as_float(__float_as_uint(a[e]) ^ flip);
+        a[e] = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(a[e]), CTRL, 0xf, 0xf, true)) + own;
+    }
+}
+
+// the stages over bits 4 .. 4 + nstages - 1 (nstages <= 6) on the 16 elements of this lane's chunk.  EXACT_ZEROS: see
+// exact_dpp_stage (the bf16 output path); otherwise one instruction per element and stage (the quantising path)
+template <bool EXACT_ZEROS>
 __device__ __forceinline__ void lane_butterflies(float (&a)[16], const LaneStages& st, int nstages) {
 #if defined(__HIP_DEVICE_COMPILE__)
-    if (nstages > 0) TI8_FWHT_DPP_STAGE(a, st.sigma[0], "quad_perm:[1,0,3,2]");
-    if (nstages > 1) TI8_FWHT_DPP_STAGE(a, st.sigma[1], "quad_perm:[2,3,0,1]");
-    if (nstages > 2) TI8_FWHT_DPP_STAGE(a, st.sigma[2], "row_half_mirror");
-    if (nstages > 3) TI8_FWHT_DPP_STAGE(a, st.sigma[3], "row_ror:8");
+    if (EXACT_ZEROS) {
+        if (nstages > 0) exact_dpp_stage<0xB1>(a, st.sigma[0]);
+        if (nstages > 1) exact_dpp_stage<0x4E>(a, st.sigma[1]);
+        if (nstages > 2) exact_dpp_stage<0x141>(a, st.sigma[2]);
+        if (nstages > 3) exact_dpp_stage<0x128>(a, st.sigma[3]);
+    } else {
+        if (nstages > 0) TI8_FWHT_DPP_STAGE(a, st.sigma[0], "quad_perm:[1,0,3,2]");
+        if (nstages > 1) TI8_FWHT_DPP_STAGE(a, st.sigma[1], "quad_perm:[2,3,0,1]");
+        if (nstages > 2) TI8_FWHT_DPP_STAGE(a, st.sigma[2], "row_half_mirror");
+        if (nstages > 3) TI8_FWHT_DPP_STAGE(a, st.sigma[3], "row_ror:8");
 #pragma unroll
-    for (int e = 0; e < 16; ++e) a[e] = a[e] * st.sign;
+        for (int e = 0; e < 16; ++e) a[e] = a[e] * st.sign;
+    }
     if (nstages > 4) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
@@ -167,7 +191,7 @@ __global__ __launch_bounds__(NT) void fwht_kernel(const uint16_t* __restrict__ x
                            bf16_lo(v0q.w), bf16_hi(v0q.w), bf16_lo(v1q.x), bf16_hi(v1q.x), bf16_lo(v1q.y), bf16_hi(v1q.y),
                            bf16_lo(v1q.z), bf16_hi(v1q.z), bf16_lo(v1q.w), bf16_hi(v1q.w)};
             butterflies<4>(a);
-            lane_butterflies(a, st, nstages);
+            lane_butterflies<!QUANT>(a, st, nstages);
 #pragma unroll
             for (int e = 0; e < 16; ++e) lds[vt * 17 + e] = a[e];   // = padded(16 vt + e)
         }
