@@ -504,6 +504,13 @@ def test_rotation_and_row_quantiser_in_one_pass(T, dev, cols):
     wide[:, 16:16 + cols] = xd
     qw, sw = T.ops.fwht_quant_row(wide[:, 16:16 + cols], clamp=True, inv_mode=INV_AMAX_DIV_127)
     assert torch.equal(qw, q) and torch.equal(sw, s)
+    # non-finite inputs spread over their row in the rotation; both ways of getting there quantise them alike
+    xn = x.clone()
+    xn[0, 5], xn[1, 7], xn[3, 9], xn[3, cols - 1], xn[5] = float("inf"), float("nan"), float("-inf"), float("inf"), -0.0
+    xnd = xn.to(dev)
+    q, s = T.ops.fwht_quant_row(xnd, clamp=True, inv_mode=INV_AMAX_DIV_127)
+    q2, s2 = T.ops.quant_row(T.ops.fwht(xnd), clamp=True, inv_mode=INV_AMAX_DIV_127)
+    assert torch.equal(q, q2) and torch.equal(s.view(torch.int32), s2.view(torch.int32))
 
 
 @pytest.mark.parametrize("R,C", [(128, 64), (256, 512), (1024, 192), (4096, 512), (8192, 128), (16384, 64), (1536, 128), (14336, 64)])
