@@ -57,6 +57,54 @@ static int walk_fwht_impl(bool quant, int64_t ldx, int64_t ldy, int64_t rows, in
     Report r{msg, msglen};
     const int64_t L = quant ? n : fwht_segment_len(cols, n);
     if (quant && cols > n) r.fail("fwht_quant_row: %lld columns exceed the transform length %lld", (long long)cols, (long long)n);
+    if (n >= 4096) {
+        // fwht_row_kernel<CH, QUANT>: 4 waves, slice by slice through a 2 x 4352-word exchange buffer, results stored from registers
+        const int CH = (int)(n / 4096);
+        const bool extended = cols < L;
+        const int valid = (int)(extended ? cols : L);
+        const int segs_per_row = extended ? 1 : (int)(cols / L);
+        const int64_t nblocks = rows * segs_per_row;
+        const int64_t lds_words = (CH > 1 ? 2 : 1) * 4 * 64 * 17;
+        if (lds_words * 4 > 65536) r.fail("fwht rows: %lld bytes of static LDS", (long long)(lds_words * 4));
+        if (quant && segs_per_row != 1) r.fail("fwht_quant_row: %d segments per row", segs_per_row);
+        std::vector<uint8_t> taken((size_t)L / 4, 0);   // every group of 4 output elements belongs to exactly one thread
+        for (int tid = 0; tid < 256 && !r.bad; ++tid) {
+            const int lane = tid & 63, w = tid >> 6, lp = (lane & ~15) | had_chunk(lane & 15);
+            for (int k = 0; k < CH; ++k) {
+                const int64_t base = (int64_t)(k & 1) * 4 * 64 * 17;
+                for (int e = 0; e < 16; ++e) r.access("fwht rows lds write", base + fwht_row_lds(w, lp, e), 1, lds_words, tid, k, e);
+                for (int ws = 0; ws < 4; ++ws) {
+                    for (int e = 0; e < 4; ++e) r.access("fwht rows lds read", base + fwht_row_lds(ws, lp, 4 * w + e), 1, lds_words, tid, k, ws, e);
+                    const int first = fwht_row_out(k, ws, lp, w);
+                    if (first < 0 || first + 4 > L || first % 4) { r.fail("fwht rows: thread %d owns elements from %d of %lld", tid, first, (long long)L); break; }
+                    ++taken[(size_t)first / 4];
+                }
+            }
+            if (quant) r.access("fwht rows lds wave maxima", w, 1, lds_words, tid);
+        }
+        for (size_t i = 0; i < taken.size() && !r.bad; ++i)
+            if (taken[i] != 1) r.fail("fwht rows: elements %lld.. are stored by %d threads", (long long)(i * 4), (int)taken[i]);
+        for (int64_t block = 0; block < nblocks && !r.bad; ++block) {
+            const int64_t xo = fwht_segment_offset(block, segs_per_row, ldx, (int)L);
+            const int64_t yo = fwht_segment_offset(block, segs_per_row, ldy, (int)L);
+            for (int tid = 0; tid < 256; ++tid) {
+                const int lane = tid & 63, w = tid >> 6, lp = (lane & ~15) | had_chunk(lane & 15);
+                for (int k = 0; k < CH; ++k) {
+                    const int first = fwht_row_chunk_first(k, w, lp);
+                    const int from = fwht_chunk_valid(first, 16, valid) ? first : 0;   // a chunk past the end re-reads the first one
+                    r.access("fwht x", xo + from, 8, x_elems, block, tid, k);
+                    r.access("fwht x", xo + from + 8, 8, x_elems, block, tid, k);
+                    for (int ws = 0; ws < 4; ++ws) {
+                        const int out = fwht_row_out(k, ws, lp, w);
+                        if (fwht_chunk_valid(out, 4, valid)) r.access(quant ? "fwht q" : "fwht y", yo + out, 4, y_elems, block, tid, k, ws);
+                    }
+                }
+                if (quant && tid == 0) r.access("fwht s", block, 1, s_elems, block);
+            }
+        }
+        *n_checked = r.checked;
+        return r.bad;
+    }
     const int NT = fwht_threads(L);
     const bool extended = cols < L;             // a zero-extended row per workgroup
     const int valid = (int)(extended ? cols : L);

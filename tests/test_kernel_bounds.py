@@ -197,7 +197,8 @@ def test_walker_sees_an_access_past_the_end(walker):
     assert walker.walk_fwht(cols, cols, rows, cols, cols, rows * cols, rows * cols, LDS_LIMIT, ctypes.byref(n), msg, 512) == 0
     assert walker.walk_fwht(cols, cols, rows, cols, cols, rows * cols - 8, rows * cols, LDS_LIMIT, ctypes.byref(n), msg, 512) == 1
     assert b"fwht x" in msg.value
-    assert walker.walk_fwht(cols, cols, rows, 32768, 32768, rows * 32768, rows * 32768, 64 * 1024, ctypes.byref(n), msg, 512) == 1   # LDS
+    # LDS: a 2048-element segment needs 8.5 KiB (lengths from 4096 on use a fixed 34 KiB exchange buffer instead)
+    assert walker.walk_fwht(2048, 2048, rows, 2048, 2048, rows * 2048, rows * 2048, 4 * 1024, ctypes.byref(n), msg, 512) == 1
     assert walker.walk_quant_row(cols, cols, rows, cols, 0, rows * cols, rows * cols, rows, ctypes.byref(n), msg, 512) == 0
     assert walker.walk_quant_row(cols, cols, rows, cols, 0, rows * cols, rows * cols, rows - 1, ctypes.byref(n), msg, 512) == 1
     assert b"quant_row s" in msg.value

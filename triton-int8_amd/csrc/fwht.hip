@@ -293,6 +293,152 @@ __global__ __launch_bounds__(NT) void fwht_kernel(const uint16_t* __restrict__ x
     }
 }
 
+// ---- segments of 4096 * CH elements (CH = 1, 2, 4, 8), one per workgroup of 4 waves, with a single trip through LDS.
+// Slice k of the segment (4096 elements) is 4 x 1024: wave w transforms elements [1024 (4k + w), + 1024) over bits 0..9
+// in registers and across its lanes (16 elements per lane, lane_butterflies).  Bits 10 and 11 pair the four waves of a
+// slice: every lane writes its 16 values to LDS and takes back elements 4w .. 4w + 3 of its chunk position from all four
+// waves (a radix-4 butterfly on each of the four elements).  Bits 12 and up pair the slices, which by then sit in the same
+// thread's registers.  A thread ends with 4 consecutive elements of 4 CH chunks and stores them from registers (8 bytes of
+// bf16, or 4 bytes of int8 behind the row's absmax when QUANT): there is no read-back pass, and the exchange buffer is
+// 17 KiB (two of them, so that one barrier per slice is enough) whatever the length.  Same stage order, same roundings as
+// fwht_kernel: bit-identical.
+template <int CH, bool QUANT>
+__global__ __launch_bounds__(256) void fwht_row_kernel(const uint16_t* __restrict__ x, int64_t ldx, uint16_t* __restrict__ y,
+                                                       int64_t ldy, int cols, float scale, int8_t* __restrict__ q, int64_t ldq,
+                                                       float* __restrict__ s, QMode mode) {
+    constexpr int L = 4096 * CH;
+    constexpr int BUF = 4 * 64 * 17;                      // one slice: [wave][chunk position] x 16 values, 17 words apart
+    __shared__ float xbuf[(CH > 1 ? 2 : 1) * BUF];   // (one buffer and a second barrier per slice measured the same)
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int valid = cols < L ? cols : L;                // cols < L: one zero-extended row per workgroup
+    const int segs_per_row = cols < L ? 1 : cols / L;
+    const uint16_t* xr = x + idx::fwht_segment_offset(blockIdx.x, segs_per_row, ldx, L);
+    const LaneStages st = lane_stages(lane, 6);
+    const int lp = (lane & ~15) | idx::had_chunk(lane & 15);   // this lane's chunk among the 64 of its wave's 1024 elements
+
+    float b[CH][16];
+    const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
+    // a chunk beyond the row's end (zero-extended rows) reads the row's first chunk instead and is then replaced by zeros:
+    // the load stays an ordinary global load (a select between the load and a constant becomes a select of addresses)
+    auto load_slice = [&](int k, uint4& lo, uint4& hi) {
+        const int first = idx::fwht_row_chunk_first(k, w, lp);
+        const bool in = idx::fwht_chunk_valid(first, 16, valid);
+        const uint16_t* p = xr + (in ? first : 0);
+        lo = *reinterpret_cast<const uint4*>(p);
+        hi = *reinterpret_cast<const uint4*>(p + 8);
+        if (!in) lo = hi = zero4;
+    };
+    uint4 lo, hi, nlo = zero4, nhi = zero4;
+    load_slice(0, lo, hi);
+#pragma unroll
+    for (int k = 0; k < CH; ++k) {
+        if (k + 1 < CH) load_slice(k + 1, nlo, nhi);
+        float a[16] = {bf16_lo(lo.x), bf16_hi(lo.x), bf16_lo(lo.y), bf16_hi(lo.y), bf16_lo(lo.z), bf16_hi(lo.z), bf16_lo(lo.w), bf16_hi(lo.w),
+                       bf16_lo(hi.x), bf16_hi(hi.x), bf16_lo(hi.y), bf16_hi(hi.y), bf16_lo(hi.z), bf16_hi(hi.z), bf16_lo(hi.w), bf16_hi(hi.w)};
+        butterflies<4>(a);
+        lane_butterflies<!QUANT>(a, st, 6);
+        float* buf = xbuf + (k & 1) * BUF;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) buf[idx::fwht_row_lds(w, lp, e)] = a[e];
+        __syncthreads();   // with two buffers this also orders the reads of slice k - 1 before the writes of slice k + 1
+        float c[4][4];
+#pragma unroll
+        for (int ws = 0; ws < 4; ++ws)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) c[ws][e] = buf[idx::fwht_row_lds(ws, lp, 4 * w + e)];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {   // bit 10: waves 0|1 and 2|3
+            const float u0 = c[0][e], v0 = c[1][e], u1 = c[2][e], v1 = c[3][e];
+            c[0][e] = u0 + v0;
+            c[1][e] = u0 - v0;
+            c[2][e] = u1 + v1;
+            c[3][e] = u1 - v1;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {   // bit 11: waves 0|2 and 1|3
+            const float u0 = c[0][e], v0 = c[2][e], u1 = c[1][e], v1 = c[3][e];
+            c[0][e] = u0 + v0;
+            c[2][e] = u0 - v0;
+            c[1][e] = u1 + v1;
+            c[3][e] = u1 - v1;
+        }
+#pragma unroll
+        for (int ws = 0; ws < 4; ++ws)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) b[k][ws * 4 + e] = c[ws][e];
+        lo = nlo;
+        hi = nhi;
+    }
+    // bits 12 and up: the slices
+#pragma unroll
+    for (int h = 1; h < CH; h <<= 1)
+#pragma unroll
+        for (int k = 0; k < CH; ++k)
+            if ((k & h) == 0) {
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    const float u = b[k][j], v = b[k + h][j];
+                    b[k][j] = u + v;
+                    b[k + h][j] = u - v;
+                }
+            }
+    // the thread's results as bf16: element idx::fwht_row_out(k, ws, lp, w) + e  <-  b[k][4 ws + e]
+    uint2 o[CH][4];
+#pragma unroll
+    for (int k = 0; k < CH; ++k)
+#pragma unroll
+        for (int ws = 0; ws < 4; ++ws) {
+            float f[4] = {b[k][ws * 4], b[k][ws * 4 + 1], b[k][ws * 4 + 2], b[k][ws * 4 + 3]};
+            if (scale != 1.0f) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) f[e] = f[e] * scale;
+            }
+            o[k][ws] = make_uint2(pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]));
+        }
+    if (!QUANT) {
+        uint16_t* yr = y + idx::fwht_segment_offset(blockIdx.x, segs_per_row, ldy, L);
+#pragma unroll
+        for (int k = 0; k < CH; ++k)
+#pragma unroll
+            for (int ws = 0; ws < 4; ++ws) {
+                const int first = idx::fwht_row_out(k, ws, lp, w);
+                if (idx::fwht_chunk_valid(first, 4, valid)) *reinterpret_cast<uint2*>(yr + first) = o[k][ws];
+            }
+        return;
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int k = 0; k < CH; ++k)
+#pragma unroll
+        for (int ws = 0; ws < 4; ++ws)
+            if (idx::fwht_chunk_valid(idx::fwht_row_out(k, ws, lp, w), 4, valid))
+                amax = fmaxf(fmaxf(amax, fmaxf(fabsf(bf16_lo(o[k][ws].x)), fabsf(bf16_hi(o[k][ws].x)))),
+                             fmaxf(fabsf(bf16_lo(o[k][ws].y)), fabsf(bf16_hi(o[k][ws].y))));
+    amax = wave_max(amax);
+    __syncthreads();                 // the last slice's exchange has been read: the buffer's first words serve the reduction
+    if (lane == 0) xbuf[w] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(xbuf[0], xbuf[1]), fmaxf(xbuf[2], xbuf[3]));
+    amax = amax_floor(amax, mode.eps_add);
+    const float mult = 127.0f / amax;
+    const int64_t row = blockIdx.x;
+    if (tid == 0) s[row] = stored_scale(amax, mult, mode);
+    int8_t* qr = q + row * ldq;
+#pragma unroll
+    for (int k = 0; k < CH; ++k)
+#pragma unroll
+        for (int ws = 0; ws < 4; ++ws) {
+            const int first = idx::fwht_row_out(k, ws, lp, w);
+            if (!idx::fwht_chunk_valid(first, 4, valid)) continue;
+            uint32_t v = put_u8(qbiased(bf16_lo(o[k][ws].x), mult), 0, 0u);
+            v = put_u8(qbiased(bf16_hi(o[k][ws].x), mult), 1, v);
+            v = put_u8(qbiased(bf16_lo(o[k][ws].y), mult), 2, v);
+            v = put_u8(qbiased(bf16_hi(o[k][ws].y), mult), 3, v);
+            *reinterpret_cast<uint32_t*>(qr + first) = v ^ UNBIAS4;
+        }
+}
+
 // ---- transposed input: y[c][r] = sum_r' H[r][r'] x[r'][c], i.e. the transform of x^T along its
 // rows without materialising x^T.  A workgroup owns W columns of x (W = 8, 4, 2, 1 as the length R
 // grows: W * R fp32 elements must fit in LDS), reads them row by row -- W bf16 = 2 W bytes per row;
@@ -439,6 +585,22 @@ static int prepare_fwht() {
     return TI8_OK;
 }
 
+#ifndef TI8_FWHT_ROW_KERNEL
+#define TI8_FWHT_ROW_KERNEL 1
+#endif
+// segments of 4096 elements and more: the kernel with one trip through LDS
+template <bool QUANT>
+static void launch_fwht_rows(int64_t n, int64_t nblocks, const uint16_t* x, int64_t ldx, uint16_t* y, int64_t ldy, int cols, float scale,
+                             int8_t* q, int64_t ldq, float* s, const QMode& mode, hipStream_t st) {
+    const dim3 grid((unsigned)nblocks), block(256);
+    switch (n) {
+        case 4096: hipLaunchKernelGGL((fwht_row_kernel<1, QUANT>), grid, block, 0, st, x, ldx, y, ldy, cols, scale, q, ldq, s, mode); break;
+        case 8192: hipLaunchKernelGGL((fwht_row_kernel<2, QUANT>), grid, block, 0, st, x, ldx, y, ldy, cols, scale, q, ldq, s, mode); break;
+        case 16384: hipLaunchKernelGGL((fwht_row_kernel<4, QUANT>), grid, block, 0, st, x, ldx, y, ldy, cols, scale, q, ldq, s, mode); break;
+        default: hipLaunchKernelGGL((fwht_row_kernel<8, QUANT>), grid, block, 0, st, x, ldx, y, ldy, cols, scale, q, ldq, s, mode); break;
+    }
+}
+
 namespace ti8 {
 int init_fwht_kernels() {
     if (int e = prepare_fwht()) return e;
@@ -508,7 +670,10 @@ extern "C" int ti8_fwht(const void* x, int64_t ldx, void* y, int64_t ldy, int64_
     const size_t shmem = (size_t)idx::fwht_lds_words(L) * sizeof(float);
     if (int e = prepare_fwht()) return e;
     const QMode none = {0, 0, 0, 0};
-    if (idx::fwht_threads(L) == 1024)
+    if (TI8_FWHT_ROW_KERNEL && n >= 4096)
+        launch_fwht_rows<false>(n, nblocks, static_cast<const uint16_t*>(x), ldx, static_cast<uint16_t*>(y), ldy, (int)cols, scale, nullptr, 0, nullptr,
+                                none, static_cast<hipStream_t>(stream));
+    else if (idx::fwht_threads(L) == 1024)
         hipLaunchKernelGGL((fwht_kernel<1024, false>), dim3((unsigned)nblocks), dim3(1024), shmem, static_cast<hipStream_t>(stream),
                            static_cast<const uint16_t*>(x), ldx, static_cast<uint16_t*>(y), ldy, (int)cols, logn, (int)L, scale,
                            (int8_t*)nullptr, (int64_t)0, (float*)nullptr, none);
@@ -539,7 +704,9 @@ extern "C" int ti8_fwht_quant_row(const void* x, int64_t ldx, int8_t* q, int64_t
     const int64_t L = n;   // one workgroup per row
     const size_t shmem = (size_t)idx::fwht_lds_words(L) * sizeof(float);
     if (int e = prepare_fwht()) return e;
-    if (idx::fwht_threads(L) == 1024)
+    if (TI8_FWHT_ROW_KERNEL && n >= 4096)
+        launch_fwht_rows<true>(n, rows, static_cast<const uint16_t*>(x), ldx, nullptr, 0, (int)cols, 1.0f, q, ldq, s, mode, static_cast<hipStream_t>(stream));
+    else if (idx::fwht_threads(L) == 1024)
         hipLaunchKernelGGL((fwht_kernel<1024, true>), dim3((unsigned)rows), dim3(1024), shmem, static_cast<hipStream_t>(stream),
                            static_cast<const uint16_t*>(x), ldx, (uint16_t*)nullptr, (int64_t)0, (int)cols, logn, (int)L, 1.0f, q, ldq, s, mode);
     else

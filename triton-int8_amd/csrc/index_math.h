@@ -147,6 +147,12 @@ TI8_HD int64_t fwht_segment_offset(int64_t block, int segs_per_row, int64_t ld, 
 TI8_HD bool fwht_chunk_valid(int first, int len, int valid) { return first + len <= valid; }
 // LDS words a workgroup needs for L elements
 TI8_HD int64_t fwht_lds_words(int64_t L) { return L + L / 16; }
+// fwht_row_kernel (segments of 4096 * CH elements on 4 waves): first element of the 16-element chunk that the lane at chunk
+// position `lp` of wave `w` takes from slice `k`; the word of its value `e` in the exchange buffer; and the first of the 4
+// consecutive elements of (slice k, wave ws, chunk position lp) that wave `w` ends up with
+TI8_HD int fwht_row_chunk_first(int k, int w, int lp) { return ((k * 4 + w) * 64 + lp) * 16; }
+TI8_HD int fwht_row_lds(int w, int lp, int e) { return (w * 64 + lp) * 17 + e; }
+TI8_HD int fwht_row_out(int k, int ws, int lp, int w) { return ((k * 4 + ws) * 64 + lp) * 16 + 4 * w; }
 // base LDS index of the radix-2^rb group `vt` in the pass over index bits [p, p + rb)
 TI8_HD int fwht_group_base(int vt, int p, int rb) {
     const int lo = vt & ((1 << p) - 1);
