@@ -2,7 +2,8 @@
 // fp32 butterflies in the fixed order stride 1, 2, 4, ..., n/2.  The order is part of
 // the contract: fp32 sums are order dependent and the CPU checker uses the same one.
 //
-// A workgroup owns L consecutive elements of one row: L = n when
+// Lengths from 4096 on: fwht_row_kernel (described there): registers, lanes, one exchange through LDS per 4096 elements.
+// Shorter lengths: fwht_kernel.  A workgroup owns L consecutive elements of one row: L = n when
 // n >= 2048, else gcd(cols, 2048) (several length-n groups).  The log2(n) stages run in
 // passes: in a pass over index bits [p, p+r) a thread gathers the 2^r elements that
 // differ only in those bits, does the butterflies in registers and hands them on through
