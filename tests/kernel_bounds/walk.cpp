@@ -144,15 +144,14 @@ static int walk_fwht_impl(bool quant, int64_t ldx, int64_t ldy, int64_t rows, in
                 if (rem > 0) pass(8 + rb2, rem);
             }
         }
-        if (quant) {   // at most 4 chunks per thread are kept in registers; the first words of LDS then hold one maximum per wave
-            for (int k = 0; k < 4; ++k)
-                if (tid + k * NT < (L >> 3)) r.access("fwht lds read-back", fwht_padded((tid + k * NT) * 8), 8, lds_words, tid, k);
+        if (quant) {   // one chunk per thread is kept in registers; the first words of LDS then hold one maximum per wave
+            if (tid < (L >> 3)) r.access("fwht lds read-back", fwht_padded(tid * 8), 8, lds_words, tid);
             r.access("fwht lds wave maxima", tid >> 6, 1, lds_words, tid);
         } else {
             for (int c = tid; c < (L >> 3); c += NT) r.access("fwht lds read-back", fwht_padded(c * 8), 8, lds_words, tid, c);
         }
     }
-    if (quant && (L >> 3) > 4 * NT) r.fail("fwht_quant_row: %lld chunks do not fit 4 per thread on %d threads", (long long)(L >> 3), NT);
+    if (quant && (L >> 3) > NT) r.fail("fwht_quant_row: %lld chunks do not fit one per thread on %d threads", (long long)(L >> 3), NT);
     for (int64_t block = 0; block < nblocks && !r.bad; ++block) {
         const int64_t xo = fwht_segment_offset(block, segs_per_row, ldx, (int)L);
         const int64_t yo = fwht_segment_offset(block, segs_per_row, ldy, (int)L);

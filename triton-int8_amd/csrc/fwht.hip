@@ -156,8 +156,7 @@ __device__ __forceinline__ void lane_butterflies(float (&a)[16], const LaneStage
 #endif
 }
 
-// NT threads per workgroup: 256, or 1024 for segments of 16384 elements and more (their LDS
-// footprint allows only one or two workgroups per CU, which 256 threads would leave idle).
+// Segments of up to 2048 elements (lengths below 4096), NT = 256 threads per workgroup.
 // QUANT: the workgroup's segment is a whole row (L >= cols), and instead of the rotated bf16 row the
 // kernel writes what the per-row quantiser makes of it -- int8 q[row][cols] and the row's scale --
 // with the quantiser's own arithmetic on the same bf16-rounded values: the rotated operand never
@@ -236,7 +235,7 @@ __global__ __launch_bounds__(NT) void fwht_kernel(const uint16_t* __restrict__ x
     }
     if (QUANT) {
         // a thread's chunks stay in registers (bf16, as they would have been stored) while the row's absmax is reduced
-        constexpr int MAXC = 4;          // L / 8 / NT: 8192 elements on 256 threads, 32768 on 1024
+        constexpr int MAXC = 1;          // L / 8 / NT: at most 2048 elements on 256 threads
         uint4 o[MAXC];
         float amax = 0.0f;
 #pragma unroll
@@ -578,17 +577,6 @@ static int prepare_fwht_t() {
     return TI8_OK;
 }
 
-static int prepare_fwht() {
-    static OncePerDevice once, once_quant;
-    hipError_t e = raise_lds_limit(once, reinterpret_cast<const void*>(fwht_kernel<1024, false>), FWHT_LDS_LIMIT);
-    if (e == hipSuccess) e = raise_lds_limit(once_quant, reinterpret_cast<const void*>(fwht_kernel<1024, true>), FWHT_LDS_LIMIT);
-    if (e != hipSuccess) return fail(TI8_ERR_HIP, "ti8_fwht: cannot raise the LDS limit: %s", hipGetErrorString(e));
-    return TI8_OK;
-}
-
-#ifndef TI8_FWHT_ROW_KERNEL
-#define TI8_FWHT_ROW_KERNEL 1
-#endif
 // segments of 4096 elements and more: the kernel with one trip through LDS
 template <bool QUANT>
 static void launch_fwht_rows(int64_t n, int64_t nblocks, const uint16_t* x, int64_t ldx, uint16_t* y, int64_t ldy, int cols, float scale,
@@ -604,7 +592,6 @@ static void launch_fwht_rows(int64_t n, int64_t nblocks, const uint16_t* x, int6
 
 namespace ti8 {
 int init_fwht_kernels() {
-    if (int e = prepare_fwht()) return e;
     if (int e = prepare_fwht_t<1024, 8>()) return e;
     if (int e = prepare_fwht_t<1024, 4>()) return e;
     if (int e = prepare_fwht_t<1024, 2>()) return e;
@@ -668,16 +655,11 @@ extern "C" int ti8_fwht(const void* x, int64_t ldx, void* y, int64_t ldy, int64_
     if (nblocks > 0x7fffffffLL) return fail(TI8_ERR_SHAPE, "ti8_fwht: too many segments");
     int logn = 0;
     while ((1LL << logn) < n) ++logn;
-    const size_t shmem = (size_t)idx::fwht_lds_words(L) * sizeof(float);
-    if (int e = prepare_fwht()) return e;
+    const size_t shmem = (size_t)idx::fwht_lds_words(L) * sizeof(float);   // at most 8.5 KiB: L <= 2048 here
     const QMode none = {0, 0, 0, 0};
-    if (TI8_FWHT_ROW_KERNEL && n >= 4096)
+    if (n >= 4096)
         launch_fwht_rows<false>(n, nblocks, static_cast<const uint16_t*>(x), ldx, static_cast<uint16_t*>(y), ldy, (int)cols, scale, nullptr, 0, nullptr,
                                 none, static_cast<hipStream_t>(stream));
-    else if (idx::fwht_threads(L) == 1024)
-        hipLaunchKernelGGL((fwht_kernel<1024, false>), dim3((unsigned)nblocks), dim3(1024), shmem, static_cast<hipStream_t>(stream),
-                           static_cast<const uint16_t*>(x), ldx, static_cast<uint16_t*>(y), ldy, (int)cols, logn, (int)L, scale,
-                           (int8_t*)nullptr, (int64_t)0, (float*)nullptr, none);
     else
         hipLaunchKernelGGL((fwht_kernel<256, false>), dim3((unsigned)nblocks), dim3(256), shmem, static_cast<hipStream_t>(stream),
                            static_cast<const uint16_t*>(x), ldx, static_cast<uint16_t*>(y), ldy, (int)cols, logn, (int)L, scale,
@@ -704,12 +686,8 @@ extern "C" int ti8_fwht_quant_row(const void* x, int64_t ldx, int8_t* q, int64_t
     while ((1LL << logn) < n) ++logn;
     const int64_t L = n;   // one workgroup per row
     const size_t shmem = (size_t)idx::fwht_lds_words(L) * sizeof(float);
-    if (int e = prepare_fwht()) return e;
-    if (TI8_FWHT_ROW_KERNEL && n >= 4096)
+    if (n >= 4096)
         launch_fwht_rows<true>(n, rows, static_cast<const uint16_t*>(x), ldx, nullptr, 0, (int)cols, 1.0f, q, ldq, s, mode, static_cast<hipStream_t>(stream));
-    else if (idx::fwht_threads(L) == 1024)
-        hipLaunchKernelGGL((fwht_kernel<1024, true>), dim3((unsigned)rows), dim3(1024), shmem, static_cast<hipStream_t>(stream),
-                           static_cast<const uint16_t*>(x), ldx, (uint16_t*)nullptr, (int64_t)0, (int)cols, logn, (int)L, 1.0f, q, ldq, s, mode);
     else
         hipLaunchKernelGGL((fwht_kernel<256, true>), dim3((unsigned)rows), dim3(256), shmem, static_cast<hipStream_t>(stream),
                            static_cast<const uint16_t*>(x), ldx, (uint16_t*)nullptr, (int64_t)0, (int)cols, logn, (int)L, 1.0f, q, ldq, s, mode);

@@ -248,7 +248,7 @@ TI8_HD int64_t fwht_segment_len(int64_t cols, int64_t n) {
     }
     return a;  // gcd(cols, 2048), a multiple of n because n divides both
 }
-TI8_HD int fwht_threads(int64_t L) { return L >= 16384 ? 1024 : 256; }
+TI8_HD int fwht_threads(int64_t) { return 256; }   // fwht_kernel: segments of up to 2048 elements (longer ones: fwht_row_kernel)
 
 // LDS-tiled GEMM: tile shape, waves and epilogue kind by shape and scale modes.  `epi` values are
 // the EPI_* constants of gemm_args.h.
