@@ -58,20 +58,20 @@ static int walk_fwht_impl(bool quant, int64_t ldx, int64_t ldy, int64_t rows, in
     const int64_t L = quant ? n : fwht_segment_len(cols, n);
     if (quant && cols > n) r.fail("fwht_quant_row: %lld columns exceed the transform length %lld", (long long)cols, (long long)n);
     if (n >= 4096) {
-        // fwht_row_kernel<CH, QUANT>: 4 waves, slice by slice through a 2 x 4352-word exchange buffer, results stored from registers
+        // fwht_row_kernel<CH, QUANT>: 4 waves, slice by slice through a 2 x 4096-word exchange buffer, results stored from registers
         const int CH = (int)(n / 4096);
         const bool extended = cols < L;
         const int valid = (int)(extended ? cols : L);
         const int segs_per_row = extended ? 1 : (int)(cols / L);
         const int64_t nblocks = rows * segs_per_row;
-        const int64_t lds_words = (CH > 1 ? 2 : 1) * 4 * 64 * 17;
+        const int64_t lds_words = (CH > 1 ? 2 : 1) * 4 * 64 * 16;
         if (lds_words * 4 > 65536) r.fail("fwht rows: %lld bytes of static LDS", (long long)(lds_words * 4));
         if (quant && segs_per_row != 1) r.fail("fwht_quant_row: %d segments per row", segs_per_row);
         std::vector<uint8_t> taken((size_t)L / 4, 0);   // every group of 4 output elements belongs to exactly one thread
         for (int tid = 0; tid < 256 && !r.bad; ++tid) {
             const int lane = tid & 63, w = tid >> 6, lp = (lane & ~15) | had_chunk(lane & 15);
             for (int k = 0; k < CH; ++k) {
-                const int64_t base = (int64_t)(k & 1) * 4 * 64 * 17;
+                const int64_t base = (int64_t)(k & 1) * 4 * 64 * 16;
                 for (int e = 0; e < 16; ++e) r.access("fwht rows lds write", base + fwht_row_lds(w, lp, e), 1, lds_words, tid, k, e);
                 for (int ws = 0; ws < 4; ++ws) {
                     for (int e = 0; e < 4; ++e) r.access("fwht rows lds read", base + fwht_row_lds(ws, lp, 4 * w + e), 1, lds_words, tid, k, ws, e);

@@ -300,15 +300,15 @@ __global__ __launch_bounds__(NT) void fwht_kernel(const uint16_t* __restrict__ x
 // waves (a radix-4 butterfly on each of the four elements).  Bits 12 and up pair the slices, which by then sit in the same
 // thread's registers.  A thread ends with 4 consecutive elements of 4 CH chunks and stores them from registers (8 bytes of
 // bf16, or 4 bytes of int8 behind the row's absmax when QUANT): there is no read-back pass, and the exchange buffer is
-// 17 KiB (two of them, so that one barrier per slice is enough) whatever the length.  Same stage order, same roundings as
+// 16 KiB (two of them, so that one barrier per slice is enough) whatever the length.  Same stage order, same roundings as
 // fwht_kernel: bit-identical.
 template <int CH, bool QUANT>
 __global__ __launch_bounds__(256) void fwht_row_kernel(const uint16_t* __restrict__ x, int64_t ldx, uint16_t* __restrict__ y,
                                                        int64_t ldy, int cols, float scale, int8_t* __restrict__ q, int64_t ldq,
                                                        float* __restrict__ s, QMode mode) {
     constexpr int L = 4096 * CH;
-    constexpr int BUF = 4 * 64 * 17;                      // one slice: [wave][chunk position] x 16 values, 17 words apart
-    __shared__ float xbuf[(CH > 1 ? 2 : 1) * BUF];   // (one buffer and a second barrier per slice measured the same)
+    constexpr int BUF = 4 * 64 * 16;                      // one slice: 4 waves x 64 chunk positions x 16 values (idx::fwht_row_lds)
+    __shared__ __attribute__((aligned(16))) float xbuf[(CH > 1 ? 2 : 1) * BUF];   // (one buffer and a second barrier per slice measured the same)
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int valid = cols < L ? cols : L;                // cols < L: one zero-extended row per workgroup
@@ -340,13 +340,18 @@ __global__ __launch_bounds__(256) void fwht_row_kernel(const uint16_t* __restric
         lane_butterflies<!QUANT>(a, st, 6);
         float* buf = xbuf + (k & 1) * BUF;
 #pragma unroll
-        for (int e = 0; e < 16; ++e) buf[idx::fwht_row_lds(w, lp, e)] = a[e];
+        for (int j = 0; j < 4; ++j)
+            *reinterpret_cast<float4*>(buf + idx::fwht_row_lds(w, lp, 4 * j)) = make_float4(a[4 * j], a[4 * j + 1], a[4 * j + 2], a[4 * j + 3]);
         __syncthreads();   // with two buffers this also orders the reads of slice k - 1 before the writes of slice k + 1
         float c[4][4];
 #pragma unroll
-        for (int ws = 0; ws < 4; ++ws)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) c[ws][e] = buf[idx::fwht_row_lds(ws, lp, 4 * w + e)];
+        for (int ws = 0; ws < 4; ++ws) {
+            const float4 v = *reinterpret_cast<const float4*>(buf + idx::fwht_row_lds(ws, lp, 4 * w));
+            c[ws][0] = v.x;
+            c[ws][1] = v.y;
+            c[ws][2] = v.z;
+            c[ws][3] = v.w;
+        }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {   // bit 10: waves 0|1 and 2|3
             const float u0 = c[0][e], v0 = c[1][e], u1 = c[2][e], v1 = c[3][e];

@@ -151,7 +151,10 @@ TI8_HD int64_t fwht_lds_words(int64_t L) { return L + L / 16; }
 // position `lp` of wave `w` takes from slice `k`; the word of its value `e` in the exchange buffer; and the first of the 4
 // consecutive elements of (slice k, wave ws, chunk position lp) that wave `w` ends up with
 TI8_HD int fwht_row_chunk_first(int k, int w, int lp) { return ((k * 4 + w) * 64 + lp) * 16; }
-TI8_HD int fwht_row_lds(int w, int lp, int e) { return (w * 64 + lp) * 17 + e; }
+// (laid out so that a lane's elements 4j .. 4j + 3 are one aligned 16-byte unit and consecutive chunk positions are
+// consecutive units: both the writes -- four units per lane -- and the reads -- unit j = w of all four waves -- are
+// 16-byte LDS accesses without bank conflicts)
+TI8_HD int fwht_row_lds(int w, int lp, int e) { return (((e >> 2) * 4 + w) * 64 + lp) * 4 + (e & 3); }
 TI8_HD int fwht_row_out(int k, int ws, int lp, int w) { return ((k * 4 + ws) * 64 + lp) * 16 + 4 * w; }
 // base LDS index of the radix-2^rb group `vt` in the pass over index bits [p, p + rb)
 TI8_HD int fwht_group_base(int vt, int p, int rb) {
