@@ -75,18 +75,17 @@ __device__ __forceinline__ void pass_dispatch(float* lds, int L, int p, int rb, 
 // chunk has the bit set: an fma whose product is exact, rounded once like the add or subtract it stands for).  That
 // leaves the upper lane of a pair with the negative of its result; both partners of every later stage carry the same
 // number of such flips, so nothing else changes and the lane multiplies by its sign (-1 for an odd number of set bits
-// among the stages that ran) at the end.  Bits 8 and 9 pair lanes 16 and 32 apart: v_permlane16_swap / v_permlane32_swap
-// of a register with its copy hand every lane the lower lane's value in one register and the upper lane's in the other,
-// so both lanes compute lower + sigma * upper, with the true sign.
+// among the stages that ran) at the end.  Bits 8 and 9 pair lanes 16 and 32 apart, through v_permlane16_swap /
+// v_permlane32_swap (described where they are used).
 struct LaneStages {
-    float sigma[6];   // per stage: -1 in lanes whose chunk has the stage's bit set
+    float sigma[4];   // per DPP stage: -1 in lanes whose chunk has the stage's bit set
     float sign;       // what the DPP stages that ran have multiplied the lane's values by
 };
 __device__ __forceinline__ LaneStages lane_stages(int lane, int nstages) {
     const int c = idx::had_chunk(lane & 15) | (lane & 48);
     LaneStages st;
 #pragma unroll
-    for (int k = 0; k < 6; ++k) st.sigma[k] = ((c >> k) & 1) ? -1.0f : 1.0f;
+    for (int k = 0; k < 4; ++k) st.sigma[k] = ((c >> k) & 1) ? -1.0f : 1.0f;
     const int ran = c & 15 & ((1 << (nstages < 4 ? nstages : 4)) - 1);
     st.sign = (__builtin_popcount(ran) & 1) ? -1.0f : 1.0f;
     return st;
@@ -121,7 +120,9 @@ __device__ __forceinline__ void exact_dpp_stage(float (&a)[16], float sigma) {
 
 // the stages over bits 4 .. 4 + nstages - 1 (nstages <= 6) on the 16 elements of this lane's chunk.  EXACT_ZEROS: see
 // exact_dpp_stage (the bf16 output path); otherwise one instruction per element and stage (the quantising path)
-template <bool EXACT_ZEROS>
+// APPLY_SIGN = false leaves the values of the one-instruction form multiplied by st.sign for a caller that multiplies
+// them by something else anyway (every later stage of this file pairs values of the same chunk position, i.e. sign)
+template <bool EXACT_ZEROS, bool APPLY_SIGN = true>
 __device__ __forceinline__ void lane_butterflies(float (&a)[16], const LaneStages& st, int nstages) {
 #if defined(__HIP_DEVICE_COMPILE__)
     if (EXACT_ZEROS) {
@@ -134,23 +135,33 @@ __device__ __forceinline__ void lane_butterflies(float (&a)[16], const LaneStage
         if (nstages > 1) TI8_FWHT_DPP_STAGE(a, st.sigma[1], "quad_perm:[2,3,0,1]");
         if (nstages > 2) TI8_FWHT_DPP_STAGE(a, st.sigma[2], "row_half_mirror");
         if (nstages > 3) TI8_FWHT_DPP_STAGE(a, st.sigma[3], "row_ror:8");
+        if (APPLY_SIGN) {
 #pragma unroll
-        for (int e = 0; e < 16; ++e) a[e] = a[e] * st.sign;
+            for (int e = 0; e < 16; ++e) a[e] = a[e] * st.sign;
+        }
     }
+    // Bits 8 and 9 pair lanes 16 and 32 apart, two elements at a time: a lane swap of the two registers brings both values
+    // of every pair into ONE lane (element e in the even rows / lower half, element e + 1 in the others), the butterfly is
+    // an ordinary add and subtract there, and the same swap takes sums and differences back to where they belong -- four
+    // instructions for two elements, true signs.
     if (nstages > 4) {
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            const int v = __float_as_int(a[e]);
-            const auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false);
-            a[e] = __builtin_fmaf(__int_as_float(r[1]), st.sigma[4], __int_as_float(r[0]));
+        for (int e = 0; e < 16; e += 2) {
+            const auto r = __builtin_amdgcn_permlane16_swap(__float_as_int(a[e]), __float_as_int(a[e + 1]), false, false);
+            const float u = __int_as_float(r[0]), v = __int_as_float(r[1]);
+            const auto t = __builtin_amdgcn_permlane16_swap(__float_as_int(u + v), __float_as_int(u - v), false, false);
+            a[e] = __int_as_float(t[0]);
+            a[e + 1] = __int_as_float(t[1]);
         }
     }
     if (nstages > 5) {
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            const int v = __float_as_int(a[e]);
-            const auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
-            a[e] = __builtin_fmaf(__int_as_float(r[1]), st.sigma[5], __int_as_float(r[0]));
+        for (int e = 0; e < 16; e += 2) {
+            const auto r = __builtin_amdgcn_permlane32_swap(__float_as_int(a[e]), __float_as_int(a[e + 1]), false, false);
+            const float u = __int_as_float(r[0]), v = __int_as_float(r[1]);
+            const auto t = __builtin_amdgcn_permlane32_swap(__float_as_int(u + v), __float_as_int(u - v), false, false);
+            a[e] = __int_as_float(t[0]);
+            a[e + 1] = __int_as_float(t[1]);
         }
     }
 #endif
@@ -337,7 +348,7 @@ __global__ __launch_bounds__(256) void fwht_row_kernel(const uint16_t* __restric
         float a[16] = {bf16_lo(lo.x), bf16_hi(lo.x), bf16_lo(lo.y), bf16_hi(lo.y), bf16_lo(lo.z), bf16_hi(lo.z), bf16_lo(lo.w), bf16_hi(lo.w),
                        bf16_lo(hi.x), bf16_hi(hi.x), bf16_lo(hi.y), bf16_hi(hi.y), bf16_lo(hi.z), bf16_hi(hi.z), bf16_lo(hi.w), bf16_hi(hi.w)};
         butterflies<4>(a);
-        lane_butterflies<!QUANT>(a, st, 6);
+        lane_butterflies<!QUANT, false>(a, st, 6);   // QUANT: the lane's sign goes into its quantisation multiplier below
         float* buf = xbuf + (k & 1) * BUF;
 #pragma unroll
         for (int j = 0; j < 4; ++j)
@@ -417,9 +428,12 @@ __global__ __launch_bounds__(256) void fwht_row_kernel(const uint16_t* __restric
     for (int k = 0; k < CH; ++k)
 #pragma unroll
         for (int ws = 0; ws < 4; ++ws)
-            if (idx::fwht_chunk_valid(idx::fwht_row_out(k, ws, lp, w), 4, valid))
-                amax = fmaxf(fmaxf(amax, fmaxf(fabsf(bf16_lo(o[k][ws].x)), fabsf(bf16_hi(o[k][ws].x)))),
-                             fmaxf(fabsf(bf16_lo(o[k][ws].y)), fabsf(bf16_hi(o[k][ws].y))));
+            if (idx::fwht_chunk_valid(idx::fwht_row_out(k, ws, lp, w), 4, valid)) {   // a chain, so that pairs become v_max3_f32
+                amax = fmaxf(amax, fabsf(bf16_lo(o[k][ws].x)));
+                amax = fmaxf(amax, fabsf(bf16_hi(o[k][ws].x)));
+                amax = fmaxf(amax, fabsf(bf16_lo(o[k][ws].y)));
+                amax = fmaxf(amax, fabsf(bf16_hi(o[k][ws].y)));
+            }
     amax = wave_max(amax);
     __syncthreads();                 // the last slice's exchange has been read: the buffer's first words serve the reduction
     if (lane == 0) xbuf[w] = amax;
@@ -429,6 +443,8 @@ __global__ __launch_bounds__(256) void fwht_row_kernel(const uint16_t* __restric
     const float mult = 127.0f / amax;
     const int64_t row = blockIdx.x;
     if (tid == 0) s[row] = stored_scale(amax, mult, mode);
+    // everything this thread holds came from chunk position lp of some wave and slice, so it carries this lane's sign
+    const float lane_mult = mult * st.sign;
     int8_t* qr = q + row * ldq;
 #pragma unroll
     for (int k = 0; k < CH; ++k)
@@ -436,10 +452,10 @@ __global__ __launch_bounds__(256) void fwht_row_kernel(const uint16_t* __restric
         for (int ws = 0; ws < 4; ++ws) {
             const int first = idx::fwht_row_out(k, ws, lp, w);
             if (!idx::fwht_chunk_valid(first, 4, valid)) continue;
-            uint32_t v = put_u8(qbiased(bf16_lo(o[k][ws].x), mult), 0, 0u);
-            v = put_u8(qbiased(bf16_hi(o[k][ws].x), mult), 1, v);
-            v = put_u8(qbiased(bf16_lo(o[k][ws].y), mult), 2, v);
-            v = put_u8(qbiased(bf16_hi(o[k][ws].y), mult), 3, v);
+            uint32_t v = put_u8(qbiased(bf16_lo(o[k][ws].x), lane_mult), 0, 0u);
+            v = put_u8(qbiased(bf16_hi(o[k][ws].x), lane_mult), 1, v);
+            v = put_u8(qbiased(bf16_lo(o[k][ws].y), lane_mult), 2, v);
+            v = put_u8(qbiased(bf16_hi(o[k][ws].y), lane_mult), 3, v);
             *reinterpret_cast<uint32_t*>(qr + first) = v ^ UNBIAS4;
         }
 }
