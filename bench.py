@@ -349,7 +349,7 @@ def main():
     # HBM-side bytes per GEMM launch: NOT measured by this run.  They come from two rocprofv3 --pmc runs of this
     # command (FETCH_SIZE, WRITE_SIZE), scaled on the device copy above, whose summary is the file named in
     # `traffic_source`; measured for these two schemes
-    traffic = {"block_channel": 855089521, "double_channel": 848883822}.get(args.scheme)
+    traffic = {"block_channel": 854975877, "double_channel": 848439911}.get(args.scheme)
     traffic_source = {"block_channel": "profiles/bench_config2_block_channel_counters.md (section 3)",
                       "double_channel": "profiles/bench_config2_double_channel_counters.md (section 3)"}.get(args.scheme)
 
